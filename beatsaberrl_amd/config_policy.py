@@ -1,0 +1,245 @@
+"""ConfigPolicy: the benchmark-config transformer policy on the HIP kernels.
+
+Same module contract as the reference's NotePolicy (python/policy.py:784,
+:1179): fp32 master parameters in a state_dict, `forward_stacked(obs) ->
+(logits (B, 29, K) fp32, value (B,) fp32)`, a stream dtype switched by an
+attribute (`.dtype`; the reference's `.fp16`), 16-bit weight replicas refreshed
+per weights version (python/fp16_linear.py:228-246, 349-376).  The
+architecture is the textbook pre-LN transformer of the benchmark configs:
+one Linear per token type, L blocks, one packed (29*K + 1, d) output matrix
+whose last row is the value.
+
+Two routes, both entirely on the C-ABI kernels:
+  * "ops":   one kernel per op (tokenizer, LayerNorm, packed QKV linear,
+             attention, out-proj + residual, LayerNorm, FFN up + act,
+             FFN down + residual, heads) - any supported shape and dtype;
+  * "fused": the whole forward in one persistent kernel reading a packed
+             weight image (16-bit dtypes, shapes the kernel is built for).
+`route="auto"` takes "fused" when the library supports the shape."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+import torch.nn as nn
+
+from . import _lib, ops
+from .fused_ln import FusedLayerNorm
+
+N_ACTION_HEADS = 29      # reference python/policy.py:409
+_DTYPES = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+class CfgBlock(nn.Module):
+    """Pre-LN block; parameter names follow the reference's Block
+    (python/policy.py:492-522): ln_attn, q/k/v/out_proj, ln_ffn, ffn.0, ffn.2."""
+
+    def __init__(self, d, ffn, act):
+        super().__init__()
+        self.ln_attn = FusedLayerNorm(d)
+        self.q_proj = nn.Linear(d, d)
+        self.k_proj = nn.Linear(d, d)
+        self.v_proj = nn.Linear(d, d)
+        self.out_proj = nn.Linear(d, d)
+        self.ln_ffn = FusedLayerNorm(d)
+        self.ffn = nn.Sequential(nn.Linear(d, ffn), nn.GELU() if act == "gelu" else nn.ReLU(), nn.Linear(ffn, d))
+
+
+class ConfigPolicy(nn.Module):
+    def __init__(self, n_layers=2, d=128, n_heads=4, ffn=512, T=16, n_gears=7, act="gelu", final_ln=False,
+                 prop_dim=100, obj_dim=16, dtype="f16", route="auto"):
+        super().__init__()
+        if act not in ("gelu", "relu"):
+            raise ValueError(f"act must be gelu or relu, got {act!r}")
+        if d % n_heads:
+            raise ValueError(f"d={d} not divisible by n_heads={n_heads}")
+        if n_layers > _lib.MAX_LAYERS:
+            raise ValueError(f"n_layers <= {_lib.MAX_LAYERS}")
+        self.n_layers, self.d, self.n_heads, self.ffn_dim, self.T = n_layers, d, n_heads, ffn, T
+        self.n_gears, self.act, self.prop_dim, self.obj_dim = n_gears, act, prop_dim, obj_dim
+        self.obs_dim = prop_dim + (T - 1) * obj_dim
+        self.n_out = N_ACTION_HEADS * n_gears + 1
+        self.prop_embed = nn.Linear(prop_dim, d)
+        self.obj_embed = nn.Linear(obj_dim, d)
+        self.blocks = nn.ModuleList(CfgBlock(d, ffn, act) for _ in range(n_layers))
+        self.final_ln = FusedLayerNorm(d) if final_ln else None
+        self.heads = nn.Linear(d, self.n_out)
+        self.dtype = dtype            # stream dtype: "f32" | "f16" | "bf16"
+        self.route = route            # "auto" | "ops" | "fused"
+        self._version = 0             # bumped by bump_weights_version()
+        self._replica = None          # (version, dtype, device) -> 16-bit weight copies
+        self._packed = None           # (version, dtype, device) -> fused-kernel weight image
+        self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
+                     "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}
+
+    # ---- weights ------------------------------------------------------------------
+    def bump_weights_version(self):
+        """Call after every in-place weight update (optimizer step, load):
+        the 16-bit replicas and the packed image are rebuilt on next use
+        (the reference's fp16_linear.bump_weights_version)."""
+        self._version += 1
+
+    def load_state_dict(self, *a, **k):
+        r = super().load_state_dict(*a, **k)
+        self.bump_weights_version()
+        return r
+
+    def _apply(self, fn, *a, **k):
+        r = super()._apply(fn, *a, **k)
+        self._replica = self._packed = None
+        return r
+
+    def _replicas(self, dt, device):
+        """Weights cast to the stream dtype (q|k|v concatenated), biases fp32."""
+        key = (self._version, dt, str(device))
+        if self._replica is not None and self._replica[0] == key:
+            return self._replica[1]
+        c = lambda w: w.detach().to(dt).contiguous()
+        f = lambda b: b.detach().float().contiguous()
+        r = {"prop_w": c(self.prop_embed.weight), "prop_b": f(self.prop_embed.bias),
+             "obj_w": c(self.obj_embed.weight), "obj_b": f(self.obj_embed.bias),
+             "heads_w": c(self.heads.weight), "heads_b": f(self.heads.bias), "blk": []}
+        for blk in self.blocks:
+            r["blk"].append({
+                "qkv_w": c(torch.cat([blk.q_proj.weight, blk.k_proj.weight, blk.v_proj.weight])),
+                "qkv_b": f(torch.cat([blk.q_proj.bias, blk.k_proj.bias, blk.v_proj.bias])),
+                "out_w": c(blk.out_proj.weight), "out_b": f(blk.out_proj.bias),
+                "w0": c(blk.ffn[0].weight), "b0": f(blk.ffn[0].bias),
+                "w2": c(blk.ffn[2].weight), "b2": f(blk.ffn[2].bias)})
+        self._replica = (key, r)
+        return r
+
+    def _desc(self, dt):
+        return _lib.CfgDesc(self.n_layers, self.d, self.n_heads, self.ffn_dim, self.T, self.n_gears,
+                            _lib.ACT_GELU if self.act == "gelu" else _lib.ACT_RELU,
+                            int(self.final_ln is not None), self.prop_dim, self.obj_dim, ops.dt_code(dt), 0)
+
+    def fused_supported(self, dt=None) -> bool:
+        dt = dt or _DTYPES[self.dtype]
+        if dt is torch.float32:
+            return False
+        return _lib.load().bsrl_cfg_pack_size(ctypes.byref(self._desc(dt))) > 0
+
+    def packed_image(self, dt, device):
+        """The fused kernel's weight image for the current weights version
+        (one cast+permute kernel over the fp32 masters)."""
+        key = (self._version, dt, str(device))
+        if self._packed is not None and self._packed[0] == key:
+            return self._packed[1]
+        lib = _lib.load()
+        desc = self._desc(dt)
+        size = lib.bsrl_cfg_pack_size(ctypes.byref(desc))
+        if size <= 0:
+            raise ops.Unsupported("fused forward does not support this shape/dtype")
+        for p in self.parameters():
+            if p.dtype is not torch.float32 or not p.is_contiguous() or p.device != device:
+                raise RuntimeError("fused forward needs contiguous fp32 master parameters on the obs device")
+        prm = _lib.CfgParams()
+        dp = lambda t: t.data_ptr()
+        prm.prop_w, prm.prop_b = dp(self.prop_embed.weight), dp(self.prop_embed.bias)
+        prm.obj_w, prm.obj_b = dp(self.obj_embed.weight), dp(self.obj_embed.bias)
+        for i, blk in enumerate(self.blocks):
+            b = prm.blk[i]
+            b.ln_attn_w, b.ln_attn_b = dp(blk.ln_attn.weight), dp(blk.ln_attn.bias)
+            b.q_w, b.q_b = dp(blk.q_proj.weight), dp(blk.q_proj.bias)
+            b.k_w, b.k_b = dp(blk.k_proj.weight), dp(blk.k_proj.bias)
+            b.v_w, b.v_b = dp(blk.v_proj.weight), dp(blk.v_proj.bias)
+            b.out_w, b.out_b = dp(blk.out_proj.weight), dp(blk.out_proj.bias)
+            b.ln_ffn_w, b.ln_ffn_b = dp(blk.ln_ffn.weight), dp(blk.ln_ffn.bias)
+            b.ffn0_w, b.ffn0_b = dp(blk.ffn[0].weight), dp(blk.ffn[0].bias)
+            b.ffn2_w, b.ffn2_b = dp(blk.ffn[2].weight), dp(blk.ffn[2].bias)
+        if self.final_ln is not None:
+            prm.final_ln_w, prm.final_ln_b = dp(self.final_ln.weight), dp(self.final_ln.bias)
+        prm.heads_w, prm.heads_b = dp(self.heads.weight), dp(self.heads.bias)
+        if self._packed is not None and self._packed[1].numel() == size and self._packed[1].device == device:
+            img = self._packed[1]          # refresh in place: the address must not move under a captured graph
+        else:
+            img = torch.empty(size, device=device, dtype=torch.uint8)
+        with torch.cuda.device(device):
+            rc = lib.bsrl_cfg_pack(ctypes.byref(desc), ctypes.byref(prm), img.data_ptr(),
+                                   torch.cuda.current_stream(device).cuda_stream)
+        if not _lib.check(rc, "bsrl_cfg_pack"):
+            raise ops.Unsupported("bsrl_cfg_pack")
+        self._packed = (key, img)
+        return img
+
+    # ---- forward ------------------------------------------------------------------
+    @torch.no_grad()
+    def forward_stacked(self, obs, n_valid=None, route=None):
+        """obs (B, obs_dim) fp32 (or the stream dtype) on the GPU; n_valid (B,)
+        int32 = attendable object tokens per env (None = all).  Returns
+        logits (B, 29, n_gears) fp32 and value (B,) fp32."""
+        if not obs.is_cuda:
+            raise RuntimeError("ConfigPolicy.forward_stacked runs on the GPU only (no CPU path)")
+        if obs.dim() != 2 or obs.shape[1] != self.obs_dim:
+            raise RuntimeError(f"obs must be (B, {self.obs_dim}), got {tuple(obs.shape)}")
+        if n_valid is not None:
+            if n_valid.dtype is not torch.int32 or n_valid.shape != (obs.shape[0],) or not n_valid.is_cuda:
+                raise RuntimeError("n_valid must be an int32 (B,) device tensor")
+            n_valid = n_valid.contiguous()
+        dt = _DTYPES[self.dtype]
+        route = route or self.route
+        if route == "auto":
+            route = "fused" if self.fused_supported(dt) else "ops"
+        if route == "fused":
+            return self._forward_fused(obs, n_valid, dt)
+        if route != "ops":
+            raise ValueError(f"route must be auto/ops/fused, got {route!r}")
+        return self._forward_ops(obs, n_valid, dt)
+
+    def forward(self, obs, n_valid=None):
+        logits, value = self.forward_stacked(obs, n_valid)
+        return list(logits.unbind(1)), value
+
+    def _forward_fused(self, obs, n_valid, dt):
+        B = obs.shape[0]
+        img = self.packed_image(dt, obs.device)
+        if obs.stride(1) != 1:
+            obs = obs.contiguous()
+        n_log = N_ACTION_HEADS * self.n_gears
+        logits = torch.empty(B, n_log, device=obs.device, dtype=torch.float32)
+        value = torch.empty(B, device=obs.device, dtype=torch.float32)
+        desc = self._desc(dt)
+        with torch.cuda.device(obs.device):
+            rc = _lib.load().bsrl_cfg_forward(ctypes.byref(desc), img.data_ptr(), obs.data_ptr(), obs.stride(0),
+                                              ops.dt_code(obs.dtype), None if n_valid is None else n_valid.data_ptr(),
+                                              logits.data_ptr(), value.data_ptr(), B,
+                                              torch.cuda.current_stream(obs.device).cuda_stream)
+        if not _lib.check(rc, "bsrl_cfg_forward"):
+            raise ops.Unsupported("bsrl_cfg_forward")
+        return logits.view(B, N_ACTION_HEADS, self.n_gears), value
+
+    def _forward_ops(self, obs, n_valid, dt):
+        B, T, d = obs.shape[0], self.T, self.d
+        r = self._replicas(dt, obs.device)
+        if obs.dtype not in (torch.float32, dt):
+            obs = obs.float()
+        x = ops.cfg_embed(obs, r["prop_w"], r["prop_b"], r["obj_w"], r["obj_b"], T, dt)       # (B, T, d)
+        for blk, w in zip(self.blocks, r["blk"]):
+            h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
+            qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                       # (B, T, 3d)
+            att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
+            x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                           # x + out(att)
+            h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)
+            fused = None
+            if dt is not torch.float32 and ops.ffn_fused_supported(d, self.ffn_dim, dt):
+                fused = ops.ffn_fused(x, h2, w["w0"], w["b0"], w["w2"], w["b2"], act=self.act)
+            if fused is not None:
+                x = fused[0]
+            else:
+                hid = ops.linear(h2, w["w0"], w["b0"], act=self.act)                          # (B, T, ffn)
+                x = ops.linear(hid, w["w2"], w["b2"], residual=x)
+        h = x[:, 0]                                                                           # (B, d), row stride T*d
+        if self.final_ln is not None:
+            h = ops.ln_fwd(h.contiguous(), self.final_ln.weight, self.final_ln.bias, self.final_ln.eps)
+        n_log = N_ACTION_HEADS * self.n_gears
+        logits, value = ops.linear(h, r["heads_w"], r["heads_b"], out_dtype=torch.float32, split=n_log)
+        return logits.view(B, N_ACTION_HEADS, self.n_gears), value.view(B)
+
+    # ---- construction helpers --------------------------------------------------------
+    @classmethod
+    def from_spec(cls, spec, **kw):
+        """spec: any object with the fields of the config description
+        (n_layers, d, n_heads, ffn, T, n_gears, act, final_ln, prop_dim, obj_dim)."""
+        return cls(spec.n_layers, spec.d, spec.n_heads, spec.ffn, spec.T, spec.n_gears, spec.act, spec.final_ln,
+                   spec.prop_dim, spec.obj_dim, **kw)

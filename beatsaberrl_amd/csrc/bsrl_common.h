@@ -1,0 +1,85 @@
+// Shared device helpers for the gfx950 policy-forward kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/bsrl.h"
+
+typedef uint16_t u16;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define WAVE 64
+
+// ---- host-side error plumbing ------------------------------------------------
+void bsrl_set_error(const char* fmt, ...);
+#define BSRL_FAIL(code, ...) do { bsrl_set_error(__VA_ARGS__); return (code); } while (0)
+#define BSRL_CHECK_LAUNCH(what) do { hipError_t e_ = hipGetLastError(); \
+    if (e_ != hipSuccess) BSRL_FAIL(BSRL_ELAUNCH, "%s: %s", what, hipGetErrorString(e_)); } while (0)
+
+static inline bool bsrl_aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- 16-bit storage types ------------------------------------------------------
+// Activations and weights are held as raw 16-bit words; the tag types below give
+// the conversions and the MFMA flavour for each format.
+struct F16 {
+    static __device__ __forceinline__ float to_f(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
+    static __device__ __forceinline__ u16 from_f(float f) { return __builtin_bit_cast(u16, (_Float16)f); }
+    // D(16x16) += A(16x32) * B(32x16); lane l holds A[l%16][8*(l/16)..+7], B[8*(l/16)..+7][l%16],
+    // D[4*(l/16)+i][l%16].
+    static __device__ __forceinline__ f32x4 mfma32(s16x8 a, s16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    // K = 16 flavour: lane l holds A[l%16][4*(l/16)..+3], B[4*(l/16)..+3][l%16].
+    static __device__ __forceinline__ f32x4 mfma16(s16x4 a, s16x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+    }
+};
+struct BF16 {
+    static __device__ __forceinline__ float to_f(u16 v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+    static __device__ __forceinline__ u16 from_f(float f) {   // round to nearest even
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (u16)(u >> 16);
+    }
+    static __device__ __forceinline__ f32x4 mfma32(s16x8 a, s16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(s16x4 a, s16x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+    }
+};
+// fp32 "storage" tag for the kernels that are templated on the I/O type
+struct F32IO { };
+
+template <typename DT> __device__ __forceinline__ float io_load(const u16* p) { return DT::to_f(*p); }
+template <typename DT> __device__ __forceinline__ void io_store(u16* p, float v) { *p = DT::from_f(v); }
+
+// ---- activations ---------------------------------------------------------------
+__device__ __forceinline__ float gelu_exact(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+template <int ACT> __device__ __forceinline__ float apply_act(float x) {
+    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_GELU) return gelu_exact(x);
+    return x;
+}
+
+// ---- wave-level reductions -------------------------------------------------------
+// Butterfly over the low `width` lanes of each width-aligned lane group.
+template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int o = WIDTH / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int o = WIDTH / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}

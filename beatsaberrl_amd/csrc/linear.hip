@@ -1,0 +1,269 @@
+// y = act(x W^T + b) (+ residual) for gfx950.
+//
+// 16-bit path: v_mfma_f32_16x16x32 (f16 / bf16), fp32 accumulate.  A workgroup
+// of 4 waves owns a 128-row x 128-column output tile (2 x 2 waves, each a
+// 64 x 64 tile = 4 x 4 MFMA tiles, 64 accumulator VGPRs).  Both operands are
+// read straight from global memory in MFMA fragment order: the weight is the
+// MFMA "A" operand (its M index is the OUTPUT column), the activation the "B"
+// operand (its N index is the ROW), so every lane ends up with 4 consecutive
+// output columns of one row and the epilogue stores 8 or 16 bytes per lane.
+// nn.Linear's (M, K) row-major weight is already K-contiguous per output
+// column, which is exactly the fragment order.  All weights of this model are
+// <= 1.2 MB and stay L2 resident; the kernel is an HBM stream over x and y.
+//
+// fp32 path: a plain LDS-tiled FMA kernel (parity configuration only).
+//
+// Replaces the vendor GEMM calls of the reference's op layer
+// (python/fp16_linear.py:134-181) and the bias+ReLU epilogues of
+// python/beat_arena_env/csrc/fp16_gemm.cu:77-111, 404-497.
+#include "bsrl_common.h"
+
+namespace {
+
+struct LinArgs {
+    const void* x; int64_t ldx;
+    const void* w;
+    const float* bias;
+    const void* res; int64_t ldr;
+    void* y; int64_t ldy;
+    void* y2; int64_t ldy2; int64_t split;
+    int64_t rows; int K; int M;
+    int out_f32;
+};
+
+// 8 consecutive k of one row, zero beyond K.  FAST: 16-byte aligned rows.
+template <bool FAST>
+__device__ __forceinline__ s16x8 load_frag(const u16* base, int64_t ld, int64_t row, int k0, int K) {
+    s16x8 r = {0, 0, 0, 0, 0, 0, 0, 0};
+    const u16* p = base + row * ld + k0;
+    if (FAST) {
+        if (k0 < K) r = *reinterpret_cast<const s16x8*>(p);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) if (k0 + j < K) r[j] = (short)p[j];
+    }
+    return r;
+}
+
+// Main loop shared by both 16-bit kernels: acc[col tile][row tile] over the wave's 64 x 64 tile.
+template <typename DT, bool FAST>
+__device__ __forceinline__ void mfma_mainloop(const LinArgs& a, int64_t row0, int col0, int r16, int g,
+                                              f32x4 (&acc)[4][4]) {
+    const u16* x = static_cast<const u16*>(a.x);
+    const u16* w = static_cast<const u16*>(a.w);
+    const int64_t last_row = a.rows - 1;
+    int64_t xr[4], wr[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {   // clamp instead of branching: out-of-range tiles are never stored
+        int64_t r = row0 + t * 16 + r16; xr[t] = r < last_row ? r : last_row;
+        int c = col0 + t * 16 + r16; wr[t] = c < a.M - 1 ? c : a.M - 1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    const int nk = (a.K + 31) / 32;
+    s16x8 xf[4], wf[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        xf[t] = load_frag<FAST>(x, a.ldx, xr[t], g * 8, a.K);
+        wf[t] = load_frag<FAST>(w, a.K, wr[t], g * 8, a.K);
+    }
+    for (int kc = 0; kc < nk; ++kc) {
+        s16x8 xn[4], wn[4];
+        const int k1 = (kc + 1) * 32 + g * 8;
+        if (kc + 1 < nk) {   // next fragments in flight while this chunk's 16 MFMAs issue
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                xn[t] = load_frag<FAST>(x, a.ldx, xr[t], k1, a.K);
+                wn[t] = load_frag<FAST>(w, a.K, wr[t], k1, a.K);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = DT::mfma32(wf[i], xf[j], acc[i][j]);
+        if (kc + 1 < nk) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) { xf[t] = xn[t]; wf[t] = wn[t]; }
+        }
+    }
+}
+
+// General epilogue: any M, any strides, optional column split into a second output.
+template <typename DT, int ACT, bool FAST>
+__global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * 128 + (wave >> 1) * 64;
+    const int col0 = blockIdx.x * 128 + (wave & 1) * 64;
+    if (col0 >= a.M) return;
+    f32x4 acc[4][4];
+    mfma_mainloop<DT, FAST>(a, row0, col0, r16, g, acc);
+    const u16* res = static_cast<const u16*>(a.res);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int col = col0 + i * 16 + g * 4;   // lane holds columns col..col+3 of its rows
+        if (col >= a.M) continue;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (a.bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) if (col + e < a.M) bv[e] = a.bias[col + e];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t row = row0 + j * 16 + r16;
+            if (row >= a.rows) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int c = col + e;
+                if (c >= a.M) break;
+                float o = apply_act<ACT>(acc[i][j][e] + bv[e]);
+                if (res) o += DT::to_f(res[row * a.ldr + c]);
+                const bool second = a.y2 && c >= a.split;
+                void* dst = second ? a.y2 : a.y;
+                const int64_t off = second ? row * a.ldy2 + (c - a.split) : row * a.ldy + c;
+                if (a.out_f32) static_cast<float*>(dst)[off] = o;
+                else static_cast<u16*>(dst)[off] = DT::from_f(o);
+            }
+        }
+    }
+}
+
+// Vector epilogue: M % 4 == 0, 4-element-aligned strides, no split: 8/16-byte stores.
+template <typename DT, int ACT>
+__global__ __launch_bounds__(256) void linear_mfma_vec_kernel(LinArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * 128 + (wave >> 1) * 64;
+    const int col0 = blockIdx.x * 128 + (wave & 1) * 64;
+    if (col0 >= a.M) return;
+    f32x4 acc[4][4];
+    mfma_mainloop<DT, true>(a, row0, col0, r16, g, acc);
+    const u16* res = static_cast<const u16*>(a.res);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int col = col0 + i * 16 + g * 4;
+        if (col >= a.M) continue;
+        float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a.bias) bv = *reinterpret_cast<const float4*>(a.bias + col);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t row = row0 + j * 16 + r16;
+            if (row >= a.rows) continue;
+            float o[4] = {apply_act<ACT>(acc[i][j][0] + bv.x), apply_act<ACT>(acc[i][j][1] + bv.y),
+                          apply_act<ACT>(acc[i][j][2] + bv.z), apply_act<ACT>(acc[i][j][3] + bv.w)};
+            if (res) {
+                uint2 rv = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
+                o[0] += DT::to_f((u16)(rv.x & 0xffff)); o[1] += DT::to_f((u16)(rv.x >> 16));
+                o[2] += DT::to_f((u16)(rv.y & 0xffff)); o[3] += DT::to_f((u16)(rv.y >> 16));
+            }
+            if (a.out_f32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(a.y) + row * a.ldy + col) = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+                uint2 ov;
+                ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
+                ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                *reinterpret_cast<uint2*>(static_cast<u16*>(a.y) + row * a.ldy + col) = ov;
+            }
+        }
+    }
+}
+
+// ---- fp32: 64x64 tile, K step 16, 4x4 outputs per thread -----------------------
+template <int ACT>
+__global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs a) {
+    __shared__ float xs[16][64 + 1];
+    __shared__ float ws[16][64 + 1];
+    const float* x = static_cast<const float*>(a.x);
+    const float* w = static_cast<const float*>(a.w);
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * 64;
+    const int col0 = blockIdx.x * 64;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < a.K; k0 += 16) {
+        for (int i = threadIdx.x; i < 64 * 16; i += 256) {
+            const int r = i >> 4, k = i & 15;
+            const int64_t row = row0 + r; const int col = col0 + r;
+            xs[k][r] = (row < a.rows && k0 + k < a.K) ? x[row * a.ldx + k0 + k] : 0.f;
+            ws[k][r] = (col < a.M && k0 + k < a.K) ? w[(int64_t)col * a.K + k0 + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            float xv[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { xv[i] = xs[k][ty * 4 + i]; wv[i] = ws[k][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    const float* res = static_cast<const float*>(a.res);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t row = row0 + ty * 4 + i;
+        if (row >= a.rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = col0 + tx * 4 + j;
+            if (c >= a.M) continue;
+            float o = apply_act<ACT>(acc[i][j] + (a.bias ? a.bias[c] : 0.f));
+            if (res) o += res[row * a.ldr + c];
+            if (a.y2 && c >= a.split) static_cast<float*>(a.y2)[row * a.ldy2 + (c - a.split)] = o;
+            else static_cast<float*>(a.y)[row * a.ldy + c] = o;
+        }
+    }
+}
+
+template <typename DT>
+void launch16(const LinArgs& a, int act, bool fast, bool vec, hipStream_t st) {
+    dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.rows + 127) / 128));
+#define GO(ACT) do { \
+        if (vec) hipLaunchKernelGGL((linear_mfma_vec_kernel<DT, ACT>), grid, dim3(256), 0, st, a); \
+        else if (fast) hipLaunchKernelGGL((linear_mfma_kernel<DT, ACT, true>), grid, dim3(256), 0, st, a); \
+        else hipLaunchKernelGGL((linear_mfma_kernel<DT, ACT, false>), grid, dim3(256), 0, st, a); } while (0)
+    if (act == BSRL_ACT_RELU) GO(BSRL_ACT_RELU);
+    else if (act == BSRL_ACT_GELU) GO(BSRL_ACT_GELU);
+    else GO(BSRL_ACT_NONE);
+#undef GO
+}
+
+}  // namespace
+
+extern "C" int bsrl_linear(const void* x, int64_t ldx, const void* w, const float* bias, const void* residual,
+                           int64_t ldr, void* y, int64_t ldy, void* y2, int64_t ldy2, int64_t split,
+                           int64_t rows, int64_t K, int64_t M, int act, int dtype, int out_dtype,
+                           bsrl_stream stream) {
+    if (!x || !w || !y) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: null pointer");
+    if (rows < 0 || K <= 0 || M <= 0 || K > (1 << 20) || M > (1 << 20))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad shape rows=%lld K=%lld M=%lld", (long long)rows, (long long)K, (long long)M);
+    if (ldx < K || ldy < (y2 ? split : M) || (residual && ldr < M))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: row stride smaller than row");
+    if (y2 && (split <= 0 || split >= M || ldy2 < M - split)) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad split");
+    if (act < 0 || act > 2) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad act %d", act);
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad dtype");
+    if (out_dtype != dtype && out_dtype != BSRL_F32) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: out_dtype must be dtype or F32");
+    if (rows == 0) return BSRL_OK;
+    if ((rows + 127) / 128 > 65535 * 16) return BSRL_UNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    LinArgs a{x, ldx, w, bias, residual, ldr, y, ldy, y2, ldy2, split, rows, (int)K, (int)M, out_dtype == BSRL_F32};
+    if (dtype == BSRL_F32) {
+        dim3 grid((unsigned)((M + 63) / 64), (unsigned)((rows + 63) / 64));
+        if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_RELU>), grid, dim3(256), 0, st, a);
+        else if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_GELU>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_NONE>), grid, dim3(256), 0, st, a);
+    } else {
+        const bool fast = K % 8 == 0 && ldx % 8 == 0 && bsrl_aligned(x, 16) && bsrl_aligned(w, 16);
+        const int osz = out_dtype == BSRL_F32 ? 4 : 2;
+        const bool vec = fast && !y2 && M % 4 == 0 && ldy % 4 == 0 && bsrl_aligned(y, 4 * osz) &&
+                         (!bias || bsrl_aligned(bias, 16)) &&
+                         (!residual || (ldr % 4 == 0 && bsrl_aligned(residual, 8)));
+        if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
+        else launch16<BF16>(a, act, fast, vec, st);
+    }
+    BSRL_CHECK_LAUNCH("bsrl_linear");
+    return BSRL_OK;
+}

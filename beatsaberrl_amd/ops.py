@@ -1,0 +1,229 @@
+"""Tensor-level wrappers of the C-ABI entry points.
+
+Each function checks what the kernel assumes (device, dtype, contiguity),
+allocates the outputs with torch (device memory + stream are torch's; the
+arithmetic is not), and enqueues on torch's current stream.  Outputs are fresh
+tensors and inputs are only borrowed - the ownership convention of the
+reference's extension ops (python/beat_arena_env/csrc/layer_norm.cu:545-547).
+A False / None return means "the kernel set does not cover this shape"
+(the reference signals the same with an empty list, fp16_gemm.cu:346-357)."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import ACT_GELU, ACT_NONE, ACT_RELU, BF16, F16, F32
+
+_DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "gelu": ACT_GELU}
+
+
+class Unsupported(RuntimeError):
+    """The kernel set has no kernel for the requested shape/dtype."""
+
+
+def dt_code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}") from None
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("bsrl ops need device tensors (there is no CPU path)")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _f32c(t, name):
+    if t is None:
+        return None
+    if t.dtype is not torch.float32 or not t.is_contiguous():
+        raise TypeError(f"{name} must be a contiguous fp32 tensor")
+    return t
+
+
+def ln_fwd(x, weight, bias, eps=1e-5, want_stats=False):
+    """y = LayerNorm(x) over the last dim; fp32 weight/bias/stats."""
+    _need_cuda(x, weight, bias)
+    d = x.shape[-1]
+    if not x.is_contiguous():
+        raise RuntimeError("ln_fwd: x must be contiguous")
+    rows = x.numel() // d
+    y = torch.empty_like(x)
+    mean = rstd = None
+    if want_stats:
+        mean = torch.empty(rows, device=x.device, dtype=torch.float32)
+        rstd = torch.empty(rows, device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_ln_fwd(x.data_ptr(), _f32c(weight, "weight").data_ptr(), _f32c(bias, "bias").data_ptr(),
+                                     y.data_ptr(), _ptr(mean), _ptr(rstd), rows, d, float(eps), dt_code(x.dtype),
+                                     _stream(x))
+    if not _lib.check(rc, "bsrl_ln_fwd"):
+        raise Unsupported(f"ln_fwd d={d} dtype={x.dtype}")
+    return (y, mean, rstd) if want_stats else y
+
+
+def ln_fwd_add(a, b, weight, bias, eps=1e-5, b_bias=None, want_stats=False):
+    """x = round(a + (b + b_bias)); y = LayerNorm(x).  Returns (x, y[, mean, rstd])."""
+    _need_cuda(a, b, weight, bias, b_bias)
+    if a.shape != b.shape or a.dtype is not b.dtype or not (a.is_contiguous() and b.is_contiguous()):
+        raise RuntimeError("ln_fwd_add: a and b must be contiguous with equal shape and dtype")
+    d = a.shape[-1]
+    rows = a.numel() // d
+    x = torch.empty_like(a)
+    y = torch.empty_like(a)
+    mean = rstd = None
+    if want_stats:
+        mean = torch.empty(rows, device=a.device, dtype=torch.float32)
+        rstd = torch.empty(rows, device=a.device, dtype=torch.float32)
+    with torch.cuda.device(a.device):
+        rc = _lib.load().bsrl_ln_fwd_add(a.data_ptr(), b.data_ptr(), _ptr(_f32c(b_bias, "b_bias")),
+                                         _f32c(weight, "weight").data_ptr(), _f32c(bias, "bias").data_ptr(),
+                                         x.data_ptr(), y.data_ptr(), _ptr(mean), _ptr(rstd), rows, d, float(eps),
+                                         dt_code(a.dtype), _stream(a))
+    if not _lib.check(rc, "bsrl_ln_fwd_add"):
+        raise Unsupported(f"ln_fwd_add d={d} dtype={a.dtype}")
+    return (x, y, mean, rstd) if want_stats else (x, y)
+
+
+def _rows2d(t):
+    """View t (..., K) as rows with one row stride; returns (tensor, rows, ld)."""
+    K = t.shape[-1]
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    if t.dim() == 1:
+        return t, 1, K
+    if t.dim() == 2:
+        return t, t.shape[0], t.stride(0)
+    # collapse leading dims if they form one stride
+    lead = t.shape[:-1]
+    st = t.stride()[:-1]
+    ld = st[-1]
+    ok = all(st[i] == st[i + 1] * lead[i + 1] for i in range(len(lead) - 1))
+    if not ok:
+        t = t.contiguous()
+        ld = K
+    rows = 1
+    for n in lead:
+        rows *= n
+    return t, rows, ld
+
+
+def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None):
+    """act(x @ w.T + bias) (+ residual).  x (..., K) in w's dtype, w (M, K)
+    contiguous, bias fp32.  split=s returns (y[..., :s], y[..., s:]) as two
+    separately stored tensors."""
+    _need_cuda(x, w, bias, residual)
+    if x.dtype is not w.dtype:
+        raise TypeError(f"linear: x is {x.dtype} but w is {w.dtype}")
+    if not w.is_contiguous() or w.dim() != 2:
+        raise RuntimeError("linear: w must be a contiguous (M, K) matrix")
+    M, K = w.shape
+    if x.shape[-1] != K:
+        raise RuntimeError(f"linear: x has K={x.shape[-1]}, w has K={K}")
+    out_dtype = out_dtype or x.dtype
+    lead = x.shape[:-1]
+    x2, rows, ldx = _rows2d(x)
+    r2, ldr = None, 0
+    if residual is not None:
+        if residual.dtype is not x.dtype or residual.shape != (*lead, M):
+            raise RuntimeError("linear: residual must be (..., M) in x's dtype")
+        r2, _, ldr = _rows2d(residual)
+    if split is None:
+        y = torch.empty(*lead, M, device=x.device, dtype=out_dtype)
+        y2, ld2, sp = None, 0, 0
+        ldy = M
+    else:
+        y = torch.empty(*lead, split, device=x.device, dtype=out_dtype)
+        y2 = torch.empty(*lead, M - split, device=x.device, dtype=out_dtype)
+        ldy, ld2, sp = split, M - split, split
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_linear(x2.data_ptr(), ldx, w.data_ptr(), _ptr(_f32c(bias, "bias")), _ptr(r2), ldr,
+                                     y.data_ptr(), ldy, _ptr(y2), ld2, sp, rows, K, M, _ACT[act],
+                                     dt_code(x.dtype), dt_code(out_dtype), _stream(x))
+    if not _lib.check(rc, "bsrl_linear"):
+        raise Unsupported(f"linear rows={rows} K={K} M={M} dtype={x.dtype}")
+    return y if split is None else (y, y2)
+
+
+def attn_fwd(q, k, v, n_heads, key_bias=None, n_valid=None):
+    """softmax(q k^T / sqrt(dh) + key_bias) v per head.  q (B, TQ, d), k/v
+    (B, T, d): any batch/row strides (views of a packed projection are fine),
+    unit last stride.  key_bias (B, T) additive in q's dtype, or n_valid (B,)
+    int32 (keys 0..n_valid[b] attendable).  Returns (B, TQ, d) contiguous."""
+    _need_cuda(q, k, v, key_bias, n_valid)
+    B, TQ, d = q.shape
+    T = k.shape[1]
+    if k.shape != (B, T, d) or v.shape != (B, T, d) or d % n_heads:
+        raise RuntimeError("attn_fwd: shape mismatch")
+    for t in (q, k, v):
+        if t.stride(2) != 1 or t.dtype is not q.dtype:
+            raise RuntimeError("attn_fwd: q/k/v need unit last stride and one dtype")
+    if key_bias is not None:
+        if key_bias.shape != (B, T) or key_bias.dtype is not q.dtype or not key_bias.is_contiguous():
+            raise RuntimeError("attn_fwd: key_bias must be contiguous (B, T) in q's dtype")
+    if n_valid is not None:
+        if n_valid.shape != (B,) or n_valid.dtype is not torch.int32 or not n_valid.is_contiguous():
+            raise RuntimeError("attn_fwd: n_valid must be contiguous int32 (B,)")
+    out = torch.empty(B, TQ, d, device=q.device, dtype=q.dtype)
+    with torch.cuda.device(q.device):
+        rc = _lib.load().bsrl_attn_fwd(q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1),
+                                       v.data_ptr(), v.stride(0), v.stride(1), _ptr(key_bias), _ptr(n_valid),
+                                       out.data_ptr(), B, T, TQ, n_heads, d // n_heads, dt_code(q.dtype), _stream(q))
+    if not _lib.check(rc, "bsrl_attn_fwd"):
+        raise Unsupported(f"attn_fwd T={T} TQ={TQ} H={n_heads} dh={d // n_heads} dtype={q.dtype}")
+    return out
+
+
+def ffn_fused_supported(d, F, dtype) -> bool:
+    return bool(_lib.load().bsrl_ffn_fused_supported(d, F, dt_code(dtype)))
+
+
+def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5):
+    """xo = x + act(h2 w0^T + b0) w2^T + b2; ho = LN(xo) when ln_w is given.
+    Returns (xo, ho) (ho None without LN), or None when unsupported."""
+    _need_cuda(x, h2, w0, w2)
+    d = x.shape[-1]
+    Fh = w0.shape[0]
+    if not (x.is_contiguous() and h2.is_contiguous() and w0.is_contiguous() and w2.is_contiguous()):
+        raise RuntimeError("ffn_fused: contiguous tensors required")
+    rows = x.numel() // d
+    xo = torch.empty_like(x)
+    ho = torch.empty_like(x) if ln_w is not None else None
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_ffn_fused(x.data_ptr(), h2.data_ptr(), w0.data_ptr(), _f32c(b0, "b0").data_ptr(),
+                                        w2.data_ptr(), _f32c(b2, "b2").data_ptr(), _ptr(_f32c(ln_w, "ln_w")),
+                                        _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), rows, d, Fh,
+                                        _ACT[act], dt_code(x.dtype), _stream(x))
+    if not _lib.check(rc, "bsrl_ffn_fused"):
+        return None
+    return xo, ho
+
+
+def cfg_embed(obs, wp, bp, wo, bo, T, dtype):
+    """Config-model tokenizer: obs (B, obs_dim) fp32 or `dtype` -> tokens (B, T, d)."""
+    _need_cuda(obs, wp, wo)
+    B = obs.shape[0]
+    d, prop_dim = wp.shape
+    obj_dim = wo.shape[1]
+    if obs.stride(1) != 1 or not (wp.is_contiguous() and wo.is_contiguous()):
+        raise RuntimeError("cfg_embed: contiguous rows required")
+    if wp.dtype is not dtype or wo.dtype is not dtype:
+        raise TypeError("cfg_embed: weights must be in the stream dtype")
+    tokens = torch.empty(B, T, d, device=obs.device, dtype=dtype)
+    with torch.cuda.device(obs.device):
+        rc = _lib.load().bsrl_cfg_embed(obs.data_ptr(), obs.stride(0), dt_code(obs.dtype), wp.data_ptr(),
+                                        _ptr(_f32c(bp, "bp")), wo.data_ptr(), _ptr(_f32c(bo, "bo")),
+                                        tokens.data_ptr(), B, T, d, prop_dim, obj_dim, dt_code(dtype), _stream(obs))
+    if not _lib.check(rc, "bsrl_cfg_embed"):
+        raise Unsupported(f"cfg_embed T={T} d={d}")
+    return tokens

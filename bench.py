@@ -1,0 +1,181 @@
+"""Headline benchmark: policy-forward env-samples/s at B = 16384, fp16, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--route auto|fused|ops]
+                    [--config 1] [--batch B] [--no-cpu] [--no-eager]
+
+A step is one whole forward (obs -> 29x7 logits + value) of the benchmark's
+config[1] model over B device-resident synthetic observations.  Prints ONE JSON
+line.  Protocol after the reference's harness (python/bench_policy_forward.py:
+72-83): inputs on the device, warm-up, timed loop closed by one device sync.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+HBM_PEAK_GBS = 8000.0
+
+
+def torch_eager_forward(m, obs, n_valid, dt):
+    """Plain torch-ROCm eager forward of the same module in the stream dtype:
+    the denominator of the '>= 10x eager' target (baseline only)."""
+    import torch
+    import torch.nn.functional as F
+    B, T, d, H = obs.shape[0], m.T, m.d, m.n_heads
+    c = lambda t: t.to(dt)
+    o = obs.to(dt)
+    t0 = F.linear(o[:, :m.prop_dim], c(m.prop_embed.weight), c(m.prop_embed.bias)).unsqueeze(1)
+    tj = F.linear(o[:, m.prop_dim:].reshape(B, T - 1, m.obj_dim), c(m.obj_embed.weight), c(m.obj_embed.bias))
+    x = torch.cat([t0, tj], 1)
+    bias = None
+    if n_valid is not None:
+        valid = torch.arange(T, device=obs.device)[None, :] <= n_valid[:, None]
+        bias = ((valid.to(dt) - 1.0) * 16384.0).view(B, 1, 1, T)
+    for blk in m.blocks:
+        h = F.layer_norm(x.float(), (d,), blk.ln_attn.weight, blk.ln_attn.bias, 1e-5).to(dt)
+        q = F.linear(h, c(blk.q_proj.weight), c(blk.q_proj.bias)).view(B, T, H, d // H).transpose(1, 2)
+        k = F.linear(h, c(blk.k_proj.weight), c(blk.k_proj.bias)).view(B, T, H, d // H).transpose(1, 2)
+        v = F.linear(h, c(blk.v_proj.weight), c(blk.v_proj.bias)).view(B, T, H, d // H).transpose(1, 2)
+        att = F.scaled_dot_product_attention(q, k, v, attn_mask=bias).transpose(1, 2).reshape(B, T, d)
+        x = x + F.linear(att, c(blk.out_proj.weight), c(blk.out_proj.bias))
+        h2 = F.layer_norm(x.float(), (d,), blk.ln_ffn.weight, blk.ln_ffn.bias, 1e-5).to(dt)
+        hid = F.linear(h2, c(blk.ffn[0].weight), c(blk.ffn[0].bias))
+        hid = F.gelu(hid) if m.act == "gelu" else F.relu(hid)
+        x = x + F.linear(hid, c(blk.ffn[2].weight), c(blk.ffn[2].bias))
+    hh = x[:, 0]
+    if m.final_ln is not None:
+        hh = F.layer_norm(hh.float(), (d,), m.final_ln.weight, m.final_ln.bias, 1e-5).to(dt)
+    out = F.linear(hh, c(m.heads.weight), c(m.heads.bias)).float()
+    return out[:, :-1].reshape(B, 29, m.n_gears), out[:, -1]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--route", default="auto", choices=("auto", "fused", "ops"))
+    ap.add_argument("--config", type=int, default=1, help="benchmark config index (1 = headline)")
+    ap.add_argument("--batch", type=int, default=0, help="override B (0 = the config's B)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-eager", action="store_true", help="skip the torch-ROCm eager leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures ONE GPU: the forward is embarrassingly data-parallel (env rows are "
+                 "independent, weights replicated, no exchange), so this build has no multi-GPU path; "
+                 "run with --gpus 1.")
+
+    import torch
+    from beatsaberrl_amd import _lib
+    from beatsaberrl_amd.config_policy import ConfigPolicy
+    from oracle import config_model as cm     # checker / CPU baseline only
+    _lib.load()
+    dev = torch.device("cuda:0")
+    c = cm.CONFIGS[args.config]
+    spec, dtype = c["spec"], c["dtype"]
+    B = args.batch or c["B"]
+    p = cm.init_params(spec, c["w_seed"])
+    obs_cpu, k_cpu = cm.make_inputs(spec, B, c["obs_seed"], c["mask"])
+    m = ConfigPolicy.from_spec(spec, dtype=dtype, route=args.route)
+    m.load_state_dict(p)
+    m = m.to(dev)
+    obs, k = obs_cpu.to(dev), k_cpu.to(dev)
+    route = args.route
+    if route == "auto":
+        route = "fused" if m.fused_supported() else "ops"
+
+    def step():
+        return m.forward_stacked(obs, k, route=route)
+
+    # parity spot check on the first 256 envs before timing anything
+    lg, v = step()
+    ref_lg, ref_v = cm.forward(p, spec, obs_cpu[:256], k_cpu[:256], emulate=None if dtype == "f32" else dtype,
+                               round_residual=(route == "ops"))
+    parity = (lg[:256].float().cpu() - ref_lg).abs().max().item()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for s, e in ev:
+        s.record()
+        step()
+        e.record()
+    torch.cuda.synchronize()
+    dt_s = time.perf_counter() - t0
+    ms_per_step = dt_s / args.steps * 1e3
+    dev_ms = sorted(s.elapsed_time(e) for s, e in ev)
+    dev_ms_avg = sum(dev_ms) / len(dev_ms)
+    value = B / (ms_per_step * 1e-3)
+
+    flops = cm.flops_per_env(spec) * B
+    # Dominant kernel: on the fused route the forward IS one kernel, so its launch
+    # duration is the event-bracketed step; on the ops route the events bracket the
+    # whole launch train and the figure is the pipeline's, not one kernel's.
+    achieved = flops / (dev_ms_avg * 1e-3) / 1e12
+    peak = MFMA_PEAK_TFLOPS[dtype]
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": None,
+                "kernel": "cfg_forward (whole forward)" if route == "fused" else "launch train (per-op route)",
+                "launch_ms_avg": round(dev_ms_avg, 4), "launch_ms_p50": round(dev_ms[len(dev_ms) // 2], 4),
+                "flop_per_launch": flops}
+
+    out = {"metric": "policy fwd env-samples/sec at B=16384 fp16 (1 GPU); % of MFMA roofline",
+           "value": round(value, 1), "unit": "env-samples/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+           "config": {"workload": f"config[{args.config}]: B={B} T={spec.T} d={spec.d} L={spec.n_layers} "
+                                  f"H={spec.n_heads}x{spec.dh} ffn={spec.ffn} {spec.act} {dtype}, "
+                                  f"key-padding mask '{c['mask']}', obs seed {c['obs_seed']}, weights seed {c['w_seed']}",
+                      "route": route, "batch": B, "parity_max_abs_logit_err_first256": round(parity, 6)},
+           "roofline": roofline}
+
+    if not args.no_eager:
+        tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
+        with torch.no_grad():
+            for _ in range(3):
+                torch_eager_forward(m, obs, k, tdt)
+            torch.cuda.synchronize()
+            n = 20
+            t0 = time.perf_counter()
+            for _ in range(n):
+                torch_eager_forward(m, obs, k, tdt)
+            torch.cuda.synchronize()
+            te = (time.perf_counter() - t0) / n
+        out["torch_eager"] = {"value": round(B / te, 1), "unit": "env-samples/s", "ms_per_step": round(te * 1e3, 4),
+                              "speedup": round(value / (B / te), 2)}
+
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            pass
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        torch.set_num_threads(cores)
+        nb = min(B, 16384)
+        for _ in range(2):
+            cm.forward(p, spec, obs_cpu[:nb], k_cpu[:nb])
+        ts = []
+        t_end = time.perf_counter() + 20.0
+        while len(ts) < 10 and (len(ts) < 3 or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            cm.forward(p, spec, obs_cpu[:nb], k_cpu[:nb])
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        out["cpu_baseline"] = {"value": round(nb / ts[len(ts) // 2], 1), "unit": "env-samples/s", "cores": cores,
+                               "kind": "port",
+                               "sample": f"oracle torch fp32 forward, B={nb} envs of the same workload, "
+                                         f"median of {len(ts)} after 2 warm-ups"}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,161 @@
+/* bsrl.h - C ABI of libbsrl_hip.so: the MI355X (gfx950) policy-forward kernels.
+ *
+ * Every entry point replaces one binding of the reference's two torch
+ * extension modules (python/beat_arena_env/csrc/layer_norm.cu:733-749 and
+ * python/beat_arena_env/csrc/fp16_gemm.cu:535-566) or one vendor call the
+ * reference's op layer makes (python/fp16_linear.py:134-181).  The ABI is plain
+ * C: raw device pointers, explicit sizes and strides (in ELEMENTS), a dtype
+ * enum and a HIP stream handle.  No entry point allocates, synchronises or
+ * keeps a pointer after it returns; all work is enqueued on `stream`
+ * (NULL = the null stream) and is safe to capture in a HIP graph.
+ *
+ * Return value of every int function: 0 = enqueued; >0 = the shape / dtype /
+ * alignment is not supported by this kernel set (the caller picks another
+ * route, the reference signals the same with an empty list,
+ * fp16_gemm.cu:346-357); <0 = invalid argument or HIP launch error, text in
+ * bsrl_last_error() (thread-local).
+ */
+#ifndef BSRL_H
+#define BSRL_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { BSRL_F32 = 0, BSRL_F16 = 1, BSRL_BF16 = 2 } bsrl_dtype;
+typedef enum { BSRL_ACT_NONE = 0, BSRL_ACT_RELU = 1, BSRL_ACT_GELU = 2 } bsrl_act;
+
+#define BSRL_OK 0
+#define BSRL_UNSUPPORTED 1
+#define BSRL_EINVAL (-1)
+#define BSRL_ELAUNCH (-2)
+
+#define BSRL_MASK_BIAS 16384.0f /* reference python/policy.py:428 */
+#define BSRL_MAX_T 48
+#define BSRL_MAX_LAYERS 8
+
+typedef void* bsrl_stream; /* hipStream_t */
+
+/* ABI version (bumped on any signature change). */
+int bsrl_version(void);
+/* Text of the last error on the calling thread ("" if none). */
+const char* bsrl_last_error(void);
+
+/* ---- LayerNorm ----------------------------------------------------------
+ * Replaces layer_norm_cuda.ln_fwd (layer_norm.cu:530-561): y = LN(x) over the
+ * last dim, fp32 weight/bias/statistics, x and y in `dtype`.  mean / rstd are
+ * optional (NULL to skip) fp32 (rows,) outputs.  x, y contiguous (rows, d). */
+int bsrl_ln_fwd(const void* x, const float* weight, const float* bias, void* y,
+                float* mean, float* rstd, int64_t rows, int64_t d, float eps,
+                int dtype, bsrl_stream stream);
+
+/* Replaces layer_norm_cuda.ln_fwd_add (layer_norm.cu:563-643):
+ * x = round(a + (b + b_bias)); y = LN(x) with statistics on the ROUNDED x.
+ * b_bias is an optional fp32 (d,) vector (NULL = none). */
+int bsrl_ln_fwd_add(const void* a, const void* b, const float* b_bias,
+                    const float* weight, const float* bias, void* x, void* y,
+                    float* mean, float* rstd, int64_t rows, int64_t d, float eps,
+                    int dtype, bsrl_stream stream);
+
+/* ---- Linear (+bias +activation +residual) --------------------------------
+ * Replaces the vendor GEMM calls of python/fp16_linear.py:134-181 (addmm / mm /
+ * _addmm_activation) and fp16_gemm.linear_relu_aux / bias_relu_
+ * (fp16_gemm.cu:77-111, 404-497):
+ *   y[r, m] = act( sum_k x[r, k] * w[m, k] + bias[m] ) + residual[r, m]
+ * x (rows, K) row stride ldx; w (M, K) contiguous nn.Linear layout in `dtype`;
+ * bias fp32 (M,) or NULL; residual in `dtype`, row stride ldr, or NULL;
+ * y row stride ldy in `out_dtype` (same as dtype, or BSRL_F32).
+ * If y2 != NULL, columns >= split go to y2[r * ldy2 + (m - split)] (fp32 when
+ * out_dtype is F32) - used to split packed heads | value.
+ * 16-bit dtypes run MFMA with fp32 accumulate; F32 runs an FMA kernel. */
+int bsrl_linear(const void* x, int64_t ldx, const void* w, const float* bias,
+                const void* residual, int64_t ldr, void* y, int64_t ldy,
+                void* y2, int64_t ldy2, int64_t split,
+                int64_t rows, int64_t K, int64_t M, int act, int dtype,
+                int out_dtype, bsrl_stream stream);
+
+/* ---- Short-sequence masked multi-head attention ----------------------------
+ * Replaces fp16_gemm.attn29_fwd (small_attn.cu:515-536) and the SDPA / fp32
+ * fallbacks it shadows (python/policy.py:684-690):
+ *   out[b, tq, h*dh:(h+1)*dh] = softmax_k(q.k / sqrt(dh) + key_bias[b, k]) v
+ * q (B, TQ, H*dh): element (b,t,c) at q[b*q_bs + t*q_rs + c]; likewise k, v
+ * (B, T, H*dh) with their own strides, so q|k|v may be views of one packed
+ * projection.  The key mask is either key_bias (B, T) in `dtype` (additive,
+ * 0 or -2^14) or n_valid (B,) int32 (keys 0..n_valid[b] attendable); pass one,
+ * or neither for no mask.  out (B, TQ, H*dh) contiguous in `dtype`.
+ * T <= 48, TQ <= T, dh in {32, 48} (16-bit) or any dh <= 64 (F32). */
+int bsrl_attn_fwd(const void* q, int64_t q_bs, int64_t q_rs,
+                  const void* k, int64_t k_bs, int64_t k_rs,
+                  const void* v, int64_t v_bs, int64_t v_rs,
+                  const void* key_bias, const int32_t* n_valid, void* out,
+                  int64_t B, int64_t T, int64_t TQ, int64_t H, int64_t dh,
+                  int dtype, bsrl_stream stream);
+
+/* ---- Fused FFN ------------------------------------------------------------
+ * Replaces fp16_gemm.ffn_fused (fused_ffn.cu:551-619):
+ *   xo = x + act(h2 w0^T + b0) w2^T + b2 ;  ho = LN_next(xo) if ln_w != NULL
+ * x, h2, xo, ho (rows, d) contiguous in `dtype` (16-bit only); w0 (F, d),
+ * w2 (d, F) in `dtype`; b0, b2, ln_w, ln_b fp32.  The hidden never reaches
+ * memory.  d in {128, 192, 256, 384}, F = multiple of 32. */
+int bsrl_ffn_fused(const void* x, const void* h2, const void* w0, const float* b0,
+                   const void* w2, const float* b2, const float* ln_w,
+                   const float* ln_b, float eps, void* xo, void* ho,
+                   int64_t rows, int64_t d, int64_t F, int act, int dtype,
+                   bsrl_stream stream);
+/* Mirrors fp16_gemm.ffn_fused_supported (fused_ffn.cu:509-525): 1 if the
+ * (d, F, dtype) combination has a kernel. */
+int bsrl_ffn_fused_supported(int64_t d, int64_t F, int dtype);
+
+/* ---- Config-model tokenizer -----------------------------------------------
+ * The benchmark configs' "linear embedding": token 0 = Wp obs[:, :prop_dim] +
+ * bp, token j = Wo obs[:, prop_dim + (j-1)*obj_dim : ...] + bo
+ * (the reference's encoder stage, python/policy.py:1224-1249, reduced to one
+ * Linear per token type).  obs (B, obs_ld) in obs_dtype (F32 or `dtype`),
+ * rounded once to `dtype` like python/policy.py:1200-1209; wp (d, prop_dim),
+ * wo (d, obj_dim) in `dtype`; tokens (B, T, d) contiguous in `dtype`. */
+int bsrl_cfg_embed(const void* obs, int64_t obs_ld, int obs_dtype,
+                   const void* wp, const float* bp, const void* wo, const float* bo,
+                   void* tokens, int64_t B, int64_t T, int64_t d,
+                   int64_t prop_dim, int64_t obj_dim, int dtype, bsrl_stream stream);
+
+/* ---- Whole config-model forward in one persistent kernel -------------------
+ * Replaces NotePolicy.forward_stacked (python/policy.py:1179-1344) for the
+ * benchmark-config model: obs -> logits (B, 29*n_gears) fp32 + value (B,) fp32.
+ * `packed` is the weight image written by bsrl_cfg_pack() for the same
+ * (n_layers, d, n_heads, ffn, T) - the analogue of the reference's flat fp16
+ * replica buffer (python/fp16_linear.py:249-346): rebuilt after each optimizer
+ * step, its address must not move while a captured graph replays. */
+typedef struct {
+    int32_t n_layers, d, n_heads, ffn, T, n_gears, act, final_ln;
+    int32_t prop_dim, obj_dim, dtype, reserved;
+} bsrl_cfg_desc;
+
+/* fp32 master parameter pointers in state_dict order (device memory). */
+typedef struct {
+    const float *prop_w, *prop_b, *obj_w, *obj_b;
+    struct {
+        const float *ln_attn_w, *ln_attn_b, *q_w, *q_b, *k_w, *k_b, *v_w, *v_b,
+            *out_w, *out_b, *ln_ffn_w, *ln_ffn_b, *ffn0_w, *ffn0_b, *ffn2_w, *ffn2_b;
+    } blk[BSRL_MAX_LAYERS];
+    const float *final_ln_w, *final_ln_b, *heads_w, *heads_b;
+} bsrl_cfg_params;
+
+/* Bytes of the packed image for `desc`, or 0 if the fused kernel does not
+ * support this shape (use the per-op entry points instead). */
+int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* desc);
+/* One cast+permute pass: fp32 masters -> packed 16-bit MFMA-fragment-major
+ * image (the analogue of fp16_linear.flat_refresh, fp16_linear.py:241-246). */
+int bsrl_cfg_pack(const bsrl_cfg_desc* desc, const bsrl_cfg_params* params,
+                  void* packed, bsrl_stream stream);
+/* obs (B, obs_ld) F32 or 16-bit; n_valid (B,) int32 or NULL (all valid). */
+int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
+                     const void* obs, int64_t obs_ld, int obs_dtype,
+                     const int32_t* n_valid, float* logits, float* value,
+                     int64_t B, bsrl_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSRL_H */

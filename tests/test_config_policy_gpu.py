@@ -1,0 +1,124 @@
+"""GPU parity of ConfigPolicy.forward_stacked (all kernels through the C ABI)
+against the CPU oracle on identical seeded weights and inputs.
+
+Gates (stated by the benchmark definition):
+  * fp32: <= 1e-5 relative (here: |d| <= 1e-5 * (|ref| + max|ref|))
+  * fp16 / bf16 logits: <= 2e-3 absolute against the oracle evaluated in the
+    same precision class (weights and GEMM operands rounded to the 16-bit type,
+    fp32 accumulate and statistics).  Against the pure-fp32 oracle a 16-bit
+    stream cannot hold 2e-3 on O(1..10) logits (the rounding-emulating oracle
+    itself is 4e-3 off at fp16 and 3e-2 at bf16), so that comparison uses the
+    reference's idiom "no worse than the replaced path's own error"
+    (python/tests/test_attn29.py:110-111): e_mine <= max(1.25 * e_emul, 2e-3).
+  * argmax gear actions identical wherever the oracle's top-2 margin > 1e-2.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from beatsaberrl_amd.config_policy import ConfigPolicy  # noqa: E402
+from oracle import config_model as cm  # noqa: E402
+
+DEV = "cuda"
+
+
+def _build(spec, seed, dtype, route, randomize_affine=True):
+    p = cm.init_params(spec, seed, randomize_affine=randomize_affine)
+    m = ConfigPolicy.from_spec(spec, dtype=dtype, route=route)
+    m.load_state_dict(p)
+    return p, m.to(DEV)
+
+
+def _check16(lg, v, p, spec, obs, k, dtype, round_residual):
+    lg, v = lg.float().cpu(), v.float().cpu()
+    ref_lg, ref_v = cm.forward(p, spec, obs, k)
+    em_lg, em_v = cm.forward(p, spec, obs, k, emulate=dtype, round_residual=round_residual)
+    e_class = (lg - em_lg).abs().max().item()
+    e_val = (v - em_v).abs().max().item()
+    e_mine = (lg - ref_lg).abs().max().item()
+    e_emul = (em_lg - ref_lg).abs().max().item()
+    print(f"\n[{dtype}] vs same-precision oracle: logits {e_class:.2e} value {e_val:.2e}; "
+          f"vs fp32 oracle: mine {e_mine:.2e}, emulated oracle {e_emul:.2e}")
+    assert e_class <= 2e-3 and e_val <= 2e-3
+    assert e_mine <= max(1.25 * e_emul, 2e-3)
+    # argmax gate against the same-precision oracle, and against fp32 where the class error allows
+    for name, r in (("class", em_lg), ("fp32", ref_lg)):
+        if name == "fp32" and dtype == "bf16":
+            continue
+        decided = cm.top2_margin(r) > 1e-2
+        same = lg.argmax(-1) == r.argmax(-1)
+        assert bool((same | ~decided).all()), f"argmax differs on a decided head ({name})"
+        assert decided.float().mean() > 0.5
+
+
+def test_config0_fp32_b256():
+    c = cm.CONFIGS[0]
+    spec = c["spec"]
+    p, m = _build(spec, c["w_seed"], "f32", "ops", randomize_affine=False)
+    obs, k = cm.make_inputs(spec, c["B"], c["obs_seed"], c["mask"])
+    lg, v = m.forward_stacked(obs.to(DEV), None)
+    ref_lg, ref_v = cm.forward(p, spec, obs, None)
+    assert lg.shape == (256, 29, 7) and lg.dtype is torch.float32 and v.shape == (256,)
+    scale = ref_lg.abs().max().item()
+    err = (lg.cpu() - ref_lg).abs()
+    assert bool((err <= 1e-5 * (ref_lg.abs() + scale)).all()), err.max().item()
+    assert bool(((v.cpu() - ref_v).abs() <= 1e-5 * (ref_v.abs() + ref_v.abs().max())).all())
+    assert torch.equal(lg.cpu().argmax(-1), ref_lg.argmax(-1)) or bool(
+        ((lg.cpu().argmax(-1) == ref_lg.argmax(-1)) | (cm.top2_margin(ref_lg) <= 1e-2)).all())
+    # the masked variant of the same model, fp32
+    obs2, k2 = cm.make_inputs(spec, 64, 9, "uniform")
+    lg2, v2 = m.forward_stacked(obs2.to(DEV), k2.to(DEV))
+    r2, rv2 = cm.forward(p, spec, obs2, k2)
+    assert bool(((lg2.cpu() - r2).abs() <= 1e-5 * (r2.abs() + r2.abs().max())).all())
+
+
+@pytest.mark.parametrize("ci,B", [(1, 1024), (2, 192), (3, 48), (4, 64), (4, 8), (4, 1)])
+def test_configs_16bit_ops_route(ci, B):
+    c = cm.CONFIGS[ci]
+    spec = c["spec"]
+    p, m = _build(spec, c["w_seed"], c["dtype"], "ops")
+    obs, k = cm.make_inputs(spec, B, c["obs_seed"], c["mask"])
+    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    _check16(lg, v, p, spec, obs, k, c["dtype"], round_residual=True)
+
+
+@pytest.mark.parametrize("act,final_ln,dtype", [("relu", True, "f16"), ("gelu", True, "bf16"), ("relu", False, "f32")])
+def test_variants_ops_route(act, final_ln, dtype):
+    spec = cm.ConfigSpec(3, 128, 4, 256, 16, act=act, final_ln=final_ln)
+    p, m = _build(spec, 21, dtype, "ops")
+    obs, k = cm.make_inputs(spec, 100, 22, "quarter_empty")
+    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    if dtype == "f32":
+        r, rv = cm.forward(p, spec, obs, k)
+        assert bool(((lg.cpu() - r).abs() <= 1e-5 * (r.abs() + r.abs().max())).all())
+    else:
+        _check16(lg, v, p, spec, obs, k, dtype, round_residual=True)
+
+
+def test_masked_slots_cannot_change_outputs_on_gpu():
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    p, m = _build(spec, 1, "f16", "ops")
+    obs, k = cm.make_inputs(spec, 64, 3, "uniform")
+    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    obs2 = obs.clone()
+    for e in range(64):
+        obs2[e, spec.prop_dim + int(k[e]) * spec.obj_dim:] = 77.0
+    lg2, v2 = m.forward_stacked(obs2.to(DEV), k.to(DEV))
+    assert torch.equal(lg, lg2) and torch.equal(v, v2)
+
+
+def test_weights_version_refreshes_replicas():
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    p, m = _build(spec, 1, "f16", "ops")
+    obs, k = cm.make_inputs(spec, 16, 3, "uniform")
+    a, _ = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    with torch.no_grad():
+        m.heads.bias.add_(1.0)
+    b, _ = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    assert torch.equal(a, b)              # stale replica until the version is bumped
+    m.bump_weights_version()
+    c2, _ = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    assert torch.allclose(c2, a + 1.0, atol=1e-3)

@@ -1,0 +1,235 @@
+"""GPU parity of the per-op kernels (called through the C ABI via
+beatsaberrl_amd.ops) against closed forms / library routines evaluated in
+fp64 or fp32 on the same rounded operands - the reference's own test idiom
+(python/tests/test_fused_ln.py:29-88, test_attn29.py:49-154,
+test_fp16_accum.py:84-89)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+from beatsaberrl_amd import ops  # noqa: E402
+
+DEV = "cuda"
+DTS = [torch.float32, torch.float16, torch.bfloat16]
+EPS16 = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
+
+
+def _rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+# ---------------------------------------------------------------- LayerNorm
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,d", [(1, 128), (7, 128), (1000, 128), (257, 192), (64, 256), (33, 384), (5, 512),
+                                    (3, 1024), (130, 64), (9, 40)])
+def test_ln_fwd(dtype, rows, d):
+    x = _rand(rows, d, dtype=dtype, seed=rows + d, scale=2.0) + 0.5
+    w = _rand(d, seed=1) * 0.3 + 1.0
+    b = _rand(d, seed=2) * 0.3
+    y, mean, rstd = ops.ln_fwd(x, w, b, 1e-5, want_stats=True)
+    xd = x.double()
+    mu = xd.mean(-1)
+    var = ((xd - mu[:, None]) ** 2).mean(-1)
+    ref = (xd - mu[:, None]) / torch.sqrt(var[:, None] + 1e-5) * w.double() + b.double()
+    assert torch.allclose(mean.double(), mu, atol=1e-5, rtol=1e-5)
+    assert torch.allclose(rstd.double(), 1 / torch.sqrt(var + 1e-5), atol=1e-5, rtol=1e-5)
+    if dtype is torch.float32:
+        lib_ref = F.layer_norm(x, (d,), w, b, 1e-5)
+        assert torch.allclose(y, lib_ref, atol=1e-5, rtol=1e-5)
+        assert torch.allclose(y.double(), ref, atol=1e-5, rtol=1e-5)
+    else:
+        err = (y.double() - ref).abs().max().item()
+        assert err <= EPS16[dtype] * (ref.abs().max().item() + 1.0), err
+        # exactly the fp32 formula rounded once
+        assert (y.double() - ref.to(dtype).double()).abs().max().item() <= 2 * EPS16[dtype] * ref.abs().max().item()
+
+
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,d", [(513, 128), (100, 192), (31, 384)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_ln_fwd_add(dtype, rows, d, with_bias):
+    a = _rand(rows, d, dtype=dtype, seed=3)
+    b = _rand(rows, d, dtype=dtype, seed=4)
+    bb = _rand(d, seed=5) if with_bias else None
+    w = _rand(d, seed=1) * 0.3 + 1.0
+    bias = _rand(d, seed=2) * 0.3
+    x, y = ops.ln_fwd_add(a, b, w, bias, 1e-5, b_bias=bb)
+    # x bitwise: a + b in fp32, or round(a + (b + bias)) from fp32 arithmetic
+    bf = b.float() if bb is None else b.float() + bb
+    x_ref = (a.float() + bf).to(dtype)
+    assert torch.equal(x, x_ref)
+    y_ref = F.layer_norm(x.float(), (d,), w, bias, 1e-5)
+    tol = 1e-5 if dtype is torch.float32 else 2 * EPS16[dtype] * (y_ref.abs().max().item() + 1)
+    assert (y.float() - y_ref).abs().max().item() <= tol
+    # the plain kernel on the rounded x gives the same bits
+    assert torch.equal(ops.ln_fwd(x, w, bias, 1e-5), y)
+
+
+# ---------------------------------------------------------------- Linear
+def _lin_ref(x, w, bias, act, res):
+    y = x.double() @ w.double().t()
+    if bias is not None:
+        y = y + bias.double()
+    if act == "relu":
+        y = torch.relu(y)
+    elif act == "gelu":
+        y = 0.5 * y * (1 + torch.erf(y / math.sqrt(2.0)))
+    if res is not None:
+        y = y + res.double()
+    return y
+
+
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,K,M", [(1, 128, 128), (127, 128, 384), (129, 128, 512), (1000, 512, 128),
+                                      (300, 192, 576), (64, 768, 192), (50, 49, 192), (77, 40, 192),
+                                      (33, 128, 204), (65, 384, 145), (19, 640, 101), (256, 100, 128),
+                                      (200, 16, 128), (130, 1536, 384)])
+def test_linear_shapes(dtype, rows, K, M):
+    x = _rand(rows, K, dtype=dtype, seed=rows)
+    w = _rand(M, K, dtype=dtype, seed=K, scale=1 / math.sqrt(K))
+    b = _rand(M, seed=M)
+    y = ops.linear(x, w, b)
+    ref = _lin_ref(x, w, b, None, None)
+    scale = ref.abs().max().item()
+    tol = 1e-5 * scale if dtype is torch.float32 else 1.2 * EPS16[dtype] * scale
+    assert y.shape == (rows, M) and y.dtype is dtype
+    assert (y.double() - ref).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("act", [None, "relu", "gelu"])
+@pytest.mark.parametrize("use_res", [False, True])
+def test_linear_epilogues(dtype, act, use_res):
+    rows, K, M = 333, 128, 256
+    x = _rand(rows, K, dtype=dtype, seed=1)
+    w = _rand(M, K, dtype=dtype, seed=2, scale=0.1)
+    b = _rand(M, seed=3)
+    res = _rand(rows, M, dtype=dtype, seed=4) if use_res else None
+    ref = _lin_ref(x, w, b, act, res)
+    scale = ref.abs().max().item()
+    for out_dtype in (dtype, torch.float32):
+        y = ops.linear(x, w, b, act=act, residual=res, out_dtype=out_dtype)
+        tol = 2e-5 * scale if out_dtype is torch.float32 and dtype is torch.float32 else (
+            1e-4 * scale if out_dtype is torch.float32 else 1.2 * EPS16[dtype] * scale)
+        assert y.dtype is out_dtype
+        assert (y.double() - ref).abs().max().item() <= tol, (dtype, act, use_res, out_dtype)
+
+
+@pytest.mark.parametrize("dtype", DTS)
+def test_linear_strided_views_split_and_packing(dtype):
+    """x as a row-strided view (token 0 of every env), split output, and the
+    packed q|k|v GEMM == three separate Linears (column-block identity)."""
+    B, T, d = 37, 16, 128
+    tok = _rand(B, T, d, dtype=dtype, seed=7)
+    w = _rand(204, d, dtype=dtype, seed=8, scale=0.1)
+    b = _rand(204, seed=9)
+    lg, val = ops.linear(tok[:, 0], w, b, out_dtype=torch.float32, split=203)
+    ref = _lin_ref(tok[:, 0], w, b, None, None)
+    assert lg.shape == (B, 203) and val.shape == (B, 1)
+    assert (torch.cat([lg, val], 1).double() - ref).abs().max().item() <= 1e-4 * ref.abs().max().item()
+    ws = [_rand(d, d, dtype=dtype, seed=20 + i, scale=0.1) for i in range(3)]
+    bs = [_rand(d, seed=30 + i) for i in range(3)]
+    packed = ops.linear(tok, torch.cat(ws).contiguous(), torch.cat(bs).contiguous())
+    assert packed.shape == (B, T, 3 * d)
+    for i in range(3):
+        assert torch.equal(packed[..., i * d:(i + 1) * d], ops.linear(tok, ws[i], bs[i]))
+
+
+def test_linear_rows_are_batch_invariant():
+    """A row's bits do not depend on the batch it sits in or on its tile phase
+    (the reference holds its kernels to this: tests/test_fused_ffn.py:332-353)."""
+    x = _rand(600, 128, dtype=torch.float16, seed=1)
+    w = _rand(384, 128, dtype=torch.float16, seed=2, scale=0.1)
+    b = _rand(384, seed=3)
+    full = ops.linear(x, w, b, act="gelu")
+    for lo, hi in ((0, 1), (5, 132), (127, 256), (300, 600)):
+        assert torch.equal(ops.linear(x[lo:hi], w, b, act="gelu"), full[lo:hi])
+
+
+# ---------------------------------------------------------------- Attention
+def _attn_ref(q, k, v, H, bias):
+    B, TQ, d = q.shape
+    T = k.shape[1]
+    dh = d // H
+    qh = q.double().view(B, TQ, H, dh).transpose(1, 2)
+    kh = k.double().view(B, T, H, dh).transpose(1, 2)
+    vh = v.double().view(B, T, H, dh).transpose(1, 2)
+    s = qh @ kh.transpose(-2, -1) / math.sqrt(dh)
+    if bias is not None:
+        s = s + bias.double().view(B, 1, 1, T)
+    return (torch.softmax(s, -1) @ vh).transpose(1, 2).reshape(B, TQ, d)
+
+
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("T,TQ,H,dh", [(16, 16, 4, 32), (29, 29, 4, 48), (29, 5, 4, 48), (29, 1, 4, 48),
+                                       (32, 32, 8, 32), (48, 48, 12, 32), (48, 1, 12, 32), (6, 6, 2, 32),
+                                       (17, 3, 4, 32)])
+@pytest.mark.parametrize("mask", ["none", "n_valid", "bias"])
+def test_attention(dtype, T, TQ, H, dh, mask):
+    B, d = 11, H * dh
+    qkv = _rand(B, T, 3 * d, dtype=dtype, seed=T + TQ)
+    q, k, v = qkv[:, :TQ, :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+    g = torch.Generator().manual_seed(5)
+    nv = torch.randint(0, T, (B,), generator=g, dtype=torch.int32)
+    nv[0] = 0
+    nv[1] = T - 1
+    valid = (torch.arange(T)[None, :] <= nv[:, None]).float()
+    bias = ((valid - 1.0) * 16384.0).to(dtype).to(DEV)
+    nvd = nv.to(DEV)
+    if mask == "none":
+        out = ops.attn_fwd(q, k, v, H)
+        ref = _attn_ref(q, k, v, H, None)
+    elif mask == "n_valid":
+        out = ops.attn_fwd(q, k, v, H, n_valid=nvd)
+        ref = _attn_ref(q, k, v, H, bias)
+    else:
+        out = ops.attn_fwd(q, k, v, H, key_bias=bias)
+        ref = _attn_ref(q, k, v, H, bias)
+    assert out.shape == (B, TQ, d) and out.is_contiguous()
+    tol = 2e-5 if dtype is torch.float32 else 3 * EPS16[dtype] * (ref.abs().max().item() + 1)
+    assert (out.double() - ref).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_attention_invariants(dtype):
+    B, T, H, dh = 9, 29, 4, 48
+    d = H * dh
+    q = _rand(B, T, d, dtype=dtype, seed=1)
+    k = _rand(B, T, d, dtype=dtype, seed=2)
+    v = _rand(B, T, d, dtype=dtype, seed=3)
+    nv = torch.tensor([0, 4, 28, 10, 5, 17, 1, 2, 3], dtype=torch.int32, device=DEV)
+    out = ops.attn_fwd(q, k, v, H, n_valid=nv)
+    # masked keys get exactly zero weight: junk in masked V/K rows changes nothing
+    k2, v2 = k.clone(), v.clone()
+    for b in range(B):
+        v2[b, int(nv[b]) + 1:] = 1000.0
+        k2[b, int(nv[b]) + 1:] = 50.0
+    assert torch.equal(ops.attn_fwd(q, k2, v2, H, n_valid=nv), out)
+    # batch-slice invariance
+    assert torch.equal(ops.attn_fwd(q[2:5], k[2:5], v[2:5], H, n_valid=nv[2:5].contiguous()), out[2:5])
+    # TQ < T == row slice of the full result (masking is key-side only)
+    for tq in (5, 1):
+        assert torch.equal(ops.attn_fwd(q[:, :tq], k, v, H, n_valid=nv), out[:, :tq])
+
+
+# ---------------------------------------------------------------- Tokenizer
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("T,d", [(16, 128), (32, 256), (48, 384), (6, 32)])
+def test_cfg_embed(dtype, T, d):
+    from oracle import config_model as cm
+    spec = cm.ConfigSpec(1, d, d // 32 if d >= 32 else 1, 4 * d, T)
+    p = cm.init_params(spec, 3)
+    B = 13
+    obs, _ = cm.make_inputs(spec, B, 4)
+    em = {torch.float32: None, torch.float16: "f16", torch.bfloat16: "bf16"}[dtype]
+    ref = cm.tokens_from_obs(p, spec, obs, emulate=em)
+    tok = ops.cfg_embed(obs.to(DEV), p["prop_embed.weight"].to(dtype).to(DEV), p["prop_embed.bias"].to(DEV),
+                        p["obj_embed.weight"].to(dtype).to(DEV), p["obj_embed.bias"].to(DEV), T, dtype)
+    assert tok.shape == (B, T, d)
+    tol = 1e-5 if dtype is torch.float32 else 1.2 * EPS16[dtype] * (ref.abs().max().item() + 1)
+    assert (tok.float().cpu() - ref).abs().max().item() <= tol
