@@ -116,13 +116,19 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnArgs a) {
         float m = -INFINITY;
 #pragma unroll
         for (int kt = 0; kt < kMaxKT; ++kt) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            // The K = 32 and K = 16 products go to SEPARATE accumulators and are summed on the
+            // VALU: chaining a 16x16x16 MFMA onto the accumulator of a 16x16x32 one lost the
+            // first product on gfx950 (measured), same-shape chains are fine.
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
             if (kt < nkt) {
                 acc = DT::mfma32(kf[kt], qf, acc);
-                if (DH == 48) acc = DT::mfma16(kf2[kt], qf2, acc);
+                if (DH == 48) acc2 = DT::mfma16(kf2[kt], qf2, acc2);
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { s[kt][i] = acc[i] * a.scale + kb[kt][i]; m = fmaxf(m, s[kt][i]); }
+            for (int i = 0; i < 4; ++i) {
+                s[kt][i] = (acc[i] + acc2[i]) * a.scale + kb[kt][i];
+                m = fmaxf(m, s[kt][i]);
+            }
         }
         m = fmaxf(m, __shfl_xor(m, 16, WAVE));
         m = fmaxf(m, __shfl_xor(m, 32, WAVE));
