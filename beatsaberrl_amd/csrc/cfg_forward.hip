@@ -1,6 +1,586 @@
-// Whole-forward persistent kernel (placeholder until the kernel lands).
+// Whole config-model policy forward in ONE persistent kernel for gfx950.
+//
+// Shape class: T = 16 tokens per env, d = 128, 4 heads x 32, FFN multiple of 32,
+// any number of layers, fp16 or bf16 operands with fp32 accumulate.
+//
+// Mapping.  One 16-row MFMA tile == one env (its 16 tokens).  A wave64 owns RT
+// envs and carries their fp32 residual stream in registers for the whole
+// forward (RT x 8 feature tiles x 4 VGPRs); LayerNorm, the QKV projection,
+// attention (one 16x16x32 MFMA per head for the scores, softmax by two
+// cross-lane butterflies, 16x16x16 MFMAs for P.V), the output projection, the
+// FFN with its hidden kept in registers, and the 29x7 + 1 output projection
+// all run wave-locally: activations never touch LDS or HBM.  The activation is
+// always the MFMA operand whose free index is the TOKEN, so a GEMM's output
+// fragment (4 consecutive features per lane) packs straight into the next
+// GEMM's input fragment; the k order this implies (features 4g..4g+3 then
+// 16+4g..16+4g+3 of each 32-chunk for lane group g) is baked into the weight
+// image by bsrl_cfg_pack, so a weight fragment is one 16-byte LDS read per lane.
+// The V projection swaps operand roles and so lands already transposed for P.V.
+//
+// Weights (~0.85 MB at 2 layers) stream from L2 through a 2-slot LDS ring in
+// 8 KB stages (8 fragments) shared by the workgroup's 4 waves: global loads are
+// issued three stages ahead into registers, written to LDS one stage ahead,
+// one barrier per stage.  HBM traffic is the obs in and the logits out.
+//
+// Replaces NotePolicy.forward_stacked (python/policy.py:1179-1344) for the
+// benchmark-config model; the weight image is the analogue of the reference's
+// flat fp16 replica buffer (python/fp16_linear.py:249-346).
 #include "bsrl_common.h"
-extern "C" int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc*) { return 0; }
-extern "C" int bsrl_cfg_pack(const bsrl_cfg_desc*, const bsrl_cfg_params*, void*, bsrl_stream) { return BSRL_UNSUPPORTED; }
-extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc*, const void*, const void*, int64_t, int, const int32_t*, float*,
-                                float*, int64_t, bsrl_stream) { return BSRL_UNSUPPORTED; }
+
+namespace {
+
+constexpr int D = 128;            // model width
+constexpr int NT = D / 16;        // feature tiles
+constexpr int KC = D / 32;        // 32-wide k chunks
+constexpr int H = 4;              // heads (dh = 32)
+constexpr int T = 16;             // tokens per env == MFMA tile rows
+constexpr int STAGE_FRAGS = 8;
+constexpr int STAGE_U4 = STAGE_FRAGS * 64;       // uint4 per stage (8 KB)
+constexpr int EMB_STAGES = NT / 2;               // 4
+constexpr int HEAD_TILES = 16;                   // 204 outputs padded to 256
+constexpr int HEAD_STAGES = HEAD_TILES * KC / STAGE_FRAGS;   // 8
+
+__host__ __device__ constexpr int layer_stages(int F) { return 3 * H + NT * KC / STAGE_FRAGS + 2 * (F / 32); }
+__host__ __device__ constexpr int total_stages(int L, int F) { return EMB_STAGES + L * layer_stages(F) + HEAD_STAGES; }
+// fp32 vector region (floats)
+constexpr int V_BP = 0, V_BO = D, V_LAYER0 = 2 * D;
+constexpr int LV_LN1G = 0, LV_LN1B = D, LV_BQ = 2 * D, LV_BK = 3 * D, LV_BV = 4 * D, LV_BOUT = 5 * D,
+              LV_LN2G = 6 * D, LV_LN2B = 7 * D, LV_B1 = 8 * D;
+__host__ __device__ constexpr int lv_b2(int F) { return 8 * D + F; }
+__host__ __device__ constexpr int lv_size(int F) { return 9 * D + F; }
+constexpr int FV_LNG = 0, FV_LNB = D, FV_BH = 2 * D, FV_SIZE = 2 * D + HEAD_TILES * 16;
+__host__ __device__ constexpr int vec_floats(int L, int F) { return V_LAYER0 + L * lv_size(F) + FV_SIZE; }
+
+struct FwdArgs {
+    const uint4* frags; const float* vec;
+    const void* obs; int64_t obs_ld; int obs_f32;
+    const int32_t* n_valid;
+    float* logits; float* value;
+    int64_t B; int n_layers, F, n_stages, n_logits, final_ln, prop_dim, obj_dim;
+};
+
+// ---- helpers -------------------------------------------------------------------
+template <typename DT> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    return (uint32_t)DT::from_f(a) | ((uint32_t)DT::from_f(b) << 16);
+}
+template <> __device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
+union Frag4 { s16x4 v; uint32_t w[2]; };
+
+// exact-erf GELU to ~2e-7 (Abramowitz-Stegun 7.1.26), 2 transcendentals
+__device__ __forceinline__ float gelu_fast(float x) {
+    const float z = fabsf(x) * 0.70710678118654752440f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(t, 1.061405429f, -1.453152027f);
+    p = fmaf(t, p, 1.421413741f);
+    p = fmaf(t, p, -0.284496736f);
+    p = fmaf(t, p, 0.254829592f);
+    p *= t;
+    const float e = __expf(-z * z);
+    const float erfa = fmaf(-p, e, 1.0f);
+    const float hx = 0.5f * x;
+    return fmaf(hx, copysignf(erfa, x), hx);
+}
+template <int ACT> __device__ __forceinline__ float act_fast(float x) {
+    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.f);
+    if (ACT == BSRL_ACT_GELU) return gelu_fast(x);
+    return x;
+}
+
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were
+// issued 3 stage-steps earlier into register set s & 1.
+struct Pipe {
+    uint4 r[2][2];
+    const uint4* img;
+    int next, n;
+};
+
+template <int P>   // P = parity of the stage about to be consumed
+__device__ __forceinline__ void advance(Pipe& p, uint4 (*lds)[STAGE_U4], int tid) {
+    lds_barrier();                                   // stage s is complete in slot P; slot 1-P is free
+    lds[1 - P][tid] = p.r[1 - P][0];                 // stage s+1 -> slot 1-P
+    lds[1 - P][tid + 256] = p.r[1 - P][1];
+    const uint4* src = p.img + (int64_t)p.next * STAGE_U4 + tid;   // stage s+3 -> the freed registers
+    p.r[1 - P][0] = src[0];
+    p.r[1 - P][1] = src[256];
+    p.next = p.next + 1 == p.n ? 0 : p.next + 1;
+}
+#define ADVANCE(par) do { if (par) advance<1>(pipe, lds, tid); else advance<0>(pipe, lds, tid); } while (0)
+#define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[par][(f) * 64 + lane]))
+
+template <typename DT, int RT, int ACT>
+__global__ __launch_bounds__(256) void cfg_forward_kernel(FwdArgs a) {
+    __shared__ uint4 lds[2][STAGE_U4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const float scale = 0.17677669529663688110f;      // 1 / sqrt(32)
+    const int64_t ntiles = (a.B + 4 * RT - 1) / (4 * RT);
+
+    Pipe pipe;
+    pipe.img = a.frags; pipe.n = a.n_stages;
+    {   // prologue: stage 0 -> LDS slot 0; stages 1, 2 in flight
+        uint4 s0a = pipe.img[tid], s0b = pipe.img[tid + 256];
+        pipe.r[1][0] = pipe.img[STAGE_U4 + tid]; pipe.r[1][1] = pipe.img[STAGE_U4 + tid + 256];
+        lds[0][tid] = s0a; lds[0][tid + 256] = s0b;
+        pipe.r[0][0] = pipe.img[2 * STAGE_U4 + tid]; pipe.r[0][1] = pipe.img[2 * STAGE_U4 + tid + 256];
+        pipe.next = 3 % pipe.n;
+    }
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t env0 = tile * (4 * RT) + wave * RT;
+        int nv[RT];
+        f32x4 x[RT][NT];
+        // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
+        {
+            Frag8 e[RT][KC];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
+                nv[rt] = a.n_valid ? a.n_valid[env] : T - 1;
+                float ev[KC][8];
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int k = 32 * c + 4 * g + (j & 3) + (j >> 2) * 16;    // permuted k order
+                        int idx; bool on;
+                        if (k < 16) { on = r16 >= 1 && k < a.obj_dim; idx = a.prop_dim + (r16 - 1) * a.obj_dim + k; }
+                        else { on = r16 == 0 && (k - 16) < a.prop_dim; idx = k - 16; }
+                        float v = 0.f;
+                        if (on) {
+                            const int64_t off = env * a.obs_ld + idx;
+                            v = a.obs_f32 ? static_cast<const float*>(a.obs)[off] : DT::to_f(static_cast<const u16*>(a.obs)[off]);
+                        }
+                        ev[c][j] = v;
+                    }
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) e[rt][c].w[w] = pack2<DT>(ev[c][2 * w], ev[c][2 * w + 1]);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 bp = *reinterpret_cast<const float4*>(a.vec + V_BP + 16 * nt + 4 * g);
+                const float4 bo = *reinterpret_cast<const float4*>(a.vec + V_BO + 16 * nt + 4 * g);
+                const float4 b = r16 == 0 ? bp : bo;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) x[rt][nt] = (f32x4){b.x, b.y, b.z, b.w};
+            }
+#pragma unroll
+            for (int st = 0; st < EMB_STAGES; ++st) {
+                ADVANCE(st & 1);
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        const s16x8 w = WFRAG(st & 1, ntl * KC + c);
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(w, e[rt][c].v, x[rt][2 * st + ntl]);
+                    }
+            }
+        }
+        // ================= transformer blocks =================
+        for (int l = 0; l < a.n_layers; ++l) {
+            const float* lv = a.vec + V_LAYER0 + l * lv_size(a.F);
+            Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
+            // ---- LN1 ----
+            auto layer_norm = [&](int goff, int boff) {
+                float4 gm[NT], bt[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    gm[nt] = *reinterpret_cast<const float4*>(lv + goff + 16 * nt + 4 * g);
+                    bt[nt] = *reinterpret_cast<const float4*>(lv + boff + 16 * nt + 4 * g);
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
+                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
+                    const float mean = s * (1.0f / D);
+                    float q = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
+                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
+                    const float rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
+                        const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
+                        const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
+                        const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
+                        hf[rt][nt >> 1].w[(nt & 1) * 2] = pack2<DT>(y0, y1);
+                        hf[rt][nt >> 1].w[(nt & 1) * 2 + 1] = pack2<DT>(y2, y3);
+                    }
+                }
+            };
+            layer_norm(LV_LN1G, LV_LN1B);
+
+            // ---- QKV + attention, head by head ----
+            Frag8 of[RT][KC];       // attention output fragments (chunk == head)
+#pragma unroll
+            for (int hd = 0; hd < H; ++hd) {
+                Frag8 qf[RT], kf[RT];
+                Frag4 vt[RT][2];
+#pragma unroll
+                for (int part = 0; part < 3; ++part) {
+                    const int par = (hd * 3 + part) & 1;        // stage parity inside the layer (layer starts even)
+                    ADVANCE(par);
+                    f32x4 acc[2][RT];
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? LV_BQ : LV_BK) + 32 * hd + 16 * ntl + 4 * g);
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
+                    }
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) {
+                            const s16x8 w = WFRAG(par, ntl * KC + c);
+#pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) {
+                                if (part < 2) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
+                                else acc[ntl][rt] = DT::mfma32(hf[rt][c].v, w, acc[ntl][rt]);   // V^T: roles swapped
+                            }
+                        }
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) {
+                            const uint32_t lo = pack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]);
+                            const uint32_t hi = pack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
+                            if (part == 0) { qf[rt].w[ntl * 2] = lo; qf[rt].w[ntl * 2 + 1] = hi; }
+                            else if (part == 1) { kf[rt].w[ntl * 2] = lo; kf[rt].w[ntl * 2 + 1] = hi; }
+                            else { vt[rt][ntl].w[0] = lo; vt[rt][ntl].w[1] = hi; }
+                        }
+                }
+                // scores^T = K Q^T (lane: query r16, keys 4g..4g+3), softmax over keys, O = P V (+ b_v)
+                const float4 bv0 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 4 * g);
+                const float4 bv1 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 16 + 4 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    f32x4 s = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                    float sv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sv[i] = (4 * g + i) <= nv[rt] ? s[i] * scale : -INFINITY;
+                    float m = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+                    m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
+                    float sum = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[i] = __expf(sv[i] - m); sum += sv[i]; }
+                    sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
+                    const float inv = __builtin_amdgcn_rcpf(sum);
+                    Frag4 pf;
+                    pf.w[0] = pack2<DT>(sv[0] * inv, sv[1] * inv);
+                    pf.w[1] = pack2<DT>(sv[2] * inv, sv[3] * inv);
+                    const f32x4 o0 = DT::mfma16(vt[rt][0].v, pf.v, (f32x4){bv0.x, bv0.y, bv0.z, bv0.w});
+                    const f32x4 o1 = DT::mfma16(vt[rt][1].v, pf.v, (f32x4){bv1.x, bv1.y, bv1.z, bv1.w});
+                    of[rt][hd].w[0] = pack2<DT>(o0[0], o0[1]); of[rt][hd].w[1] = pack2<DT>(o0[2], o0[3]);
+                    of[rt][hd].w[2] = pack2<DT>(o1[0], o1[1]); of[rt][hd].w[3] = pack2<DT>(o1[2], o1[3]);
+                }
+            }
+            // ---- output projection, accumulated onto the residual ----
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 b = *reinterpret_cast<const float4*>(lv + LV_BOUT + 16 * nt + 4 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) { x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w; }
+            }
+#pragma unroll
+            for (int st = 0; st < NT / 2; ++st) {
+                ADVANCE(st & 1);            // 12 stages precede: parity restarts even
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        const s16x8 w = WFRAG(st & 1, ntl * KC + c);
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(w, of[rt][c].v, x[rt][2 * st + ntl]);
+                    }
+            }
+            // ---- LN2 + FFN (hidden stays in registers, 32 hidden units per step) ----
+            layer_norm(LV_LN2G, LV_LN2B);
+            const int b2off = lv_b2(a.F);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 b = *reinterpret_cast<const float4*>(lv + b2off + 16 * nt + 4 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) { x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w; }
+            }
+            for (int ch = 0; ch < a.F / 32; ++ch) {
+                ADVANCE(0);
+                f32x4 acc[2][RT];
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const float4 b = *reinterpret_cast<const float4*>(lv + LV_B1 + 32 * ch + 16 * ntl + 4 * g);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
+                }
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        const s16x8 w = WFRAG(0, ntl * KC + c);
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
+                    }
+                Frag8 hid[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        hid[rt].w[ntl * 2] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][0]), act_fast<ACT>(acc[ntl][rt][1]));
+                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][2]), act_fast<ACT>(acc[ntl][rt][3]));
+                    }
+                ADVANCE(1);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const s16x8 w = WFRAG(1, nt);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w, hid[rt].v, x[rt][nt]);
+                }
+            }
+        }
+        // ================= readout: token 0 of every env -> 29*K logits + value =================
+        {
+            float4 gm[NT], bt[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                gm[nt] = make_float4(1.f, 1.f, 1.f, 1.f); bt[nt] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            const float* fv = a.vec + V_LAYER0 + a.n_layers * lv_size(a.F);
+            if (a.final_ln) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    gm[nt] = *reinterpret_cast<const float4*>(fv + FV_LNG + 16 * nt + 4 * g);
+                    bt[nt] = *reinterpret_cast<const float4*>(fv + FV_LNB + 16 * nt + 4 * g);
+                }
+            }
+            Frag8 rf[KC];           // B operand: lane (env r16 < RT, group g)
+#pragma unroll
+            for (int c = 0; c < KC; ++c) rf[c].u = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                float mean = 0.f, rstd = 1.f;
+                if (a.final_ln) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
+                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
+                    mean = s * (1.0f / D);
+                    float q = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
+                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
+                    rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
+                    const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
+                    const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
+                    const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
+                    // row 0 of this env's tile sits in lanes 16*g; hand it to lane (r16 == rt, g)
+                    const uint32_t lo = __shfl(pack2<DT>(y0, y1), 16 * g, WAVE);
+                    const uint32_t hi = __shfl(pack2<DT>(y2, y3), 16 * g, WAVE);
+                    if (r16 == rt) { rf[nt >> 1].w[(nt & 1) * 2] = lo; rf[nt >> 1].w[(nt & 1) * 2 + 1] = hi; }
+                }
+            }
+            const int64_t env = env0 + r16;
+            const bool store = r16 < RT && env < a.B;
+#pragma unroll
+            for (int st = 0; st < HEAD_STAGES; ++st) {
+                ADVANCE(st & 1);            // an even number of stages precedes the readout
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int nt = 2 * st + ntl;
+                    const float4 b = *reinterpret_cast<const float4*>(fv + FV_BH + 16 * nt + 4 * g);
+                    f32x4 acc = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int c = 0; c < KC; ++c) acc = DT::mfma32(WFRAG(st & 1, ntl * KC + c), rf[c].v, acc);
+                    if (store) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int col = 16 * nt + 4 * g + i;
+                            if (col < a.n_logits) a.logits[env * a.n_logits + col] = acc[i];
+                            else if (col == a.n_logits) a.value[env] = acc[i];
+                        }
+                    }
+                }
+            }
+        }
+    }
+    lds_barrier();   // every wave leaves together; no LDS slot is read after this point
+}
+
+// ---- weight image ------------------------------------------------------------------
+struct PackArgs {
+    bsrl_cfg_params p;
+    void* frags; float* vec;
+    int n_layers, F, n_stages, n_out, prop_dim, obj_dim, final_ln;
+};
+
+__device__ __forceinline__ int perm_k(int c, int gg, int j) { return 32 * c + 4 * gg + (j & 3) + (j >> 2) * 16; }
+
+// one wave per fragment, one lane per 16-byte slot
+template <typename DT>
+__global__ __launch_bounds__(256) void cfg_pack_frags_kernel(PackArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= a.n_stages * STAGE_FRAGS) return;
+    const int n16 = lane & 15, gg = lane >> 4;
+    const int lstages = layer_stages(a.F);
+    const int emb_end = EMB_STAGES * STAGE_FRAGS;
+    const int layers_end = emb_end + a.n_layers * lstages * STAGE_FRAGS;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = 0.f;
+    if (f < emb_end) {
+        const int st = f / 8, r = f % 8, nt = 2 * st + r / KC, c = r % KC, n = 16 * nt + n16;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = perm_k(c, gg, j);
+            if (k < 16) { if (k < a.obj_dim) v[j] = a.p.obj_w[n * a.obj_dim + k]; }
+            else if (k - 16 < a.prop_dim) v[j] = a.p.prop_w[n * a.prop_dim + (k - 16)];
+        }
+    } else if (f < layers_end) {
+        const int l = (f - emb_end) / (lstages * 8), r = (f - emb_end) % (lstages * 8);
+        const float* src; int ld, n, kbase = 0, c;
+        if (r < 3 * H * 8) {
+            const int hd = r / 24, rr = r % 24, part = rr / 8, q = rr % 8;
+            src = part == 0 ? a.p.blk[l].q_w : part == 1 ? a.p.blk[l].k_w : a.p.blk[l].v_w;
+            ld = D; n = 32 * hd + 16 * (q / KC) + n16; c = q % KC;
+        } else if (r < 3 * H * 8 + NT * KC) {
+            const int r2 = r - 3 * H * 8;
+            src = a.p.blk[l].out_w; ld = D; n = 16 * (r2 / KC) + n16; c = r2 % KC;
+        } else {
+            const int r3 = r - 3 * H * 8 - NT * KC, ch = r3 / 16, q = r3 % 16;
+            if (q < 8) { src = a.p.blk[l].ffn0_w; ld = D; n = 32 * ch + 16 * (q / KC) + n16; c = q % KC; }
+            else { src = a.p.blk[l].ffn2_w; ld = a.F; n = 16 * (q - 8) + n16; c = 0; kbase = 32 * ch; }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + perm_k(c, gg, j)];
+    } else {
+        const int r = f - layers_end, n = 16 * (r / KC) + n16, c = r % KC;
+        if (n < a.n_out) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = a.p.heads_w[n * D + perm_k(c, gg, j)];
+        }
+    }
+    uint4 o;
+    o.x = pack2<DT>(v[0], v[1]); o.y = pack2<DT>(v[2], v[3]); o.z = pack2<DT>(v[4], v[5]); o.w = pack2<DT>(v[6], v[7]);
+    static_cast<uint4*>(a.frags)[(int64_t)f * 64 + lane] = o;
+}
+
+__global__ __launch_bounds__(256) void cfg_pack_vec_kernel(PackArgs a) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int total = vec_floats(a.n_layers, a.F);
+    if (i >= total) return;
+    float v = 0.f;
+    if (i < V_LAYER0) v = i < V_BO ? a.p.prop_b[i] : a.p.obj_b[i - V_BO];
+    else if (i < V_LAYER0 + a.n_layers * lv_size(a.F)) {
+        const int l = (i - V_LAYER0) / lv_size(a.F), r = (i - V_LAYER0) % lv_size(a.F);
+        const auto& b = a.p.blk[l];
+        if (r < LV_B1) {
+            const float* srcs[8] = {b.ln_attn_w, b.ln_attn_b, b.q_b, b.k_b, b.v_b, b.out_b, b.ln_ffn_w, b.ln_ffn_b};
+            v = srcs[r / D][r % D];
+        } else if (r < lv_b2(a.F)) v = b.ffn0_b[r - LV_B1];
+        else v = b.ffn2_b[r - lv_b2(a.F)];
+    } else {
+        const int r = i - V_LAYER0 - a.n_layers * lv_size(a.F);
+        if (r < FV_LNB) v = a.final_ln ? a.p.final_ln_w[r] : 1.f;
+        else if (r < FV_BH) v = a.final_ln ? a.p.final_ln_b[r - FV_LNB] : 0.f;
+        else v = (r - FV_BH) < a.n_out ? a.p.heads_b[r - FV_BH] : 0.f;
+    }
+    a.vec[i] = v;
+}
+
+bool shape_ok(const bsrl_cfg_desc* d) {
+    return d && d->d == D && d->n_heads == H && d->T == T && d->ffn > 0 && d->ffn % 32 == 0 && d->ffn <= 4096 &&
+           d->n_layers >= 1 && d->n_layers <= BSRL_MAX_LAYERS && (d->dtype == BSRL_F16 || d->dtype == BSRL_BF16) &&
+           d->obj_dim >= 1 && d->obj_dim <= 16 && d->prop_dim >= 1 && d->prop_dim <= D - 16 &&
+           d->n_gears >= 1 && 29 * d->n_gears + 1 <= HEAD_TILES * 16 && (d->act == BSRL_ACT_GELU || d->act == BSRL_ACT_RELU);
+}
+int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
+
+template <typename DT, int RT>
+void launch_fwd(const FwdArgs& a, int act, unsigned grid, hipStream_t st) {
+    if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((cfg_forward_kernel<DT, RT, BSRL_ACT_GELU>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((cfg_forward_kernel<DT, RT, BSRL_ACT_RELU>), dim3(grid), dim3(256), 0, st, a);
+}
+
+}  // namespace
+
+extern "C" int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* d) {
+    if (!shape_ok(d)) return 0;
+    return frag_bytes(d) + (int64_t)vec_floats(d->n_layers, d->ffn) * 4;
+}
+
+extern "C" int bsrl_cfg_pack(const bsrl_cfg_desc* d, const bsrl_cfg_params* p, void* packed, bsrl_stream stream) {
+    if (!d || !p || !packed) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_pack: null pointer");
+    if (!shape_ok(d)) return BSRL_UNSUPPORTED;
+    if (!bsrl_aligned(packed, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_pack: image must be 16-byte aligned");
+    if (!p->prop_w || !p->prop_b || !p->obj_w || !p->obj_b || !p->heads_w || !p->heads_b ||
+        (d->final_ln && (!p->final_ln_w || !p->final_ln_b)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_pack: null parameter pointer");
+    for (int l = 0; l < d->n_layers; ++l) {
+        const float* const* q = reinterpret_cast<const float* const*>(&p->blk[l]);
+        for (int i = 0; i < 16; ++i) if (!q[i]) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_pack: null parameter pointer in block %d", l);
+    }
+    PackArgs a;
+    a.p = *p;
+    a.frags = packed;
+    a.vec = reinterpret_cast<float*>(static_cast<char*>(packed) + frag_bytes(d));
+    a.n_layers = d->n_layers; a.F = d->ffn; a.n_stages = total_stages(d->n_layers, d->ffn);
+    a.n_out = 29 * d->n_gears + 1; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim; a.final_ln = d->final_ln;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const unsigned nf = (unsigned)(a.n_stages * STAGE_FRAGS);
+    if (d->dtype == BSRL_F16) hipLaunchKernelGGL((cfg_pack_frags_kernel<F16>), dim3((nf + 3) / 4), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((cfg_pack_frags_kernel<BF16>), dim3((nf + 3) / 4), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(cfg_pack_vec_kernel, dim3((vec_floats(a.n_layers, a.F) + 255) / 256), dim3(256), 0, st, a);
+    BSRL_CHECK_LAUNCH("bsrl_cfg_pack");
+    return BSRL_OK;
+}
+
+extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
+                                int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
+                                bsrl_stream stream) {
+    if (!d || !packed || !obs || !logits || !value) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: null pointer");
+    if (!shape_ok(d)) return BSRL_UNSUPPORTED;
+    if (B < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: negative batch");
+    if (obs_dtype != BSRL_F32 && obs_dtype != d->dtype) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: obs must be F32 or the stream dtype");
+    if (obs_ld < d->prop_dim + (d->T - 1) * d->obj_dim) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: obs_ld smaller than an obs row");
+    if (!bsrl_aligned(packed, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: image must be 16-byte aligned");
+    if (B == 0) return BSRL_OK;
+    FwdArgs a;
+    a.frags = static_cast<const uint4*>(packed);
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(packed) + frag_bytes(d));
+    a.obs = obs; a.obs_ld = obs_ld; a.obs_f32 = obs_dtype == BSRL_F32;
+    a.n_valid = n_valid; a.logits = logits; a.value = value; a.B = B;
+    a.n_layers = d->n_layers; a.F = d->ffn; a.n_stages = total_stages(d->n_layers, d->ffn);
+    a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    constexpr int RT = 4;
+    const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
+    const unsigned grid = (unsigned)(ntiles < cus ? ntiles : cus);
+    if (d->dtype == BSRL_F16) launch_fwd<F16, RT>(a, d->act, grid, st);
+    else launch_fwd<BF16, RT>(a, d->act, grid, st);
+    BSRL_CHECK_LAUNCH("bsrl_cfg_forward");
+    return BSRL_OK;
+}
