@@ -26,6 +26,7 @@
 // benchmark-config model; the weight image is the analogue of the reference's
 // flat fp16 replica buffer (python/fp16_linear.py:249-346).
 #include "bsrl_common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -72,19 +73,20 @@ template <> __device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
 union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
 union Frag4 { s16x4 v; uint32_t w[2]; };
 
-// exact-erf GELU to ~2e-7 (Abramowitz-Stegun 7.1.26), 2 transcendentals
+// GELU(x) = x * Phi(x) with Phi(x) ~= sigmoid(x * (c0 + c1 x^2 + c2 x^4)): 7 full-rate ops + exp2 + rcp.
+// Coefficients are a minimax fit of x * sigmoid(.) to the exact-erf GELU on [-9, 9]:
+// max abs error 2.5e-5, i.e. below half an fp16 ulp of any hidden unit >= 0.06 (the
+// result is rounded to the 16-bit type straight after).  The polynomial argument is
+// clamped to [-9, 9], outside which sigmoid is 0 / 1 to fp32 precision anyway.
 __device__ __forceinline__ float gelu_fast(float x) {
-    const float z = fabsf(x) * 0.70710678118654752440f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-    float p = fmaf(t, 1.061405429f, -1.453152027f);
-    p = fmaf(t, p, 1.421413741f);
-    p = fmaf(t, p, -0.284496736f);
-    p = fmaf(t, p, 0.254829592f);
-    p *= t;
-    const float e = __expf(-z * z);
-    const float erfa = fmaf(-p, e, 1.0f);
-    const float hx = 0.5f * x;
-    return fmaf(hx, copysignf(erfa, x), hx);
+    constexpr float L2E = 1.44269504088896340736f;
+    constexpr float C0 = -1.59501576f * L2E, C1 = -7.40113019e-02f * L2E, C2 = 7.03035067e-04f * L2E;
+    const float xc = __builtin_amdgcn_fmed3f(x, -9.0f, 9.0f);
+    const float x2 = xc * xc;
+    float q = fmaf(C2, x2, C1);
+    q = fmaf(q, x2, C0);
+    const float e = __builtin_amdgcn_exp2f(xc * q);          // exp(-u)
+    return x * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 template <int ACT> __device__ __forceinline__ float act_fast(float x) {
     if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.f);
@@ -94,43 +96,47 @@ template <int ACT> __device__ __forceinline__ float act_fast(float x) {
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were
-// issued 3 stage-steps earlier into register set s & 1.
-struct Pipe {
-    uint4 r[2][2];
-    const uint4* img;
-    int next, n;
-};
-
-template <int P>   // P = parity of the stage about to be consumed
-__device__ __forceinline__ void advance(Pipe& p, uint4 (*lds)[STAGE_U4], int tid) {
-    lds_barrier();                                   // stage s is complete in slot P; slot 1-P is free
-    lds[1 - P][tid] = p.r[1 - P][0];                 // stage s+1 -> slot 1-P
-    lds[1 - P][tid + 256] = p.r[1 - P][1];
-    const uint4* src = p.img + (int64_t)p.next * STAGE_U4 + tid;   // stage s+3 -> the freed registers
-    p.r[1 - P][0] = src[0];
-    p.r[1 - P][1] = src[256];
-    p.next = p.next + 1 == p.n ? 0 : p.next + 1;
-}
-#define ADVANCE(par) do { if (par) advance<1>(pipe, lds, tid); else advance<0>(pipe, lds, tid); } while (0)
+// Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were issued 3
+// stage-steps earlier into the register pair of the same parity (pr0a/pr0b or pr1a/pr1b).
+// The four registers are plain named locals (never an indexed array: the prefetched data
+// must stay in VGPRs while in flight, a stack slot would force a wait right after the load).
+// ADVANCE_P(P): P = parity of the stage about to be consumed.
+#define ADVANCE_P(P, RA, RB) do { \
+        lds_barrier();                                   /* stage s complete in slot P; slot 1-P free */ \
+        lds[1 - (P)][tid] = RA;                          /* stage s+1 -> slot 1-P */ \
+        lds[1 - (P)][tid + 256] = RB; \
+        const uint4* src_ = img + (int64_t)pnext * STAGE_U4 + tid;   /* stage s+3 -> the freed registers */ \
+        RA = src_[0]; \
+        RB = src_[256]; \
+        pnext = pnext + 1 == a.n_stages ? 0 : pnext + 1; \
+    } while (0)
+#define ADVANCE(par) do { if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
 #define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[par][(f) * 64 + lane]))
 
 template <typename DT, int RT, int ACT>
-__global__ __launch_bounds__(256) void cfg_forward_kernel(FwdArgs a) {
+__global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     __shared__ uint4 lds[2][STAGE_U4];
+    extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
+    const float* vlds = reinterpret_cast<const float*>(vlds4);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const float scale = 0.17677669529663688110f;      // 1 / sqrt(32)
     const int64_t ntiles = (a.B + 4 * RT - 1) / (4 * RT);
 
-    Pipe pipe;
-    pipe.img = a.frags; pipe.n = a.n_stages;
+    const uint4* img = a.frags;
+    uint4 pr0a, pr0b, pr1a, pr1b;
+    int pnext;
     {   // prologue: stage 0 -> LDS slot 0; stages 1, 2 in flight
-        uint4 s0a = pipe.img[tid], s0b = pipe.img[tid + 256];
-        pipe.r[1][0] = pipe.img[STAGE_U4 + tid]; pipe.r[1][1] = pipe.img[STAGE_U4 + tid + 256];
+        const uint4 s0a = img[tid], s0b = img[tid + 256];
+        pr1a = img[STAGE_U4 + tid]; pr1b = img[STAGE_U4 + tid + 256];
         lds[0][tid] = s0a; lds[0][tid + 256] = s0b;
-        pipe.r[0][0] = pipe.img[2 * STAGE_U4 + tid]; pipe.r[0][1] = pipe.img[2 * STAGE_U4 + tid + 256];
-        pipe.next = 3 % pipe.n;
+        pr0a = img[2 * STAGE_U4 + tid]; pr0b = img[2 * STAGE_U4 + tid + 256];
+        pnext = 3 % a.n_stages;
+        // No global load other than the weight pipeline may sit in the steady state: vmcnt retires
+        // in order, so waiting on a late bias load would also drain the prefetches issued before it.
+        const int nv4 = vec_floats(a.n_layers, a.F) / 4;
+        for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        lds_barrier();
     }
 
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -167,8 +173,8 @@ __global__ __launch_bounds__(256) void cfg_forward_kernel(FwdArgs a) {
             }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const float4 bp = *reinterpret_cast<const float4*>(a.vec + V_BP + 16 * nt + 4 * g);
-                const float4 bo = *reinterpret_cast<const float4*>(a.vec + V_BO + 16 * nt + 4 * g);
+                const float4 bp = *reinterpret_cast<const float4*>(vlds + V_BP + 16 * nt + 4 * g);
+                const float4 bo = *reinterpret_cast<const float4*>(vlds + V_BO + 16 * nt + 4 * g);
                 const float4 b = r16 == 0 ? bp : bo;
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) x[rt][nt] = (f32x4){b.x, b.y, b.z, b.w};
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(256) void cfg_forward_kernel(FwdArgs a) {
         }
         // ================= transformer blocks =================
         for (int l = 0; l < a.n_layers; ++l) {
-            const float* lv = a.vec + V_LAYER0 + l * lv_size(a.F);
+            const float* lv = vlds + V_LAYER0 + l * lv_size(a.F);
             Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
             // ---- LN1 ----
             auto layer_norm = [&](int goff, int boff) {
@@ -359,7 +365,7 @@ __global__ __launch_bounds__(256) void cfg_forward_kernel(FwdArgs a) {
             for (int nt = 0; nt < NT; ++nt) {
                 gm[nt] = make_float4(1.f, 1.f, 1.f, 1.f); bt[nt] = make_float4(0.f, 0.f, 0.f, 0.f);
             }
-            const float* fv = a.vec + V_LAYER0 + a.n_layers * lv_size(a.F);
+            const float* fv = vlds + V_LAYER0 + a.n_layers * lv_size(a.F);
             if (a.final_ln) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
@@ -516,10 +522,21 @@ bool shape_ok(const bsrl_cfg_desc* d) {
 }
 int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
 
+template <typename DT, int RT, int ACT>
+int launch_fwd_act(const FwdArgs& a, unsigned grid, hipStream_t st) {
+    const size_t dyn = (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
+    auto kern = cfg_forward_kernel<DT, RT, ACT>;
+    if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+            return BSRL_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), dyn, st, a);
+    return BSRL_OK;
+}
 template <typename DT, int RT>
-void launch_fwd(const FwdArgs& a, int act, unsigned grid, hipStream_t st) {
-    if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((cfg_forward_kernel<DT, RT, BSRL_ACT_GELU>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((cfg_forward_kernel<DT, RT, BSRL_ACT_RELU>), dim3(grid), dim3(256), 0, st, a);
+int launch_fwd(const FwdArgs& a, int act, unsigned grid, hipStream_t st) {
+    if (act == BSRL_ACT_GELU) return launch_fwd_act<DT, RT, BSRL_ACT_GELU>(a, grid, st);
+    return launch_fwd_act<DT, RT, BSRL_ACT_RELU>(a, grid, st);
 }
 
 }  // namespace
@@ -576,11 +593,20 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-    constexpr int RT = 4;
-    const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
-    const unsigned grid = (unsigned)(ntiles < cus ? ntiles : cus);
-    if (d->dtype == BSRL_F16) launch_fwd<F16, RT>(a, d->act, grid, st);
-    else launch_fwd<BF16, RT>(a, d->act, grid, st);
+    int rc;
+    static const int rt_env = getenv("BSRL_CFG_RT") ? atoi(getenv("BSRL_CFG_RT")) : 4;
+    if (rt_env == 2) {
+        constexpr int RT = 2;
+        const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
+        const unsigned grid = (unsigned)(ntiles < 2 * cus ? ntiles : 2 * cus);
+        rc = d->dtype == BSRL_F16 ? launch_fwd<F16, RT>(a, d->act, grid, st) : launch_fwd<BF16, RT>(a, d->act, grid, st);
+    } else {
+        constexpr int RT = 4;
+        const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
+        const unsigned grid = (unsigned)(ntiles < cus ? ntiles : cus);
+        rc = d->dtype == BSRL_F16 ? launch_fwd<F16, RT>(a, d->act, grid, st) : launch_fwd<BF16, RT>(a, d->act, grid, st);
+    }
+    if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH("bsrl_cfg_forward");
     return BSRL_OK;
 }
