@@ -69,6 +69,10 @@ class ConfigPolicy(nn.Module):
         self._version = 0             # bumped by bump_weights_version()
         self._replica = None          # (version, dtype, device) -> 16-bit weight copies
         self._packed = None           # (version, dtype, device) -> fused-kernel weight image
+        self._workspace = None        # scratch of the pruned fused route (grown on demand, then reused)
+        # final-block query pruning on the fused route (the reference's n_queries path,
+        # python/policy.py:533-539): exact; False = one persistent kernel computing every token
+        self.prune_final = True
         self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
                      "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}
 
@@ -200,11 +204,19 @@ class ConfigPolicy(nn.Module):
         logits = torch.empty(B, n_log, device=obs.device, dtype=torch.float32)
         value = torch.empty(B, device=obs.device, dtype=torch.float32)
         desc = self._desc(dt)
+        lib = _lib.load()
+        ws_ptr, ws_bytes = None, 0
+        if self.prune_final:
+            ws_bytes = lib.bsrl_cfg_workspace_size(ctypes.byref(desc), B)
+            ws = self._workspace
+            if ws is None or ws.numel() < ws_bytes or ws.device != obs.device:
+                ws = self._workspace = torch.empty(ws_bytes, device=obs.device, dtype=torch.uint8)
+            ws_ptr = ws.data_ptr()
         with torch.cuda.device(obs.device):
-            rc = _lib.load().bsrl_cfg_forward(ctypes.byref(desc), img.data_ptr(), obs.data_ptr(), obs.stride(0),
-                                              ops.dt_code(obs.dtype), None if n_valid is None else n_valid.data_ptr(),
-                                              logits.data_ptr(), value.data_ptr(), B,
-                                              torch.cuda.current_stream(obs.device).cuda_stream)
+            rc = lib.bsrl_cfg_forward(ctypes.byref(desc), img.data_ptr(), obs.data_ptr(), obs.stride(0),
+                                      ops.dt_code(obs.dtype), None if n_valid is None else n_valid.data_ptr(),
+                                      logits.data_ptr(), value.data_ptr(), B, ws_ptr, ws_bytes,
+                                      torch.cuda.current_stream(obs.device).cuda_stream)
         if not _lib.check(rc, "bsrl_cfg_forward"):
             raise ops.Unsupported("bsrl_cfg_forward")
         return logits.view(B, N_ACTION_HEADS, self.n_gears), value

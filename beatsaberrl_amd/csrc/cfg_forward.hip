@@ -26,7 +26,6 @@
 // benchmark-config model; the weight image is the analogue of the reference's
 // flat fp16 replica buffer (python/fp16_linear.py:249-346).
 #include "bsrl_common.h"
-#include <stdlib.h>
 
 namespace {
 
@@ -57,7 +56,8 @@ struct FwdArgs {
     const void* obs; int64_t obs_ld; int obs_f32;
     const int32_t* n_valid;
     float* logits; float* value;
-    int64_t B; int n_layers, F, n_stages, n_logits, final_ln, prop_dim, obj_dim;
+    uint32_t* ws;
+    int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
 };
 
 // ---- helpers -------------------------------------------------------------------
@@ -108,12 +108,24 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
         const uint4* src_ = img + (int64_t)pnext * STAGE_U4 + tid;   /* stage s+3 -> the freed registers */ \
         RA = src_[0]; \
         RB = src_[256]; \
-        pnext = pnext + 1 == a.n_stages ? 0 : pnext + 1; \
+        pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1; \
     } while (0)
 #define ADVANCE(par) do { if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
 #define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[par][(f) * 64 + lane]))
+// all 8 fragments of the current stage -> registers in one burst of LDS reads (one wait instead of 8)
+#define LOAD_STAGE(par, W) s16x8 W[STAGE_FRAGS]; _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = WFRAG(par, f_)
 
-template <typename DT, int RT, int ACT>
+// MODE_FULL: the whole forward, one launch, every token of the last block computed.
+// MODE_HEAD + MODE_TAIL: final-block query pruning (the reference's n_queries path,
+//   python/policy.py:533-539: exact, because masking is key-side only).  HEAD runs the
+//   tokenizer, blocks 0..L-2 and the last block's LN + QKV + attention, and parks the
+//   token-0 row of every env (fp32 residual + attention-output fragments) in the
+//   workspace; TAIL re-tiles those rows 16 envs per MFMA tile and runs the last block's
+//   output projection + FFN and the 29*K + 1 output projection on them.
+enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
+constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
+
+template <typename DT, int RT, int ACT, int MODE>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     __shared__ uint4 lds[2][STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
@@ -121,17 +133,20 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const float scale = 0.17677669529663688110f;      // 1 / sqrt(32)
-    const int64_t ntiles = (a.B + 4 * RT - 1) / (4 * RT);
+    constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? 16 : 1;     // envs per 16-row MFMA tile
+    constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
+    const int64_t ntiles = (a.B + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
     const uint4* img = a.frags;
     uint4 pr0a, pr0b, pr1a, pr1b;
     int pnext;
-    {   // prologue: stage 0 -> LDS slot 0; stages 1, 2 in flight
-        const uint4 s0a = img[tid], s0b = img[tid + 256];
-        pr1a = img[STAGE_U4 + tid]; pr1b = img[STAGE_U4 + tid + 256];
+    {   // prologue: first stage -> LDS slot 0; the next two in flight (stage counts per mode are even)
+        const int s0 = a.s_begin;
+        const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
+        pr1a = img[(int64_t)(s0 + 1) * STAGE_U4 + tid]; pr1b = img[(int64_t)(s0 + 1) * STAGE_U4 + tid + 256];
         lds[0][tid] = s0a; lds[0][tid + 256] = s0b;
-        pr0a = img[2 * STAGE_U4 + tid]; pr0b = img[2 * STAGE_U4 + tid + 256];
-        pnext = 3 % a.n_stages;
+        pr0a = img[(int64_t)(s0 + 2) * STAGE_U4 + tid]; pr0b = img[(int64_t)(s0 + 2) * STAGE_U4 + tid + 256];
+        pnext = s0 + 3 >= a.s_end ? a.s_begin + (s0 + 3 - a.s_end) : s0 + 3;
         // No global load other than the weight pipeline may sit in the steady state: vmcnt retires
         // in order, so waiting on a late bias load would also drain the prefetches issued before it.
         const int nv4 = vec_floats(a.n_layers, a.F) / 4;
@@ -140,11 +155,245 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     }
 
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t env0 = tile * (4 * RT) + wave * RT;
+        const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
         int nv[RT];
         f32x4 x[RT][NT];
-        // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
-        {
+        Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
+        Frag8 of[RT][KC];       // attention output fragments (chunk == head)
+
+        // y = LN(x) * gamma + beta (or the raw x when !affine), packed as operand fragments
+        auto norm_to_frags = [&](const float* gptr, const float* bptr, bool normalise, Frag8 (&dst)[RT][KC]) {
+            float4 gm[NT], bt[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                gm[nt] = make_float4(1.f, 1.f, 1.f, 1.f); bt[nt] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (normalise) {
+                    gm[nt] = *reinterpret_cast<const float4*>(gptr + 16 * nt + 4 * g);
+                    bt[nt] = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                float mean = 0.f, rstd = 1.f;
+                if (normalise) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
+                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
+                    mean = s * (1.0f / D);
+                    float q = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
+                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
+                    rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
+                }
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
+                    const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
+                    const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
+                    const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
+                    dst[rt][nt >> 1].w[(nt & 1) * 2] = pack2<DT>(y0, y1);
+                    dst[rt][nt >> 1].w[(nt & 1) * 2 + 1] = pack2<DT>(y2, y3);
+                }
+            }
+        };
+        auto add_bias = [&](const float* bptr) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 b = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) { x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w; }
+            }
+        };
+
+        // ---- LN1 + QKV + attention of one block (12 stages), head by head: fills `of` ----
+        auto attention = [&](const float* lv) {
+            norm_to_frags(lv + LV_LN1G, lv + LV_LN1B, true, hf);
+#pragma unroll
+            for (int hd = 0; hd < H; ++hd) {
+                Frag8 qf[RT], kf[RT];
+                Frag4 vt[RT][2];
+#pragma unroll
+                for (int part = 0; part < 3; ++part) {
+                    const int par = (hd * 3 + part) & 1;        // stage parity (the block starts on an even stage)
+                    ADVANCE(par);
+                    LOAD_STAGE(par, wf);
+                    f32x4 acc[2][RT];
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                        if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? LV_BQ : LV_BK) + 32 * hd + 16 * ntl + 4 * g);
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
+                    }
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) {
+                                const s16x8 w = wf[ntl * KC + c];
+                                if (part < 2) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
+                                else acc[ntl][rt] = DT::mfma32(hf[rt][c].v, w, acc[ntl][rt]);   // V^T: roles swapped
+                            }
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) {
+                            const uint32_t lo = pack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]);
+                            const uint32_t hi = pack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
+                            if (part == 0) { qf[rt].w[ntl * 2] = lo; qf[rt].w[ntl * 2 + 1] = hi; }
+                            else if (part == 1) { kf[rt].w[ntl * 2] = lo; kf[rt].w[ntl * 2 + 1] = hi; }
+                            else { vt[rt][ntl].w[0] = lo; vt[rt][ntl].w[1] = hi; }
+                        }
+                }
+                // scores^T = K Q^T (lane: query r16, keys 4g..4g+3), softmax over keys, O = P V (+ b_v)
+                const float4 bv0 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 4 * g);
+                const float4 bv1 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 16 + 4 * g);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    f32x4 sc = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                    float sv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sv[i] = (4 * g + i) <= nv[rt] ? sc[i] * scale : -INFINITY;
+                    float m = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+                    m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
+                    float sum = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[i] = __expf(sv[i] - m); sum += sv[i]; }
+                    sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
+                    const float inv = __builtin_amdgcn_rcpf(sum);
+                    Frag4 pf;
+                    pf.w[0] = pack2<DT>(sv[0] * inv, sv[1] * inv);
+                    pf.w[1] = pack2<DT>(sv[2] * inv, sv[3] * inv);
+                    const f32x4 o0 = DT::mfma16(vt[rt][0].v, pf.v, (f32x4){bv0.x, bv0.y, bv0.z, bv0.w});
+                    const f32x4 o1 = DT::mfma16(vt[rt][1].v, pf.v, (f32x4){bv1.x, bv1.y, bv1.z, bv1.w});
+                    of[rt][hd].w[0] = pack2<DT>(o0[0], o0[1]); of[rt][hd].w[1] = pack2<DT>(o0[2], o0[3]);
+                    of[rt][hd].w[2] = pack2<DT>(o1[0], o1[1]); of[rt][hd].w[3] = pack2<DT>(o1[2], o1[3]);
+                }
+            }
+        };
+
+        // ---- output projection onto the residual (4 stages), then LN2 + FFN (2 * F/32 stages) ----
+        auto proj_and_ffn = [&](const float* lv) {
+            add_bias(lv + LV_BOUT);
+#pragma unroll
+            for (int st = 0; st < NT / 2; ++st) {
+                ADVANCE(st & 1);            // 12 stages precede in the block: parity restarts even
+                LOAD_STAGE(st & 1, wf);
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], of[rt][c].v, x[rt][2 * st + ntl]);
+            }
+            norm_to_frags(lv + LV_LN2G, lv + LV_LN2B, true, hf);
+            add_bias(lv + lv_b2(a.F));
+            // Software-pipelined over 32-wide hidden chunks: the up-projection MFMAs of chunk ch+1
+            // are issued next to the activation (VALU) of chunk ch, then the down-projection of
+            // chunk ch runs.  Stage order in the image: W1(0), {W1(ch+1), W2(ch)}..., W2(last).
+            const int nch = a.F / 32;
+            f32x4 accA[2][RT];
+            auto ffn_up = [&](const s16x8 (&w1)[STAGE_FRAGS], int ch, f32x4 (&acc)[2][RT]) {
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const float4 b = *reinterpret_cast<const float4*>(lv + LV_B1 + 32 * ch + 16 * ntl + 4 * g);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
+                }
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, acc[ntl][rt]);
+            };
+            auto ffn_act = [&](const f32x4 (&acc)[2][RT], Frag8 (&hid)[RT]) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        hid[rt].w[ntl * 2] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][0]), act_fast<ACT>(acc[ntl][rt][1]));
+                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][2]), act_fast<ACT>(acc[ntl][rt][3]));
+                    }
+            };
+            auto ffn_down = [&](const s16x8 (&w2)[STAGE_FRAGS], const Frag8 (&hid)[RT]) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w2[nt], hid[rt].v, x[rt][nt]);
+            };
+            {
+                ADVANCE(0);
+                LOAD_STAGE(0, w1);
+                ffn_up(w1, 0, accA);
+            }
+            for (int ch = 0; ch < nch - 1; ++ch) {
+                Frag8 hid[RT];
+                f32x4 accB[2][RT];
+                {
+                    ADVANCE(1);
+                    LOAD_STAGE(1, w1);
+                    ffn_up(w1, ch + 1, accB);
+                    ffn_act(accA, hid);
+                }
+                {
+                    ADVANCE(0);
+                    LOAD_STAGE(0, w2);
+                    ffn_down(w2, hid);
+                }
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) accA[ntl][rt] = accB[ntl][rt];
+            }
+            {
+                Frag8 hid[RT];
+                ffn_act(accA, hid);
+                ADVANCE(1);
+                LOAD_STAGE(1, w2);
+                ffn_down(w2, hid);
+            }
+        };
+
+        // ---- 29*K + 1 output projection (8 stages); rf[i] = operand fragments whose rows are envs,
+        //      row r16 of tile i being env env_base + i * 16 + r16 (stored when r16 < rows_valid) ----
+        auto heads = [&](auto& rf, int64_t env_base, int rows_valid, const float* fvp) {
+            constexpr int NR = sizeof(rf) / sizeof(rf[0]);
+#pragma unroll
+            for (int st = 0; st < HEAD_STAGES; ++st) {
+                ADVANCE(st & 1);            // an even number of stages precedes the readout
+                LOAD_STAGE(st & 1, wf);
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int nt = 2 * st + ntl;
+                    const float4 b = *reinterpret_cast<const float4*>(fvp + FV_BH + 16 * nt + 4 * g);
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) {
+                        f32x4 acc = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                        for (int c = 0; c < KC; ++c) acc = DT::mfma32(wf[ntl * KC + c], rf[i][c].v, acc);
+                        const int64_t env = env_base + i * 16 + r16;
+                        if (r16 < rows_valid && env < a.B) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int col = 16 * nt + 4 * g + e;
+                                if (col < a.n_logits) a.logits[env * a.n_logits + col] = acc[e];
+                                else if (col == a.n_logits) a.value[env] = acc[e];
+                            }
+                        }
+                    }
+                }
+            }
+        };
+        const float* fv = vlds + V_LAYER0 + a.n_layers * lv_size(a.F);
+
+        if (MODE != MODE_TAIL) {
+            // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
             Frag8 e[RT][KC];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -182,251 +431,73 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 #pragma unroll
             for (int st = 0; st < EMB_STAGES; ++st) {
                 ADVANCE(st & 1);
+                LOAD_STAGE(st & 1, wf);
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
 #pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        const s16x8 w = WFRAG(st & 1, ntl * KC + c);
+                    for (int ntl = 0; ntl < 2; ++ntl)
 #pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(w, e[rt][c].v, x[rt][2 * st + ntl]);
-                    }
+                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], e[rt][c].v, x[rt][2 * st + ntl]);
             }
-        }
-        // ================= transformer blocks =================
-        for (int l = 0; l < a.n_layers; ++l) {
-            const float* lv = vlds + V_LAYER0 + l * lv_size(a.F);
-            Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
-            // ---- LN1 ----
-            auto layer_norm = [&](int goff, int boff) {
-                float4 gm[NT], bt[NT];
+            // ================= transformer blocks =================
+            const int dense_layers = MODE == MODE_FULL ? a.n_layers : a.n_layers - 1;
+            for (int l = 0; l < dense_layers; ++l) {
+                const float* lv = vlds + V_LAYER0 + l * lv_size(a.F);
+                attention(lv);
+                proj_and_ffn(lv);
+            }
+            if (MODE == MODE_HEAD) {
+                // last block: attention only, then park token 0 (lanes r16 == 0) for the TAIL launch
+                attention(vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F));
+                if (r16 == 0) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    gm[nt] = *reinterpret_cast<const float4*>(lv + goff + 16 * nt + 4 * g);
-                    bt[nt] = *reinterpret_cast<const float4*>(lv + boff + 16 * nt + 4 * g);
-                }
+                    for (int rt = 0; rt < RT; ++rt) {
+                        const int64_t env = env0 + rt;
+                        if (env < a.B) {
+                            uint4* dst = reinterpret_cast<uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                    float s = 0.f;
+                            for (int nt = 0; nt < NT; ++nt) dst[nt] = __builtin_bit_cast(uint4, x[rt][nt]);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
-                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
-                    const float mean = s * (1.0f / D);
-                    float q = 0.f;
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
-                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
-                    const float rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
-                        const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
-                        const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
-                        const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
-                        hf[rt][nt >> 1].w[(nt & 1) * 2] = pack2<DT>(y0, y1);
-                        hf[rt][nt >> 1].w[(nt & 1) * 2 + 1] = pack2<DT>(y2, y3);
-                    }
-                }
-            };
-            layer_norm(LV_LN1G, LV_LN1B);
-
-            // ---- QKV + attention, head by head ----
-            Frag8 of[RT][KC];       // attention output fragments (chunk == head)
-#pragma unroll
-            for (int hd = 0; hd < H; ++hd) {
-                Frag8 qf[RT], kf[RT];
-                Frag4 vt[RT][2];
-#pragma unroll
-                for (int part = 0; part < 3; ++part) {
-                    const int par = (hd * 3 + part) & 1;        // stage parity inside the layer (layer starts even)
-                    ADVANCE(par);
-                    f32x4 acc[2][RT];
-#pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
-                        if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? LV_BQ : LV_BK) + 32 * hd + 16 * ntl + 4 * g);
-#pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
-                    }
-#pragma unroll
-                    for (int c = 0; c < KC; ++c)
-#pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl) {
-                            const s16x8 w = WFRAG(par, ntl * KC + c);
-#pragma unroll
-                            for (int rt = 0; rt < RT; ++rt) {
-                                if (part < 2) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
-                                else acc[ntl][rt] = DT::mfma32(hf[rt][c].v, w, acc[ntl][rt]);   // V^T: roles swapped
-                            }
+                            for (int c = 0; c < KC; ++c) dst[NT + c] = of[rt][c].u;
                         }
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl) {
-                            const uint32_t lo = pack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]);
-                            const uint32_t hi = pack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
-                            if (part == 0) { qf[rt].w[ntl * 2] = lo; qf[rt].w[ntl * 2 + 1] = hi; }
-                            else if (part == 1) { kf[rt].w[ntl * 2] = lo; kf[rt].w[ntl * 2 + 1] = hi; }
-                            else { vt[rt][ntl].w[0] = lo; vt[rt][ntl].w[1] = hi; }
-                        }
-                }
-                // scores^T = K Q^T (lane: query r16, keys 4g..4g+3), softmax over keys, O = P V (+ b_v)
-                const float4 bv0 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 4 * g);
-                const float4 bv1 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 16 + 4 * g);
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                    f32x4 s = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
-                    float sv[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) sv[i] = (4 * g + i) <= nv[rt] ? s[i] * scale : -INFINITY;
-                    float m = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-                    m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
-                    float sum = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { sv[i] = __expf(sv[i] - m); sum += sv[i]; }
-                    sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
-                    const float inv = __builtin_amdgcn_rcpf(sum);
-                    Frag4 pf;
-                    pf.w[0] = pack2<DT>(sv[0] * inv, sv[1] * inv);
-                    pf.w[1] = pack2<DT>(sv[2] * inv, sv[3] * inv);
-                    const f32x4 o0 = DT::mfma16(vt[rt][0].v, pf.v, (f32x4){bv0.x, bv0.y, bv0.z, bv0.w});
-                    const f32x4 o1 = DT::mfma16(vt[rt][1].v, pf.v, (f32x4){bv1.x, bv1.y, bv1.z, bv1.w});
-                    of[rt][hd].w[0] = pack2<DT>(o0[0], o0[1]); of[rt][hd].w[1] = pack2<DT>(o0[2], o0[3]);
-                    of[rt][hd].w[2] = pack2<DT>(o1[0], o1[1]); of[rt][hd].w[3] = pack2<DT>(o1[2], o1[3]);
-                }
-            }
-            // ---- output projection, accumulated onto the residual ----
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const float4 b = *reinterpret_cast<const float4*>(lv + LV_BOUT + 16 * nt + 4 * g);
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) { x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w; }
-            }
-#pragma unroll
-            for (int st = 0; st < NT / 2; ++st) {
-                ADVANCE(st & 1);            // 12 stages precede: parity restarts even
-#pragma unroll
-                for (int c = 0; c < KC; ++c)
-#pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        const s16x8 w = WFRAG(st & 1, ntl * KC + c);
-#pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(w, of[rt][c].v, x[rt][2 * st + ntl]);
                     }
-            }
-            // ---- LN2 + FFN (hidden stays in registers, 32 hidden units per step) ----
-            layer_norm(LV_LN2G, LV_LN2B);
-            const int b2off = lv_b2(a.F);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const float4 b = *reinterpret_cast<const float4*>(lv + b2off + 16 * nt + 4 * g);
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) { x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w; }
-            }
-            for (int ch = 0; ch < a.F / 32; ++ch) {
-                ADVANCE(0);
-                f32x4 acc[2][RT];
-#pragma unroll
-                for (int ntl = 0; ntl < 2; ++ntl) {
-                    const float4 b = *reinterpret_cast<const float4*>(lv + LV_B1 + 32 * ch + 16 * ntl + 4 * g);
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
                 }
+            } else {
+                // ================= readout: token 0 of every env -> 29*K logits + value =================
+                Frag8 yf[RT][KC];
+                norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
+                Frag8 rf[1][KC];        // B operand: lane (env r16 < RT, group g)
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
-#pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        const s16x8 w = WFRAG(0, ntl * KC + c);
-#pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
-                    }
-                Frag8 hid[RT];
+                for (int c = 0; c < KC; ++c) rf[0][c].u = make_uint4(0, 0, 0, 0);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        hid[rt].w[ntl * 2] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][0]), act_fast<ACT>(acc[ntl][rt][1]));
-                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][2]), act_fast<ACT>(acc[ntl][rt][3]));
-                    }
-                ADVANCE(1);
+                    for (int c = 0; c < KC; ++c)
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const s16x8 w = WFRAG(1, nt);
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w, hid[rt].v, x[rt][nt]);
-                }
+                        for (int w = 0; w < 4; ++w) {
+                            // row 0 of this env's tile sits in lanes 16*g; hand it to lane (r16 == rt, g)
+                            const uint32_t v = __shfl(yf[rt][c].w[w], 16 * g, WAVE);
+                            if (r16 == rt) rf[0][c].w[w] = v;
+                        }
+                heads(rf, env0, RT, fv);
             }
-        }
-        // ================= readout: token 0 of every env -> 29*K logits + value =================
-        {
-            float4 gm[NT], bt[NT];
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                gm[nt] = make_float4(1.f, 1.f, 1.f, 1.f); bt[nt] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-            const float* fv = vlds + V_LAYER0 + a.n_layers * lv_size(a.F);
-            if (a.final_ln) {
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    gm[nt] = *reinterpret_cast<const float4*>(fv + FV_LNG + 16 * nt + 4 * g);
-                    bt[nt] = *reinterpret_cast<const float4*>(fv + FV_LNB + 16 * nt + 4 * g);
-                }
-            }
-            Frag8 rf[KC];           // B operand: lane (env r16 < RT, group g)
-#pragma unroll
-            for (int c = 0; c < KC; ++c) rf[c].u = make_uint4(0, 0, 0, 0);
+        } else {
+            // ================= TAIL: rows are envs (token 0 of each) =================
+            const float* lv = vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                float mean = 0.f, rstd = 1.f;
-                if (a.final_ln) {
-                    float s = 0.f;
+                int64_t env = env0 + rt * 16 + r16; env = env < a.B ? env : a.B - 1;
+                nv[rt] = 0;
+                const uint4* src = reinterpret_cast<const uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
-                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
-                    mean = s * (1.0f / D);
-                    float q = 0.f;
+                for (int nt = 0; nt < NT; ++nt) x[rt][nt] = __builtin_bit_cast(f32x4, src[nt]);
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
-                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
-                    rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
-                }
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
-                    const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
-                    const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
-                    const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
-                    // row 0 of this env's tile sits in lanes 16*g; hand it to lane (r16 == rt, g)
-                    const uint32_t lo = __shfl(pack2<DT>(y0, y1), 16 * g, WAVE);
-                    const uint32_t hi = __shfl(pack2<DT>(y2, y3), 16 * g, WAVE);
-                    if (r16 == rt) { rf[nt >> 1].w[(nt & 1) * 2] = lo; rf[nt >> 1].w[(nt & 1) * 2 + 1] = hi; }
-                }
+                for (int c = 0; c < KC; ++c) of[rt][c].u = src[NT + c];
             }
-            const int64_t env = env0 + r16;
-            const bool store = r16 < RT && env < a.B;
-#pragma unroll
-            for (int st = 0; st < HEAD_STAGES; ++st) {
-                ADVANCE(st & 1);            // an even number of stages precedes the readout
-#pragma unroll
-                for (int ntl = 0; ntl < 2; ++ntl) {
-                    const int nt = 2 * st + ntl;
-                    const float4 b = *reinterpret_cast<const float4*>(fv + FV_BH + 16 * nt + 4 * g);
-                    f32x4 acc = {b.x, b.y, b.z, b.w};
-#pragma unroll
-                    for (int c = 0; c < KC; ++c) acc = DT::mfma32(WFRAG(st & 1, ntl * KC + c), rf[c].v, acc);
-                    if (store) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int col = 16 * nt + 4 * g + i;
-                            if (col < a.n_logits) a.logits[env * a.n_logits + col] = acc[i];
-                            else if (col == a.n_logits) a.value[env] = acc[i];
-                        }
-                    }
-                }
-            }
+            proj_and_ffn(lv);
+            Frag8 yf[RT][KC];
+            norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
+            heads(yf, env0, 16, fv);
         }
     }
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
@@ -473,9 +544,14 @@ __global__ __launch_bounds__(256) void cfg_pack_frags_kernel(PackArgs a) {
             const int r2 = r - 3 * H * 8;
             src = a.p.blk[l].out_w; ld = D; n = 16 * (r2 / KC) + n16; c = r2 % KC;
         } else {
-            const int r3 = r - 3 * H * 8 - NT * KC, ch = r3 / 16, q = r3 % 16;
-            if (q < 8) { src = a.p.blk[l].ffn0_w; ld = D; n = 32 * ch + 16 * (q / KC) + n16; c = q % KC; }
-            else { src = a.p.blk[l].ffn2_w; ld = a.F; n = 16 * (q - 8) + n16; c = 0; kbase = 32 * ch; }
+            // FFN stage order: W1(0), {W1(ch+1), W2(ch)} for ch = 0..nch-2, W2(nch-1)
+            const int r3 = r - 3 * H * 8 - NT * KC, s3 = r3 / 8, q = r3 % 8, nch = a.F / 32;
+            bool up; int ch;
+            if (s3 == 0) { up = true; ch = 0; }
+            else if (s3 == 2 * nch - 1) { up = false; ch = nch - 1; }
+            else { up = ((s3 - 1) & 1) == 0; ch = (s3 - 1) / 2 + (up ? 1 : 0); }
+            if (up) { src = a.p.blk[l].ffn0_w; ld = D; n = 32 * ch + 16 * (q / KC) + n16; c = q % KC; }
+            else { src = a.p.blk[l].ffn2_w; ld = a.F; n = 16 * q + n16; c = 0; kbase = 32 * ch; }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + perm_k(c, gg, j)];
@@ -522,21 +598,34 @@ bool shape_ok(const bsrl_cfg_desc* d) {
 }
 int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
 
-template <typename DT, int RT, int ACT>
-int launch_fwd_act(const FwdArgs& a, unsigned grid, hipStream_t st) {
+template <typename DT, int RT, int ACT, int MODE>
+int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
     const size_t dyn = (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
-    auto kern = cfg_forward_kernel<DT, RT, ACT>;
+    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE>;
     if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), dyn, st, a);
+    const int64_t per_wg = 4 * RT * (MODE == MODE_TAIL ? 16 : 1);
+    const int64_t ntiles = (a.B + per_wg - 1) / per_wg;
+    const int64_t resident = (int64_t)cus * (RT <= 2 ? 2 : 1);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < resident ? ntiles : resident)), dim3(256), dyn, st, a);
     return BSRL_OK;
 }
-template <typename DT, int RT>
-int launch_fwd(const FwdArgs& a, int act, unsigned grid, hipStream_t st) {
-    if (act == BSRL_ACT_GELU) return launch_fwd_act<DT, RT, BSRL_ACT_GELU>(a, grid, st);
-    return launch_fwd_act<DT, RT, BSRL_ACT_RELU>(a, grid, st);
+
+template <typename DT, int ACT>
+int launch_all(FwdArgs a, bool pruned, int cus, hipStream_t st) {
+    const int ls = layer_stages(a.F), total = total_stages(a.n_layers, a.F);
+    if (!pruned) {
+        a.s_begin = 0; a.s_end = total;
+        return launch_one<DT, 2, ACT, MODE_FULL>(a, cus, st);
+    }
+    const int split = EMB_STAGES + (a.n_layers - 1) * ls + 3 * H;
+    a.s_begin = 0; a.s_end = split;
+    int rc = launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
+    if (rc != BSRL_OK) return rc;
+    a.s_begin = split; a.s_end = total;
+    return launch_one<DT, 1, ACT, MODE_TAIL>(a, cus, st);
 }
 
 }  // namespace
@@ -572,9 +661,14 @@ extern "C" int bsrl_cfg_pack(const bsrl_cfg_desc* d, const bsrl_cfg_params* p, v
     return BSRL_OK;
 }
 
+extern "C" int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* d, int64_t B) {
+    if (!shape_ok(d) || B <= 0) return 0;
+    return B * 4 * WS_DWORDS * (int64_t)sizeof(uint32_t);
+}
+
 extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
                                 int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
-                                bsrl_stream stream) {
+                                void* workspace, int64_t workspace_bytes, bsrl_stream stream) {
     if (!d || !packed || !obs || !logits || !value) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: null pointer");
     if (!shape_ok(d)) return BSRL_UNSUPPORTED;
     if (B < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: negative batch");
@@ -587,25 +681,20 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.vec = reinterpret_cast<const float*>(static_cast<const char*>(packed) + frag_bytes(d));
     a.obs = obs; a.obs_ld = obs_ld; a.obs_f32 = obs_dtype == BSRL_F32;
     a.n_valid = n_valid; a.logits = logits; a.value = value; a.B = B;
-    a.n_layers = d->n_layers; a.F = d->ffn; a.n_stages = total_stages(d->n_layers, d->ffn);
+    a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
+    a.ws = static_cast<uint32_t*>(workspace);
+    const bool pruned = workspace && workspace_bytes >= bsrl_cfg_workspace_size(d, B);
+    if (workspace && !bsrl_aligned(workspace, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: workspace must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
     int rc;
-    static const int rt_env = getenv("BSRL_CFG_RT") ? atoi(getenv("BSRL_CFG_RT")) : 4;
-    if (rt_env == 2) {
-        constexpr int RT = 2;
-        const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
-        const unsigned grid = (unsigned)(ntiles < 2 * cus ? ntiles : 2 * cus);
-        rc = d->dtype == BSRL_F16 ? launch_fwd<F16, RT>(a, d->act, grid, st) : launch_fwd<BF16, RT>(a, d->act, grid, st);
-    } else {
-        constexpr int RT = 4;
-        const int64_t ntiles = (B + 4 * RT - 1) / (4 * RT);
-        const unsigned grid = (unsigned)(ntiles < cus ? ntiles : cus);
-        rc = d->dtype == BSRL_F16 ? launch_fwd<F16, RT>(a, d->act, grid, st) : launch_fwd<BF16, RT>(a, d->act, grid, st);
-    }
+    if (d->dtype == BSRL_F16)
+        rc = d->act == BSRL_ACT_GELU ? launch_all<F16, BSRL_ACT_GELU>(a, pruned, cus, st) : launch_all<F16, BSRL_ACT_RELU>(a, pruned, cus, st);
+    else
+        rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, cus, st);
     if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH("bsrl_cfg_forward");
     return BSRL_OK;

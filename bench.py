@@ -65,6 +65,8 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="override B (0 = the config's B)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-eager", action="store_true", help="skip the torch-ROCm eager leg")
+    ap.add_argument("--no-prune", action="store_true",
+                    help="fused route: one persistent kernel computing every token of the last block")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures ONE GPU: the forward is embarrassingly data-parallel (env rows are "
@@ -85,6 +87,7 @@ def main():
     m = ConfigPolicy.from_spec(spec, dtype=dtype, route=args.route)
     m.load_state_dict(p)
     m = m.to(dev)
+    m.prune_final = not args.no_prune
     obs, k = obs_cpu.to(dev), k_cpu.to(dev)
     route = args.route
     if route == "auto":
@@ -115,17 +118,25 @@ def main():
     dev_ms_avg = sum(dev_ms) / len(dev_ms)
     value = B / (ms_per_step * 1e-3)
 
-    flops = cm.flops_per_env(spec) * B
-    # Dominant kernel: on the fused route the forward IS one kernel, so its launch
-    # duration is the event-bracketed step; on the ops route the events bracket the
-    # whole launch train and the figure is the pipeline's, not one kernel's.
-    achieved = flops / (dev_ms_avg * 1e-3) / 1e12
+    # FLOPs per forward: the dense algorithmic figure (every token of every block), and the
+    # EXECUTED figure when the fused route prunes the final block to token 0 (the reference's
+    # own n_queries path): the roofline fraction is quoted on executed work only.
+    dense_flops = cm.flops_per_env(spec) * B
+    pruned = route == "fused" and m.prune_final
+    exec_flops = dense_flops
+    if pruned:
+        d_, T_, F_ = spec.d, spec.T, spec.ffn
+        saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the 15 unread tokens
+        exec_flops = dense_flops - 2 * saved * B
+    achieved = exec_flops / (dev_ms_avg * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[dtype]
+    kname = ("cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
+             "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else "launch train (per-op route)")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": None,
-                "kernel": "cfg_forward (whole forward)" if route == "fused" else "launch train (per-op route)",
+                "frac": round(achieved / peak, 4), "traffic": None, "kernel": kname,
                 "launch_ms_avg": round(dev_ms_avg, 4), "launch_ms_p50": round(dev_ms[len(dev_ms) // 2], 4),
-                "flop_per_launch": flops}
+                "flop_per_launch": exec_flops, "dense_flop_per_forward": dense_flops,
+                "dense_equivalent_frac": round(dense_flops / (dev_ms_avg * 1e-3) / 1e12 / peak, 4)}
 
     out = {"metric": "policy fwd env-samples/sec at B=16384 fp16 (1 GPU); % of MFMA roofline",
            "value": round(value, 1), "unit": "env-samples/s", "n_gpus": 1, "steps": args.steps,

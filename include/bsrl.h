@@ -149,11 +149,22 @@ int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* desc);
  * image (the analogue of fp16_linear.flat_refresh, fp16_linear.py:241-246). */
 int bsrl_cfg_pack(const bsrl_cfg_desc* desc, const bsrl_cfg_params* params,
                   void* packed, bsrl_stream stream);
-/* obs (B, obs_ld) F32 or 16-bit; n_valid (B,) int32 or NULL (all valid). */
+/* Bytes of scratch the pruned two-launch form of bsrl_cfg_forward needs for B envs
+ * (768 B per env), or 0 if the shape is unsupported. */
+int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
+/* obs (B, obs_ld) F32 or 16-bit; n_valid (B,) int32 or NULL (all valid).
+ * workspace == NULL (or smaller than bsrl_cfg_workspace_size): ONE persistent
+ * kernel computes every token of every block.  With a workspace: final-block
+ * query pruning, the reference's n_queries path (python/policy.py:533-539,
+ * :1302-1305; exact, masking is key-side only) - launch 1 runs the tokenizer,
+ * blocks 0..L-2 and the last block's attention and parks each env's token-0
+ * row in the workspace, launch 2 runs the last block's output projection +
+ * FFN and the heads on those rows, 16 envs per MFMA tile. */
 int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      const void* obs, int64_t obs_ld, int obs_dtype,
                      const int32_t* n_valid, float* logits, float* value,
-                     int64_t B, bsrl_stream stream);
+                     int64_t B, void* workspace, int64_t workspace_bytes,
+                     bsrl_stream stream);
 
 #ifdef __cplusplus
 }

@@ -141,12 +141,16 @@ def test_weights_version_refreshes_replicas(route):
 
 
 # ------------------------------------------------------------------ fused whole-forward kernel
+@pytest.mark.parametrize("prune", [False, True])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("B", [1, 8, 64, 1000, 4096])
-def test_fused_route_config1(dtype, B):
+def test_fused_route_config1(dtype, B, prune):
+    """prune=False: one persistent kernel, every token of the last block; prune=True: the
+    two-launch form with final-block query pruning (same results to the precision class)."""
     c = cm.CONFIGS[1]
     spec = c["spec"]
     p, m = _build(spec, c["w_seed"], dtype, "fused")
+    m.prune_final = prune
     assert m.fused_supported()
     obs, k = cm.make_inputs(spec, B, c["obs_seed"], c["mask"])
     lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
@@ -160,8 +164,10 @@ def test_fused_route_variants(act, final_ln, L, ffn, dtype):
     spec = cm.ConfigSpec(L, 128, 4, ffn, 16, act=act, final_ln=final_ln)
     p, m = _build(spec, 31, dtype, "fused")
     obs, k = cm.make_inputs(spec, 333, 32, "quarter_empty")
-    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
-    _check16(lg, v, p, spec, obs, k, dtype, round_residual=False)
+    for prune in (False, True):
+        m.prune_final = prune
+        lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+        _check16(lg, v, p, spec, obs, k, dtype, round_residual=False)
 
 
 def test_fused_route_other_obs_layouts_and_no_mask():
@@ -176,10 +182,12 @@ def test_fused_route_other_obs_layouts_and_no_mask():
     assert torch.equal(lg, lg2) and torch.equal(v, v2)       # the kernel rounds fp32 obs to fp16 once on entry
 
 
-def test_fused_route_invariants():
+@pytest.mark.parametrize("prune", [False, True])
+def test_fused_route_invariants(prune):
     c = cm.CONFIGS[1]
     spec = c["spec"]
     p, m = _build(spec, 1, "f16", "fused")
+    m.prune_final = prune
     obs, k = cm.make_inputs(spec, 700, 3, "uniform")
     od, kd = obs.to(DEV), k.to(DEV)
     lg, v = m.forward_stacked(od, kd)
@@ -199,6 +207,10 @@ def test_fused_route_invariants():
     # repeated launches are bitwise reproducible
     l5, v5 = m.forward_stacked(od, kd)
     assert torch.equal(l5, lg) and torch.equal(v5, v)
+    # pruned and unpruned forms agree to fp32-accumulation-order level on most logits
+    m.prune_final = not prune
+    l6, _ = m.forward_stacked(od, kd)
+    assert (l6 - lg).abs().max().item() < 5e-3
 
 
 def test_fused_unsupported_shapes_fall_to_ops_route():
