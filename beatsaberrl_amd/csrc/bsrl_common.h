@@ -70,6 +70,27 @@ template <int ACT> __device__ __forceinline__ float apply_act(float x) {
     if (ACT == BSRL_ACT_GELU) return gelu_exact(x);
     return x;
 }
+// GELU(x) = x * Phi(x) with Phi(x) ~= sigmoid(x * (c0 + c1 x^2 + c2 x^4)): 7 full-rate ops + exp2 + rcp.
+// Coefficients are a minimax fit of x * sigmoid(.) to the exact-erf GELU on [-9, 9]: max abs error
+// 2.5e-5, below half an fp16 ulp of any value >= 0.06, so it is only used where the result is rounded
+// to a 16-bit type straight after.  The polynomial argument is clamped to [-9, 9], outside which the
+// sigmoid is 0 / 1 to fp32 precision anyway.
+__device__ __forceinline__ float gelu_fast(float x) {
+    constexpr float L2E = 1.44269504088896340736f;
+    constexpr float C0 = -1.59501576f * L2E, C1 = -7.40113019e-02f * L2E, C2 = 7.03035067e-04f * L2E;
+    const float xc = __builtin_amdgcn_fmed3f(x, -9.0f, 9.0f);
+    const float x2 = xc * xc;
+    float q = fmaf(C2, x2, C1);
+    q = fmaf(q, x2, C0);
+    const float e = __builtin_amdgcn_exp2f(xc * q);          // exp(-u)
+    return x * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+// activation for values about to be rounded to fp16 / bf16
+template <int ACT> __device__ __forceinline__ float apply_act16(float x) {
+    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_GELU) return gelu_fast(x);
+    return x;
+}
 
 // ---- wave-level reductions -------------------------------------------------------
 // Butterfly over the low `width` lanes of each width-aligned lane group.

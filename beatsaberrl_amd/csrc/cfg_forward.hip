@@ -73,27 +73,6 @@ template <> __device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
 union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
 union Frag4 { s16x4 v; uint32_t w[2]; };
 
-// GELU(x) = x * Phi(x) with Phi(x) ~= sigmoid(x * (c0 + c1 x^2 + c2 x^4)): 7 full-rate ops + exp2 + rcp.
-// Coefficients are a minimax fit of x * sigmoid(.) to the exact-erf GELU on [-9, 9]:
-// max abs error 2.5e-5, i.e. below half an fp16 ulp of any hidden unit >= 0.06 (the
-// result is rounded to the 16-bit type straight after).  The polynomial argument is
-// clamped to [-9, 9], outside which sigmoid is 0 / 1 to fp32 precision anyway.
-__device__ __forceinline__ float gelu_fast(float x) {
-    constexpr float L2E = 1.44269504088896340736f;
-    constexpr float C0 = -1.59501576f * L2E, C1 = -7.40113019e-02f * L2E, C2 = 7.03035067e-04f * L2E;
-    const float xc = __builtin_amdgcn_fmed3f(x, -9.0f, 9.0f);
-    const float x2 = xc * xc;
-    float q = fmaf(C2, x2, C1);
-    q = fmaf(q, x2, C0);
-    const float e = __builtin_amdgcn_exp2f(xc * q);          // exp(-u)
-    return x * __builtin_amdgcn_rcpf(e + 1.0f);
-}
-template <int ACT> __device__ __forceinline__ float act_fast(float x) {
-    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.f);
-    if (ACT == BSRL_ACT_GELU) return gelu_fast(x);
-    return x;
-}
-
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were issued 3
@@ -317,8 +296,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                     for (int ntl = 0; ntl < 2; ++ntl) {
-                        hid[rt].w[ntl * 2] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][0]), act_fast<ACT>(acc[ntl][rt][1]));
-                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(act_fast<ACT>(acc[ntl][rt][2]), act_fast<ACT>(acc[ntl][rt][3]));
+                        hid[rt].w[ntl * 2] = pack2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
+                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
                     }
             };
             auto ffn_down = [&](const s16x8 (&w2)[STAGE_FRAGS], const Frag8 (&hid)[RT]) {

@@ -1,6 +1,184 @@
-// Fused FFN (placeholder until the kernel lands: reports "unsupported").
+// Fused FFN for gfx950:  xo = x + act(h2 W0^T + b0) W2^T + b2 ;  ho = LayerNorm(xo).
+//
+// A workgroup of 4 waves owns 64*RT rows; each wave keeps its 16*RT-row slice
+// of the fp32 output accumulator (residual + b2 folded in) and its h2 operand
+// fragments in registers for the whole kernel.  The hidden layer is walked in
+// chunks of 32 units: the chunk's W0 rows and W2 columns are staged once per
+// workgroup in LDS in MFMA fragment order (W0 in plain k order - it meets h2
+// as loaded from memory; W2 in the order in which the up-projection's
+// accumulator tiles pack into an operand: k = 4g..4g+3 then 16+4g..16+4g+3 for
+// lane group g), the up-projection runs on the matrix cores, bias + activation
+// + the single rounding to the 16-bit type happen in registers, and the
+// down-projection accumulates straight onto the residual.  The hidden
+// activation (R x F) never reaches memory.
+//
+// Rounding points follow the reference kernel (python/beat_arena_env/csrc/
+// fused_ffn.cu:42-59): fp32 accumulate in both GEMMs, hidden = act(S + b0)
+// rounded once, xo = round(x + (O + b2)), LayerNorm statistics on the ROUNDED
+// xo, ho rounded once.  A row's result depends only on that row and the
+// weights (fixed k order, no atomics), whatever R is.
+// Replaces fp16_gemm.ffn_fused (fused_ffn.cu:242-485, 551-619).
 #include "bsrl_common.h"
-extern "C" int bsrl_ffn_fused_supported(int64_t, int64_t, int) { return 0; }
-extern "C" int bsrl_ffn_fused(const void*, const void*, const void*, const float*, const void*, const float*,
-                              const float*, const float*, float, void*, void*, int64_t, int64_t, int64_t, int, int,
-                              bsrl_stream) { return BSRL_UNSUPPORTED; }
+
+namespace {
+
+struct FfnArgs {
+    const u16 *x, *h2, *w0, *w2;
+    const float *b0, *b2, *ln_w, *ln_b;
+    u16 *xo, *ho;
+    int64_t rows; int F; float eps;
+};
+
+template <typename DT> __device__ __forceinline__ uint32_t pk2(float a, float b) {
+    return (uint32_t)DT::from_f(a) | ((uint32_t)DT::from_f(b) << 16);
+}
+
+template <typename DT, int D, int RT, int ACT>
+__global__ __launch_bounds__(256) void ffn_fused_kernel(FfnArgs a) {
+    constexpr int NT = D / 16, KC = D / 32, NFR = 2 * KC + NT;
+    __shared__ uint4 wl[NFR * 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RT * 16);
+
+    f32x4 xa[RT][NT];
+    union { s16x8 v; uint4 u; uint32_t w[4]; } hf[RT][KC];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        int64_t row = row0 + rt * 16 + r16; row = row < a.rows ? row : a.rows - 1;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) hf[rt][c].u = *reinterpret_cast<const uint4*>(a.h2 + row * D + 32 * c + 8 * g);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint2 xv = *reinterpret_cast<const uint2*>(a.x + row * D + 16 * nt + 4 * g);
+            const float4 b = *reinterpret_cast<const float4*>(a.b2 + 16 * nt + 4 * g);
+            xa[rt][nt] = (f32x4){DT::to_f((u16)(xv.x & 0xffff)) + b.x, DT::to_f((u16)(xv.x >> 16)) + b.y,
+                                 DT::to_f((u16)(xv.y & 0xffff)) + b.z, DT::to_f((u16)(xv.y >> 16)) + b.w};
+        }
+    }
+    const int nch = a.F / 32;
+    for (int ch = 0; ch < nch; ++ch) {
+        __syncthreads();                       // the previous chunk's fragments are no longer read
+        for (int f = wave; f < NFR; f += 4) {
+            uint4 v;
+            if (f < 2 * KC) {
+                const int ntl = f / KC, c = f % KC;
+                v = *reinterpret_cast<const uint4*>(a.w0 + (int64_t)(32 * ch + 16 * ntl + r16) * D + 32 * c + 8 * g);
+            } else {
+                const u16* p = a.w2 + (int64_t)(16 * (f - 2 * KC) + r16) * a.F + 32 * ch + 4 * g;
+                const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 16);
+                v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
+            wl[f * 64 + lane] = v;
+        }
+        __syncthreads();
+        f32x4 acc[2][RT];
+#pragma unroll
+        for (int ntl = 0; ntl < 2; ++ntl) {
+            const float4 b = *reinterpret_cast<const float4*>(a.b0 + 32 * ch + 16 * ntl + 4 * g);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
+        }
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+            for (int ntl = 0; ntl < 2; ++ntl) {
+                const s16x8 w = __builtin_bit_cast(s16x8, wl[(ntl * KC + c) * 64 + lane]);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = DT::mfma32(w, hf[rt][c].v, acc[ntl][rt]);
+            }
+        union { s16x8 v; uint32_t w[4]; } hid[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int ntl = 0; ntl < 2; ++ntl) {
+                hid[rt].w[ntl * 2] = pk2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
+                hid[rt].w[ntl * 2 + 1] = pk2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
+            }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const s16x8 w = __builtin_bit_cast(s16x8, wl[(2 * KC + nt) * 64 + lane]);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) xa[rt][nt] = DT::mfma32(w, hid[rt].v, xa[rt][nt]);
+        }
+    }
+    // epilogue: round, store, optional LayerNorm on the rounded row
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int64_t row = row0 + rt * 16 + r16;
+        const bool live = row < a.rows;
+        float s = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint32_t lo = pk2<DT>(xa[rt][nt][0], xa[rt][nt][1]), hi = pk2<DT>(xa[rt][nt][2], xa[rt][nt][3]);
+            if (live) *reinterpret_cast<uint2*>(a.xo + row * D + 16 * nt + 4 * g) = make_uint2(lo, hi);
+            xa[rt][nt] = (f32x4){DT::to_f((u16)(lo & 0xffff)), DT::to_f((u16)(lo >> 16)),
+                                 DT::to_f((u16)(hi & 0xffff)), DT::to_f((u16)(hi >> 16))};
+            s += (xa[rt][nt][0] + xa[rt][nt][1]) + (xa[rt][nt][2] + xa[rt][nt][3]);
+        }
+        if (a.ho) {
+            s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
+            const float mean = s * (1.0f / D);
+            float q = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { const float t = xa[rt][nt][i] - mean; q = fmaf(t, t, q); }
+            q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
+            const float rstd = 1.0f / sqrtf(q * (1.0f / D) + a.eps);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 gm = *reinterpret_cast<const float4*>(a.ln_w + 16 * nt + 4 * g);
+                const float4 bt = *reinterpret_cast<const float4*>(a.ln_b + 16 * nt + 4 * g);
+                const uint32_t lo = pk2<DT>((xa[rt][nt][0] - mean) * rstd * gm.x + bt.x, (xa[rt][nt][1] - mean) * rstd * gm.y + bt.y);
+                const uint32_t hi = pk2<DT>((xa[rt][nt][2] - mean) * rstd * gm.z + bt.z, (xa[rt][nt][3] - mean) * rstd * gm.w + bt.w);
+                if (live) *reinterpret_cast<uint2*>(a.ho + row * D + 16 * nt + 4 * g) = make_uint2(lo, hi);
+            }
+        }
+    }
+}
+
+template <typename DT, int D, int RT>
+void launch(const FfnArgs& a, int act, hipStream_t st) {
+    const unsigned grid = (unsigned)((a.rows + 64 * RT - 1) / (64 * RT));
+    if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_RELU>), dim3(grid), dim3(256), 0, st, a);
+    else if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_GELU>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_NONE>), dim3(grid), dim3(256), 0, st, a);
+}
+
+template <typename DT>
+void dispatch(const FfnArgs& a, int64_t d, int act, hipStream_t st) {
+    if (d == 128) launch<DT, 128, 4>(a, act, st);
+    else if (d == 192) launch<DT, 192, 2>(a, act, st);
+    else if (d == 256) launch<DT, 256, 2>(a, act, st);
+    else launch<DT, 384, 1>(a, act, st);
+}
+
+}  // namespace
+
+extern "C" int bsrl_ffn_fused_supported(int64_t d, int64_t F, int dtype) {
+    return (d == 128 || d == 192 || d == 256 || d == 384) && F > 0 && F % 32 == 0 &&
+           (dtype == BSRL_F16 || dtype == BSRL_BF16);
+}
+
+extern "C" int bsrl_ffn_fused(const void* x, const void* h2, const void* w0, const float* b0, const void* w2,
+                              const float* b2, const float* ln_w, const float* ln_b, float eps, void* xo, void* ho,
+                              int64_t rows, int64_t d, int64_t F, int act, int dtype, bsrl_stream stream) {
+    if (!x || !h2 || !w0 || !b0 || !w2 || !b2 || !xo) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_fused: null pointer");
+    if ((ln_w == nullptr) != (ho == nullptr) || (ln_w == nullptr) != (ln_b == nullptr))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_fused: ln_w, ln_b and ho go together");
+    if (rows < 0 || d <= 0 || F <= 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_fused: bad shape");
+    if (act < 0 || act > 2) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_fused: bad act %d", act);
+    if (!bsrl_ffn_fused_supported(d, F, dtype)) return BSRL_UNSUPPORTED;
+    const void* ptrs[] = {x, h2, w0, w2, xo, ho, b0, b2, ln_w, ln_b};
+    for (const void* p : ptrs) if (p && !bsrl_aligned(p, 16)) return BSRL_UNSUPPORTED;
+    if (rows == 0) return BSRL_OK;
+    FfnArgs a{static_cast<const u16*>(x), static_cast<const u16*>(h2), static_cast<const u16*>(w0),
+              static_cast<const u16*>(w2), b0, b2, ln_w, ln_b, static_cast<u16*>(xo), static_cast<u16*>(ho),
+              rows, (int)F, eps};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == BSRL_F16) dispatch<F16>(a, d, act, st);
+    else dispatch<BF16>(a, d, act, st);
+    BSRL_CHECK_LAUNCH("bsrl_ffn_fused");
+    return BSRL_OK;
+}

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
             for (int e = 0; e < 4; ++e) {
                 const int c = col + e;
                 if (c >= a.M) break;
-                float o = apply_act<ACT>(acc[i][j][e] + bv[e]);
+                float o = a.out_f32 ? apply_act<ACT>(acc[i][j][e] + bv[e]) : apply_act16<ACT>(acc[i][j][e] + bv[e]);
                 if (res) o += DT::to_f(res[row * a.ldr + c]);
                 const bool second = a.y2 && c >= a.split;
                 void* dst = second ? a.y2 : a.y;
@@ -151,8 +151,9 @@ __global__ __launch_bounds__(256) void linear_mfma_vec_kernel(LinArgs a) {
         for (int j = 0; j < 4; ++j) {
             const int64_t row = row0 + j * 16 + r16;
             if (row >= a.rows) continue;
-            float o[4] = {apply_act<ACT>(acc[i][j][0] + bv.x), apply_act<ACT>(acc[i][j][1] + bv.y),
-                          apply_act<ACT>(acc[i][j][2] + bv.z), apply_act<ACT>(acc[i][j][3] + bv.w)};
+            float o[4] = {acc[i][j][0] + bv.x, acc[i][j][1] + bv.y, acc[i][j][2] + bv.z, acc[i][j][3] + bv.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = a.out_f32 ? apply_act<ACT>(o[e]) : apply_act16<ACT>(o[e]);
             if (res) {
                 uint2 rv = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
                 o[0] += DT::to_f((u16)(rv.x & 0xffff)); o[1] += DT::to_f((u16)(rv.x >> 16));

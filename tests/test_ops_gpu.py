@@ -151,6 +151,59 @@ def test_linear_rows_are_batch_invariant():
         assert torch.equal(ops.linear(x[lo:hi], w, b, act="gelu"), full[lo:hi])
 
 
+# ---------------------------------------------------------------- Fused FFN
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,d,Fh", [(1, 128, 512), (127, 128, 512), (129, 192, 768), (1000, 192, 768),
+                                       (300, 256, 1024), (77, 384, 1536), (513, 128, 64)])
+@pytest.mark.parametrize("act,with_ln", [("relu", True), ("gelu", False), ("gelu", True)])
+def test_ffn_fused(dtype, rows, d, Fh, act, with_ln):
+    """Closed form with the reference's rounding points (python/tests/test_fused_ffn.py:252-266):
+    hidden rounded once, fp32 accumulate, out = round(x + (O + b2)), LN on the rounded out."""
+    assert ops.ffn_fused_supported(d, Fh, dtype)
+    x = _rand(rows, d, dtype=dtype, seed=1)
+    h2 = _rand(rows, d, dtype=dtype, seed=2)
+    w0 = _rand(Fh, d, dtype=dtype, seed=3, scale=1 / math.sqrt(d))
+    w2 = _rand(d, Fh, dtype=dtype, seed=4, scale=1 / math.sqrt(Fh))
+    b0, b2 = _rand(Fh, seed=5) * 0.3, _rand(d, seed=6) * 0.3
+    lw, lb = (_rand(d, seed=7) * 0.2 + 1.0, _rand(d, seed=8) * 0.2) if with_ln else (None, None)
+    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act=act, ln_w=lw, ln_b=lb)
+    pre = h2.double() @ w0.double().t() + b0.double()
+    hid = (torch.relu(pre) if act == "relu" else 0.5 * pre * (1 + torch.erf(pre / math.sqrt(2.0)))).to(dtype).double()
+    ref = x.double() + hid @ w2.double().t() + b2.double()
+    scale = ref.abs().max().item()
+    # the hidden's rounding can flip one 16-bit ulp near ties: allow a little over one output ulp
+    assert (xo.double() - ref).abs().max().item() <= 1.5 * EPS16[dtype] * scale
+    # unfused path through the same library: error class no worse (reference idiom, test_fused_ffn.py:295-306)
+    un = ops.linear(ops.linear(h2, w0, b0, act=act), w2, b2, residual=x)
+    e_new = (xo.double() - ref).norm() / ref.norm()
+    e_old = (un.double() - ref).norm() / ref.norm()
+    assert e_new <= max(1.1 * e_old, 2e-3)
+    if with_ln:
+        ln_ref = F.layer_norm(xo.float(), (d,), lw, lb, 1e-5)
+        assert (ho.float() - ln_ref).abs().max().item() <= 2 * EPS16[dtype] * (ln_ref.abs().max().item() + 1)
+    else:
+        assert ho is None
+
+
+def test_ffn_fused_rows_are_batch_invariant():
+    d, Fh = 192, 768
+    x = _rand(400, d, dtype=torch.float16, seed=1)
+    h2 = _rand(400, d, dtype=torch.float16, seed=2)
+    w0 = _rand(Fh, d, dtype=torch.float16, seed=3, scale=0.07)
+    w2 = _rand(d, Fh, dtype=torch.float16, seed=4, scale=0.04)
+    b0, b2, lw, lb = _rand(Fh, seed=5), _rand(d, seed=6), _rand(d, seed=7) + 1, _rand(d, seed=8)
+    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb)
+    for lo, hi in ((0, 1), (3, 130), (127, 256), (271, 400)):
+        a, b = ops.ffn_fused(x[lo:hi].contiguous(), h2[lo:hi].contiguous(), w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb)
+        assert torch.equal(a, xo[lo:hi]) and torch.equal(b, ho[lo:hi])
+
+
+def test_ffn_fused_unsupported_shapes_say_so():
+    assert not ops.ffn_fused_supported(160, 640, torch.float16)
+    assert not ops.ffn_fused_supported(128, 500, torch.float16)
+    assert not ops.ffn_fused_supported(128, 512, torch.float32)
+
+
 # ---------------------------------------------------------------- Attention
 def _attn_ref(q, k, v, H, bias):
     B, TQ, d = q.shape
