@@ -1,0 +1,430 @@
+"""NotePolicy on the HIP kernels: a drop-in for the reference's policy module (forward).
+
+Same constructor arguments, parameter names / shapes / registration order (hence the
+same state_dict and checkpoints) and the same `forward_stacked(obs) -> (logits
+(B, 29, k_max) fp32, value (B,) fp32)` contract as the reference (python/policy.py:
+784-1097 ctor, :1179-1344 forward, :1346-1403 critic).  What runs where:
+
+  * on the C-ABI kernels: every Linear (token encoders, packed q|k|v, output
+    projections with the residual add in the epilogue, FFNs - fused with the next
+    block's LayerNorm when `fused_ffn` is on -, SimBa trunk, packed heads, critic
+    projections and MLP), every LayerNorm, every attention (blocks, the final block's
+    5 lead queries, the critic's single query);
+  * in torch on the GPU (data movement and O(B x 24) elementwise work): the obs lane
+    gathers, the 22 note-geometry lanes, token concatenation, the key-bias build, the
+    ragged-head scatter and the 101-bin value expectation.
+
+Stream dtype: `policy.fp16 = True` runs the 16-bit stream (fp16; set `stream_dtype =
+torch.bfloat16` for bf16) exactly as the reference's switch does (python/policy.py:
+1085-1090); otherwise fp32 kernels.  There is no CPU path and no torch fallback for
+the kernel ops.  Not implemented (raise at construction): value_residual, the simbav2
+trunk."""
+from __future__ import annotations
+
+import contextlib
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import fp16_linear as _fl
+from . import obs_layout as L
+from . import ops
+from .fused_ln import FusedLayerNorm
+
+OBS_DIM = L.OBS_DIM
+N_NOTE_SLOTS = L.N_NOTE_SLOTS
+NOTE_FEAT = L.NOTE_FEAT
+OFF_NOTES = L.OFF_NOTES
+OFF_NOTE_MASK = L.OFF_NOTE_MASK
+SABER_FEAT, TORSO_FEAT, LEG_FEAT = L.SABER_FEAT, L.TORSO_FEAT, L.LEG_FEAT
+NOTE_GEO_FEAT = L.NOTE_GEO_FEAT
+N_ACTION_HEADS = L.N_ACTION_HEADS
+MASK_BIAS = L.MASK_BIAS
+MASKED_LOGIT = L.MASKED_LOGIT
+TRUNK_ARCHS = ("simba", "simbav2")
+
+
+def _mlp(sizes, act=nn.ReLU):
+    layers = []
+    for i in range(len(sizes) - 1):
+        layers.append(nn.Linear(sizes[i], sizes[i + 1]))
+        if i < len(sizes) - 2:
+            layers.append(act())
+    return nn.Sequential(*layers)
+
+
+def _lin(m: nn.Linear, x, act=None, residual=None):
+    """A Linear on the kernels in x's dtype (fp32 master weights, 16-bit replica when needed)."""
+    return ops.linear(x, _fl._replica(m.weight, x.dtype), _fl._bias32(m.bias), act=act, residual=residual)
+
+
+def _seq(seq: nn.Sequential, x):
+    """Linear (ReLU Linear)* with each ReLU in its producer's epilogue (reference
+    python/policy.py:76-145, `_seq` / `_run`)."""
+    ms = list(seq)
+    i = 0
+    while i < len(ms):
+        m = ms[i]
+        if not isinstance(m, nn.Linear):
+            raise RuntimeError(f"unsupported module in Sequential: {type(m).__name__}")
+        relu = i + 1 < len(ms) and isinstance(ms[i + 1], nn.ReLU)
+        x = _lin(m, x, act="relu" if relu else None)
+        i += 2 if relu else 1
+    return x
+
+
+def note_geo(notes, sabers, z_asinh, flux, z_off):
+    """The 22 hand-relative geometry lanes per entity slot, fp32 (reference
+    python/policy.py:329-404): per hand [dp x, dp y (half-metres), asinh(dp z / 8),
+    asinh(|dp| / 8), seconds-to-plane / 3, v.d, b.d], then per hand the blade-frame
+    block [along, perp, cut (asinh(m / 2)), vt.d]."""
+    z_m = torch.sinh(notes[..., 2]) * float(z_asinh)
+    tx, ty = notes[..., 0], notes[..., 1]
+    if flux:
+        bar = notes[..., 9] > 0.5
+        tx, ty = torch.where(bar, notes[..., 12], tx), torch.where(bar, notes[..., 13], ty)
+    npos = torch.stack([tx * L.X_NORM, ty * L.Y_NORM, z_m], -1)
+    cutd = torch.stack([notes[..., 6], notes[..., 7], torch.zeros_like(tx)], -1)
+    not_wall = 1.0 - notes[..., 14:15]
+    speed = (-notes[..., 3:4] * L.Z_SCALE).clamp_min(1e-3)
+    tpl = ((z_m - (z_off * L.X_NORM)[:, None])[..., None] / speed).clamp(-0.5, 3.0) / 3.0
+    base, blade = [], []
+    for hand in range(2):
+        w = sabers[:, hand]
+        wpos = torch.stack([w[:, L.S_WPOS] * L.X_NORM, w[:, L.S_WPOS + 1] * L.Y_NORM, w[:, L.S_WPOS + 2]], -1)
+        dpm = npos - wpos[:, None]
+        dp = dpm * 0.5
+        dist = torch.asinh(dp.norm(dim=-1, keepdim=True) * 0.25)
+        dp = torch.cat([dp[..., :2], torch.asinh(dp[..., 2:3] * 0.25)], -1)
+        v = w[:, L.S_WVEL:L.S_WVEL + 3] * L.V_NORM
+        vhat = v / (v.norm(dim=-1, keepdim=True) + 0.05)
+        b = w[:, L.S_BLADE:L.S_BLADE + 3]
+        base += [dp, dist, tpl, (vhat[:, None] * cutd).sum(-1, keepdim=True) * not_wall,
+                 (b[:, None] * cutd).sum(-1, keepdim=True) * not_wall]
+        ab = (dpm * b[:, None]).sum(-1, keepdim=True)
+        vt = w[:, L.S_TIPV:L.S_TIPV + 3]
+        pn = torch.linalg.cross(b, vt * L.V_NORM)
+        nhat = pn / (pn.norm(dim=-1, keepdim=True) + 0.05)
+        blade += [torch.asinh((ab - L.HANDLE_LEN) * 0.5),
+                  torch.asinh((dpm - ab * b[:, None]).norm(dim=-1, keepdim=True) * 0.5),
+                  torch.asinh((dpm * nhat[:, None]).sum(-1, keepdim=True) * 0.5),
+                  (vt[:, None] * cutd).sum(-1, keepdim=True) * not_wall]
+    return torch.cat(base + blade, -1)
+
+
+class Block(nn.Module):
+    """Pre-LN transformer block; parameters as the reference's Block
+    (python/policy.py:492-522): ln_attn, q/k/v/out_proj, ln_ffn, ffn.{0,2}."""
+
+    def __init__(self, d: int, n_heads: int = 4, ffn_mult: int = 4):
+        super().__init__()
+        if n_heads < 2 or d % n_heads:
+            raise ValueError(f"embed {d} must split into >= 2 heads, got n_heads={n_heads}")
+        self.ln_attn = FusedLayerNorm(d)
+        self.q_proj = nn.Linear(d, d)
+        self.k_proj = nn.Linear(d, d)
+        self.v_proj = nn.Linear(d, d)
+        self.out_proj = nn.Linear(d, d)
+        self.ln_ffn = FusedLayerNorm(d)
+        self.ffn = _mlp([d, ffn_mult * d, d])
+        self.d, self.n_heads, self.dh = d, n_heads, d // n_heads
+
+    def forward(self, x, attn_bias, h=None, n_queries=0, next_ln=None):
+        """x (B, T, d); attn_bias (B, T) additive key bias; h = ln_attn(x) if the
+        previous block's fused FFN already produced it.  n_queries > 0 computes only
+        the first n_queries rows (keys / values still span all T): exact, masking is
+        key-side only (reference python/policy.py:533-539).  Returns (x_out, h_next)
+        with h_next = next_ln(x_out) when the fused FFN produced it, else None."""
+        d = self.d
+        if h is None:
+            h = self.ln_attn(x)
+        if n_queries:
+            wkv, bkv = _fl.packed_halves([self.k_proj, self.v_proj], x.dtype)
+            kv = ops.linear(h, wkv, bkv)                                   # (B, T, 2d)
+            hq = h[:, :n_queries]
+            q = _lin(self.q_proj, hq)                                      # (B, nq, d)
+            att = ops.attn_fwd(q, kv[..., :d], kv[..., d:], self.n_heads, key_bias=attn_bias)
+            x = x[:, :n_queries].contiguous()
+        else:
+            wqkv, bqkv = _fl.packed_halves([self.q_proj, self.k_proj, self.v_proj], x.dtype)
+            qkv = ops.linear(h, wqkv, bqkv)                                # (B, T, 3d)
+            att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, key_bias=attn_bias)
+        x = _lin(self.out_proj, att, residual=x)                           # x + out(att), one rounding
+        h2 = self.ln_ffn(x)
+        if _fl.fused_ffn_ok(x, self.ffn, next_ln):
+            r = _fl.fused_ffn(x, h2, self.ffn, next_ln)
+            return (r, None) if next_ln is None else r
+        hid = _lin(self.ffn[0], h2, act="relu")
+        return _lin(self.ffn[2], hid, residual=x), None
+
+
+def build_head_gears(n_gears: int) -> tuple:
+    """Per-joint gear counts of this build: uniform (the reference falls back to the
+    same when its env constants are not importable, python/policy.py:1555-1564)."""
+    return (n_gears,) * N_ACTION_HEADS
+
+
+class NotePolicy(nn.Module):
+    def __init__(self, embed: int = 128, trunk_dim: int = 256, encoder: str = "transformer", n_blocks: int = 3,
+                 n_heads: int = 4, n_gears: int = 3, ffn_mult: int = 4, note_geo: bool = False,
+                 value_bins: int = 101, value_vmax: float = 6.0, value_sigma: float = 0.75,
+                 trunk_hidden: int | None = None, z_asinh: float = 8.0, game: str = "standard",
+                 fp16_accum: str = "off", fused_ffn: str = "off", emb_ln: bool = False,
+                 value_residual: bool = False, final_ln: bool = False, trunk_arch: str = "simba",
+                 head_gears: tuple | list | None = None):
+        super().__init__()
+        if trunk_arch not in TRUNK_ARCHS:
+            raise ValueError(f"trunk_arch must be one of {TRUNK_ARCHS}, got {trunk_arch!r}")
+        if trunk_arch != "simba":
+            raise NotImplementedError("the simbav2 trunk is not built on the HIP kernels yet")
+        if value_residual:
+            raise NotImplementedError("value_residual is not built on the HIP kernels yet")
+        if game not in ("standard", "flux"):
+            raise ValueError(f"game must be 'standard' or 'flux', got {game!r}")
+        if not float(z_asinh) > 0:
+            raise ValueError(f"z_asinh must be > 0 (metres), got {z_asinh}")
+        if fp16_accum not in _fl.ACCUM_MODES:
+            raise ValueError(f"fp16_accum must be one of {_fl.ACCUM_MODES}, got {fp16_accum!r}")
+        if fused_ffn not in _fl.FFN_MODES:
+            raise ValueError(f"fused_ffn must be one of {_fl.FFN_MODES}, got {fused_ffn!r}")
+        if encoder != "transformer":
+            raise ValueError(f"unknown encoder: {encoder}")
+        if n_gears not in (3, 5, 7):
+            raise ValueError(f"n_gears must be 3/5/7, got {n_gears}")
+        if value_bins <= 1:
+            raise ValueError(f"value_bins must be > 1, got {value_bins}")
+        self.encoder, self.embed, self.n_heads, self.n_gears = encoder, embed, n_heads, n_gears
+        head_gears = tuple(int(k) for k in (head_gears if head_gears is not None else build_head_gears(n_gears)))
+        if len(head_gears) != N_ACTION_HEADS or not all(3 <= k <= 7 for k in head_gears):
+            raise ValueError(f"head_gears must be {N_ACTION_HEADS} counts in [3, 7], got {head_gears}")
+        self.head_sizes = head_gears
+        self.k_max = max(head_gears)
+        H = int(trunk_hidden) if trunk_hidden else trunk_dim
+        # arch record, key for key the reference's (python/policy.py:857-928)
+        self.arch = {"embed": embed, "trunk_dim": trunk_dim, "n_blocks": n_blocks, "n_heads": n_heads,
+                     "n_gears": n_gears, "obs_dim": OBS_DIM, "ffn_mult": ffn_mult, "critic": "adapool_v1",
+                     "n_action_heads": N_ACTION_HEADS, "body_token": True, "body_tokens": 3,
+                     "note_geo": bool(note_geo), "note_geo_norm": True, "blade_geo": 1, "z_asinh": float(z_asinh),
+                     "trunk_arch": trunk_arch, "trunk_hidden": H, "value_bins": int(value_bins),
+                     "value_vmax": float(value_vmax), "value_sigma": float(value_sigma), "game": game,
+                     "fp16_accum": fp16_accum, "fused_ffn": fused_ffn, "emb_ln": bool(emb_ln),
+                     "value_residual": False, "final_ln": bool(final_ln)}
+        if head_gears != (n_gears,) * N_ACTION_HEADS:
+            self.arch["head_gears"] = list(head_gears)
+        self.value_bins = int(value_bins)
+        self.value_sigma_bins = float(value_sigma)
+        centers = torch.linspace(-float(value_vmax), float(value_vmax), self.value_bins)
+        self.register_buffer("value_centers", centers, persistent=False)
+        self.value_sigma = float(value_sigma) * float(centers[1] - centers[0])
+        self.note_geo, self.z_asinh, self.game = bool(note_geo), float(z_asinh), game
+        # parameter registration order == the reference's (state_dict layout contract)
+        self.note_mlp = _mlp([NOTE_FEAT + (NOTE_GEO_FEAT if note_geo else 0), embed, embed])
+        self.saber_mlp = _mlp([SABER_FEAT + 2, embed, embed])
+        self.body_tokens, self.n_lead = 3, L.N_LEAD
+        self.torso_mlp = _mlp([TORSO_FEAT, embed, embed])
+        self.leg_mlp = _mlp([LEG_FEAT + 2, embed, embed])
+        self.value_residual = False
+        self.emb_ln = FusedLayerNorm(embed) if emb_ln else None
+        self.blocks = nn.ModuleList(Block(embed, n_heads, ffn_mult) for _ in range(n_blocks))
+        self.final_ln = FusedLayerNorm(embed) if final_ln else None
+        self.trunk_arch = trunk_arch
+        self.trunk_proj = nn.Linear(self.n_lead * embed, trunk_dim)
+        self.trunk_ln1 = FusedLayerNorm(trunk_dim)
+        self.trunk_fc1 = nn.Linear(trunk_dim, H)
+        self.trunk_fc2 = nn.Linear(H, trunk_dim)
+        self.trunk_ln2 = FusedLayerNorm(trunk_dim)
+        self.heads = nn.ModuleList(nn.Linear(trunk_dim, n) for n in self.head_sizes)
+        if min(self.head_sizes) < self.k_max:
+            self.register_buffer("_gear_valid", torch.tensor([[a < k for a in range(self.k_max)]
+                                                              for k in self.head_sizes]), persistent=False)
+            self.register_buffer("_gear_idx", torch.tensor([j * self.k_max + a for j, k in enumerate(self.head_sizes)
+                                                            for a in range(k)], dtype=torch.long), persistent=False)
+        else:
+            self._gear_valid = self._gear_idx = None
+        self.critic_ln = FusedLayerNorm(embed)
+        self.critic_q = nn.Linear(embed, embed)
+        self.critic_k = nn.Linear(embed, embed)
+        self.critic_v = nn.Linear(embed, embed)
+        self.critic_out = nn.Linear(embed, embed)
+        self.critic_mlp = _mlp([embed + trunk_dim, trunk_dim, trunk_dim, self.value_bins])
+        self.register_buffer("_saber_idx", torch.tensor(L.SABER_L_IDX + L.SABER_R_IDX, dtype=torch.long),
+                             persistent=False)
+        self.register_buffer("_body_idx", torch.tensor(L.BODY3_IDX, dtype=torch.long), persistent=False)
+        self.register_buffer("_hand_id", torch.eye(2), persistent=False)
+        self.fp16 = False                       # True: 16-bit stream (python/policy.py:1085-1090)
+        self.stream_dtype = torch.float16       # the 16-bit type used when fp16 is on
+        self.fp16_accum = fp16_accum
+        self.fused_ffn = fused_ffn
+        self.upgraded_from = None
+        self._value_logits = None
+        self._ent_h = None
+
+    # ---- weights ---------------------------------------------------------------------
+    def flatten_fp16(self):
+        """The reference repacks every master into one flat buffer here
+        (python/policy.py:1405-1423); this build keeps per-tensor replicas that are
+        recast in place per weights version, so only the replicas are (re)built."""
+        self.refresh_fp16_caches()
+
+    def refresh_fp16_caches(self):
+        """Force every 16-bit replica up to date for the current weights version
+        (python/policy.py:1448-1461): call after optimizer steps under a captured graph."""
+        if not self.fp16:
+            return
+        dt = self.stream_dtype
+        for m in self.modules():
+            if isinstance(m, nn.Linear):
+                _fl._replica(m.weight, dt)
+        for blk in self.blocks:
+            _fl.packed_halves([blk.q_proj, blk.k_proj, blk.v_proj], dt)
+            _fl.packed_halves([blk.k_proj, blk.v_proj], dt)
+        _fl.packed_halves([self.critic_k, self.critic_v], dt)
+        _fl.packed_halves(list(self.heads), dt)
+
+    def load_state_dict(self, *a, **k):
+        r = super().load_state_dict(*a, **k)
+        _fl.bump_weights_version()
+        return r
+
+    # ---- forward -----------------------------------------------------------------------
+    def _split(self, obs):
+        sabers = obs.index_select(1, self._saber_idx)
+        body = obs.index_select(1, self._body_idx)
+        notes = obs[:, OFF_NOTES:OFF_NOTE_MASK].reshape(-1, N_NOTE_SLOTS, NOTE_FEAT)
+        note_mask = obs[:, OFF_NOTE_MASK:OFF_NOTE_MASK + N_NOTE_SLOTS]
+        return sabers, body, notes, note_mask
+
+    @torch.no_grad()
+    def forward_stacked(self, obs):
+        """obs (B, 630) on the GPU -> logits (B, 29, k_max) fp32, value (B,) fp32."""
+        if not obs.is_cuda:
+            raise RuntimeError("NotePolicy.forward_stacked runs on the GPU only (no CPU path)")
+        if obs.dim() != 2 or obs.shape[1] != OBS_DIM:
+            raise RuntimeError(f"obs must be (B, {OBS_DIM}), got {tuple(obs.shape)}")
+        with contextlib.ExitStack() as modes:
+            if self.fp16 and self.fp16_accum != "off":
+                modes.enter_context(_fl.fp16_accum(self.fp16_accum))
+            if self.fp16 and self.fused_ffn != "off":
+                modes.enter_context(_fl.ffn_fusion(self.fused_ffn))
+            return self._forward_stacked(obs)
+
+    def _forward_stacked(self, obs):
+        dt = self.stream_dtype if self.fp16 else torch.float32
+        B, d = obs.shape[0], self.embed
+        obs = obs.to(dt)                       # the 16-bit stream consumes the ROUNDED obs (policy.py:1200-1209)
+        sabers, body, notes, note_mask = self._split(obs)
+        sab3 = sabers.reshape(B, 2, SABER_FEAT)
+        if self.note_geo:
+            geo = note_geo(notes.float(), sab3.float(), self.z_asinh, self.game == "flux", obs[:, L.OBS_HEAD_Z].float())
+            notes = torch.cat([notes, geo.to(dt)], dim=-1)                 # (B, 24, 40)
+        hand_id = self._hand_id.to(dt).expand(B, 2, 2)
+        tok_saber = _seq(self.saber_mlp, torch.cat([sab3, hand_id], dim=-1))
+        tok_torso = _seq(self.torso_mlp, body[:, :TORSO_FEAT].contiguous()).unsqueeze(1)
+        legs = torch.cat([body[:, TORSO_FEAT:].reshape(B, 2, LEG_FEAT), hand_id], dim=-1)
+        tok_leg = _seq(self.leg_mlp, legs)
+        tok_note = _seq(self.note_mlp, notes.contiguous())
+        x = torch.cat([tok_saber, tok_torso, tok_leg, tok_note], dim=1)   # (B, 29, d)
+        attn_bias = F.pad((note_mask - 1.0) * MASK_BIAS, (self.n_lead, 0)).contiguous()   # (B, 29)
+        if self.emb_ln is not None:
+            x = self.emb_ln(x)
+        h = None
+        nb = len(self.blocks)
+        for i in range(nb - 1):
+            x, h = self.blocks[i](x, attn_bias, h=h, next_ln=self.blocks[i + 1].ln_attn)
+        x_res = x                                                          # the stream entering the final block
+        lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead)
+        if self.final_ln is not None:
+            lead = self.final_ln(lead)
+        hfeat = self._trunk(lead.reshape(B, self.n_lead * d))
+        wh, bh = _fl.packed_halves(list(self.heads), dt)
+        out = ops.linear(hfeat, wh, bh, out_dtype=torch.float32)           # (B, sum n_j) fp32
+        value = self._critic(x_res, hfeat, attn_bias)
+        if self._gear_idx is not None:
+            out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
+        return out.view(B, N_ACTION_HEADS, self.k_max), value
+
+    def _trunk(self, x):
+        """SimBa readout: proj -> LN1 -> fc1 -> ReLU -> fc2 -> (+proj) -> LN2 (policy.py:1107-1138)."""
+        t = _lin(self.trunk_proj, x)
+        u = self.trunk_ln1(t)
+        r = _lin(self.trunk_fc1, u, act="relu")
+        return self.trunk_ln2(_lin(self.trunk_fc2, r, residual=t))
+
+    def _critic(self, x_res, hfeat, attn_bias):
+        """adapool_v1 value path (policy.py:1346-1403): LN -> query from the torso token ->
+        packed k|v -> 1-query attention pool -> out -> MLP -> HL-Gauss expectation."""
+        B, T, d = x_res.shape
+        hv = self.critic_ln(x_res)
+        q = _lin(self.critic_q, hv[:, 2:3])                                # (B, 1, d)
+        wkv, bkv = _fl.packed_halves([self.critic_k, self.critic_v], x_res.dtype)
+        kv = ops.linear(hv, wkv, bkv)
+        a = ops.attn_fwd(q, kv[..., :d], kv[..., d:], self.n_heads, key_bias=attn_bias).view(B, d)
+        a = _lin(self.critic_out, a)
+        z = torch.cat([a, hfeat], dim=-1)
+        z = _lin(self.critic_mlp[0], z, act="relu")
+        z = _lin(self.critic_mlp[2], z, act="relu")
+        m = self.critic_mlp[4]
+        logits = ops.linear(z, _fl._replica(m.weight, z.dtype), _fl._bias32(m.bias), out_dtype=torch.float32)
+        self._value_logits = None
+        return torch.softmax(logits, dim=-1) @ self.value_centers
+
+    def forward(self, obs):
+        logits, value = self.forward_stacked(obs)
+        return list(logits.unbind(1)), value
+
+    @torch.no_grad()
+    def get_action_and_value(self, obs, action=None, need_entropy=True):
+        """log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) on the
+        kernel forward's logits (reference python/policy.py:1467-1516); this epilogue is
+        plain torch on the (B, 29, K) fp32 logits."""
+        logits, value = self.forward_stacked(obs)
+        logsm = torch.log_softmax(logits, dim=-1)
+        if action is None:
+            score = logsm - torch.empty_like(logsm).exponential_().log()
+            if self._gear_valid is not None:
+                score = score.masked_fill(~self._gear_valid, -math.inf)
+            action = score.argmax(-1)
+        elif action.dtype is not torch.long:
+            action = action.long()
+        logprob = logsm.gather(-1, action.unsqueeze(-1)).squeeze(-1).sum(-1)
+        entropy = None
+        if need_entropy:
+            ent_h = -(logsm.exp() * logsm).sum(-1)
+            self._ent_h = ent_h
+            entropy = ent_h.sum(-1)
+        return action, logprob, entropy, value
+
+
+def load_policy(ckpt, game: str = "standard") -> NotePolicy:
+    """Rebuild a NotePolicy from a checkpoint dict {"arch", "state_dict"} written by the
+    reference trainer (python/policy.py:1589-1696); refuses the same stale layouts."""
+    arch = ckpt.get("arch", {})
+    if arch.get("blade_geo", 0) != 1:
+        raise SystemExit("only obs-630 (blade_geo 1) checkpoints are supported by this build")
+    if arch.get("game", "standard") != game:
+        raise SystemExit(f"checkpoint plays game {arch.get('game', 'standard')!r} but this tool plays {game!r}")
+    if (arch.get("body_tokens", 1) != 3 or arch.get("obs_dim") != OBS_DIM
+            or arch.get("n_action_heads") != N_ACTION_HEADS or "ffn_mult" not in arch
+            or not arch.get("body_token", False)):
+        raise SystemExit(f"checkpoint is not the obs-{OBS_DIM} / 29-head / 3-body-token layout: {dict(arch)}")
+    z_asinh = arch.get("z_asinh")
+    if z_asinh is None or not float(z_asinh) > 0:
+        raise SystemExit(f"checkpoint arch has z_asinh {z_asinh!r}")
+    if arch.get("note_geo", False) and not arch.get("note_geo_norm", False):
+        raise SystemExit("checkpoint has the raw-metre note-geo lanes (no note_geo_norm marker)")
+    if arch.get("dwa"):
+        raise ValueError("checkpoint uses --dwa, which no code path can rebuild")
+    policy = NotePolicy(
+        embed=arch["embed"], trunk_dim=arch["trunk_dim"], n_blocks=arch["n_blocks"], n_heads=arch["n_heads"],
+        n_gears=arch["n_gears"], ffn_mult=arch["ffn_mult"], note_geo=arch.get("note_geo", False),
+        trunk_hidden=arch.get("trunk_hidden"), value_bins=arch["value_bins"],
+        value_vmax=arch.get("value_vmax", 6.0), value_sigma=arch.get("value_sigma", 0.75),
+        z_asinh=float(z_asinh), game=game, fp16_accum=arch.get("fp16_accum", "off"),
+        fused_ffn=arch.get("fused_ffn", "off"), emb_ln=arch.get("emb_ln", False),
+        value_residual=arch.get("value_residual", False), final_ln=arch.get("final_ln", False),
+        trunk_arch=arch.get("trunk_arch", "simba"),
+        head_gears=(arch.get("head_gears") or (arch["n_gears"],) * N_ACTION_HEADS))
+    policy.load_state_dict(ckpt["state_dict"])
+    return policy

@@ -1,0 +1,150 @@
+"""GPU parity of the NotePolicy drop-in (every kernel through the C ABI):
+  * fp32 kernels against the golden vectors the REFERENCE's own module produced
+    (tests/golden/notepolicy_*.npz) - 1e-5 relative;
+  * the 16-bit stream at production-like shapes against the CPU oracle (itself pinned on
+    those vectors), with the class-relative gates of tests/test_config_policy_gpu.py, plus
+    the reference's own fp16-vs-fp32 bar: logits within 2e-2 of max|logit|
+    (python/tests/test_trunk_simba.py:142-162)."""
+import glob
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from beatsaberrl_amd import fp16_linear as fl  # noqa: E402
+from beatsaberrl_amd.policy import NotePolicy, load_policy  # noqa: E402
+from oracle import note_policy_ref as nr  # noqa: E402
+
+DEV = "cuda"
+GOLD = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "notepolicy_*.npz")))
+
+
+def _make_obs(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    obs = torch.randn(n, nr.OBS_DIM, generator=g) * 0.7
+    obs[:, nr.OFF_MASK:nr.OFF_MASK + 24] = (torch.rand(n, 24, generator=g) < 0.6).float()
+    obs[0, nr.OFF_MASK:nr.OFF_MASK + 24] = 0.0
+    notes = obs[:, nr.OFF_NOTES:nr.OFF_MASK].view(n, 24, 18)
+    notes[..., 14] = (torch.rand(n, 24, generator=g) < 0.3).float()
+    return obs
+
+
+@pytest.mark.parametrize("path", GOLD, ids=[os.path.basename(p)[:-4] for p in GOLD])
+def test_fp32_matches_reference_golden_vectors(path):
+    arch, sd, obs, logits, value = nr.load_fixture(path)
+    m = load_policy({"arch": arch, "state_dict": sd}, game=arch["game"]).to(DEV)
+    lg, v = m.forward_stacked(obs.to(DEV))
+    lg, v = lg.cpu(), v.cpu()
+    assert lg.shape == logits.shape and lg.dtype is torch.float32
+    live = logits > -1e8
+    assert torch.equal(lg[~live], logits[~live])
+    scale = logits[live].abs().max().item()
+    assert bool(((lg[live] - logits[live]).abs() <= 1e-5 * (logits[live].abs() + scale)).all()), \
+        (lg[live] - logits[live]).abs().max().item()
+    assert bool(((v - value).abs() <= 1e-5 * (value.abs() + value.abs().max())).all())
+    lst, v2 = m(obs.to(DEV))
+    assert len(lst) == 29 and torch.equal(lst[3].cpu(), lg[:, 3])
+
+
+@pytest.mark.parametrize("path", GOLD[:2], ids=[os.path.basename(p)[:-4] for p in GOLD[:2]])
+def test_fp16_stream_on_golden_vectors(path):
+    arch, sd, obs, logits, value = nr.load_fixture(path)
+    m = load_policy({"arch": arch, "state_dict": sd}, game=arch["game"]).to(DEV)
+    m.fp16 = True
+    lg, v = m.forward_stacked(obs.to(DEV))
+    live = logits > -1e8
+    assert (lg.cpu()[live] - logits[live]).abs().max().item() <= 2e-2 * logits[live].abs().max().item()
+    assert (v.cpu() - value).abs().max().item() <= 2e-2 * 6.0
+
+
+def _big(seed, **kw):
+    torch.manual_seed(seed)
+    m = NotePolicy(**kw)
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.dim() == 1:
+                p.add_(0.1 * torch.randn_like(p))
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    return m, sd
+
+
+@pytest.mark.parametrize("kw,dtype,ffn", [
+    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "on"),
+    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "off"),
+    (dict(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4), "f16", "on"),
+    (dict(embed=128, trunk_dim=256, n_blocks=2, n_heads=4, n_gears=7, ffn_mult=2, emb_ln=True, final_ln=True,
+          note_geo=True, head_gears=tuple(7 if j in (8, 15) else 5 for j in range(29))), "bf16", "on"),
+    (dict(embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f32", "off"),
+])
+def test_production_shapes_against_the_oracle(kw, dtype, ffn):
+    m, sd = _big(5, **kw)
+    m = m.to(DEV)
+    obs = _make_obs(96, 7)
+    ref_lg, ref_v = nr.forward(sd, m.arch, obs)
+    live = ref_lg > -1e8
+    if dtype == "f32":
+        lg, v = m.forward_stacked(obs.to(DEV))
+        lg, v = lg.cpu(), v.cpu()
+        scale = ref_lg[live].abs().max().item()
+        assert bool(((lg[live] - ref_lg[live]).abs() <= 1e-5 * (ref_lg[live].abs() + scale)).all())
+        assert (v - ref_v).abs().max().item() <= 1e-5 * (ref_v.abs().max().item() + 1)
+        return
+    m.fp16 = True
+    m.stream_dtype = torch.float16 if dtype == "f16" else torch.bfloat16
+    m.fused_ffn = ffn
+    lg, v = m.forward_stacked(obs.to(DEV))
+    lg, v = lg.cpu(), v.cpu()
+    em_lg, em_v = nr.forward(sd, m.arch, obs, emulate=dtype)
+    e_mine = (lg[live] - ref_lg[live]).abs().max().item()
+    e_emul = (em_lg[live] - ref_lg[live]).abs().max().item()
+    e_class = (lg[live] - em_lg[live]).abs().max().item()
+    print(f"\n[{dtype} ffn={ffn}] mine-vs-fp32 {e_mine:.2e}  emulated-vs-fp32 {e_emul:.2e}  mine-vs-emulated {e_class:.2e}")
+    assert torch.equal(lg[~live], ref_lg[~live])
+    assert e_mine <= max(1.25 * e_emul, 2e-3) and e_class <= max(e_emul, 2e-3)
+    assert (v - ref_v).abs().max().item() <= max(1.25 * (em_v - ref_v).abs().max().item(), e_emul, 2e-3)
+    if dtype == "f16":
+        assert e_mine <= 2e-2 * ref_lg[live].abs().max().item()      # the reference's own fp16 bar
+        top = ref_lg.topk(2, -1).values
+        decided = (top[..., 0] - top[..., 1]) > 1e-2
+        assert bool(((lg.argmax(-1) == ref_lg.argmax(-1)) | ~decided).all())
+
+
+def test_invariants_and_sampling_epilogue():
+    m, sd = _big(9, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,
+                 head_gears=tuple(7 if j == 4 else 5 for j in range(29)))
+    m = m.to(DEV)
+    m.fp16, m.fused_ffn = True, "on"
+    obs = _make_obs(50, 3)
+    od = obs.to(DEV)
+    lg, v = m.forward_stacked(od)
+    # junk in masked entity slots changes nothing (python/tests/test_policy.py:42-63)
+    obs2 = obs.clone()
+    mask = obs[:, nr.OFF_MASK:nr.OFF_MASK + 24] > 0.5
+    notes = obs2[:, nr.OFF_NOTES:nr.OFF_MASK].view(-1, 24, 18)
+    notes[~mask] = 5.0
+    lg2, v2 = m.forward_stacked(obs2.to(DEV))
+    assert torch.equal(lg, lg2) and torch.equal(v, v2)
+    # batch invariance: an env's bits do not depend on its neighbours
+    lg3, v3 = m.forward_stacked(od[7:23].contiguous())
+    assert torch.equal(lg3, lg[7:23]) and torch.equal(v3, v[7:23])
+    # fp32 obs and pre-rounded fp16 obs give the same bits (python/policy.py:1200-1209)
+    lg4, _ = m.forward_stacked(od.half())
+    assert torch.equal(lg4, lg)
+    # replicas refresh on a version bump
+    with torch.no_grad():
+        m.heads[0].weight.zero_()
+    assert torch.equal(m.forward_stacked(od)[0], lg)
+    fl.bump_weights_version()
+    lg5, _ = m.forward_stacked(od)
+    assert torch.allclose(lg5[:, 0, :5], m.heads[0].bias.expand(50, 5), atol=1e-6)
+    # sampling epilogue: valid gears only, log-prob consistent with the logits
+    torch.manual_seed(0)
+    act, logp, ent, val = m.get_action_and_value(od)
+    assert act.shape == (50, 29) and int(act[:, 4].max()) <= 6 and int(act[:, :4].max()) <= 4
+    lsm = torch.log_softmax(lg5, -1)
+    assert torch.allclose(logp, lsm.gather(-1, act.unsqueeze(-1)).squeeze(-1).sum(-1), atol=1e-5)
+    assert bool((ent > 0).all()) and torch.equal(val, m.forward_stacked(od)[1])
+    _, logp2, _, _ = m.get_action_and_value(od, action=act.to(torch.uint8), need_entropy=False)
+    assert torch.allclose(logp2, logp)
