@@ -272,70 +272,140 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             }
             norm_to_frags(lv + LV_LN2G, lv + LV_LN2B, true, hf);
             add_bias(lv + lv_b2(a.F));
-            // Software-pipelined over 32-wide hidden chunks: the up-projection MFMAs of chunk ch+1
-            // are issued next to the activation (VALU) of chunk ch, then the down-projection of
-            // chunk ch runs.  Stage order in the image: W1(0), {W1(ch+1), W2(ch)}..., W2(last).
+            // Software-pipelined over 32-wide hidden chunks.  MFMA and VALU work only overlap when they
+            // alternate finely inside one wave (measured on gfx950: 2 waves per SIMD running an MFMA
+            // phase and a VALU phase side by side take the SUM of the two), so every phase pairs 8*RT
+            // MFMAs with half a chunk of activation work, pinned two MFMAs + one activation at a time:
+            //   phase 1 (stage W1(ch+1)): up-projection of chunk ch+1  ||  activation of chunk ch, upper row tiles
+            //   phase 2 (stage W2(ch))  : down-projection of chunk ch  ||  activation of chunk ch+1, lower row tiles
+            // Stage order in the image: W1(0), {W1(ch+1), W2(ch)}..., W2(last).
             const int nch = a.F / 32;
+            constexpr int RH = RT / 2;                  // row tiles per activation half (RT == 1: no split)
             f32x4 accA[2][RT];
-            auto ffn_up = [&](const s16x8 (&w1)[STAGE_FRAGS], int ch, f32x4 (&acc)[2][RT]) {
+            Frag8 hidA[RT];                             // activation of the current chunk, as operand fragments
+            auto up_init = [&](int ch, f32x4 (&acc)[2][RT]) {
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
                     const float4 b = *reinterpret_cast<const float4*>(lv + LV_B1 + 32 * ch + 16 * ntl + 4 * g);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = (f32x4){b.x, b.y, b.z, b.w};
                 }
+            };
+            // activation of one (row tile, n-tile) accumulator = 4 hidden units -> 2 packed dwords
+            auto act4 = [&](const f32x4& v, Frag8& dst, int ntl) {
+                dst.w[ntl * 2] = pack2<DT>(apply_act16<ACT>(v[0]), apply_act16<ACT>(v[1]));
+                dst.w[ntl * 2 + 1] = pack2<DT>(apply_act16<ACT>(v[2]), apply_act16<ACT>(v[3]));
+            };
+            if (RT == 1) {
+                // single row tile (TAIL launch): plain chunk loop, no split
+                {
+                    ADVANCE(0);
+                    LOAD_STAGE(0, w1);
+                    up_init(0, accA);
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
+                }
+                for (int ch = 0; ch < nch; ++ch) {
+                    act4(accA[0][0], hidA[0], 0); act4(accA[1][0], hidA[0], 1);
+                    if (ch + 1 < nch) {
+                        ADVANCE(1);
+                        LOAD_STAGE(1, w1);
+                        up_init(ch + 1, accA);
+#pragma unroll
+                        for (int c = 0; c < KC; ++c)
+#pragma unroll
+                            for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
+                        ADVANCE(0);
+                    } else {
+                        ADVANCE(1);
+                    }
+                    s16x8 w2[STAGE_FRAGS];
+                    if (ch + 1 < nch) {
+#pragma unroll
+                        for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(0, f);
+                    } else {
+#pragma unroll
+                        for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(1, f);
+                    }
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
+                }
+            } else {
+                {   // prologue: up-projection of chunk 0, activation of its lower row tiles
+                    ADVANCE(0);
+                    LOAD_STAGE(0, w1);
+                    up_init(0, accA);
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) accA[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, accA[ntl][rt]);
+#pragma unroll
+                    for (int rt = 0; rt < RH; ++rt) { act4(accA[0][rt], hidA[rt], 0); act4(accA[1][rt], hidA[rt], 1); }
+                }
+                for (int ch = 0; ch < nch - 1; ++ch) {
+                    f32x4 accB[2][RT];
+                    Frag8 hidB[RT];
+                    float ga[RH > 0 ? RH : 1][8];       // activations of the half in flight, fp32 until packed
+                    {   // phase 1
+                        ADVANCE(1);
+                        LOAD_STAGE(1, w1);
+                        up_init(ch + 1, accB);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int c = 0; c < KC; ++c)
+#pragma unroll
+                            for (int ntl = 0; ntl < 2; ++ntl) {
+#pragma unroll
+                                for (int rt = 0; rt < RT; ++rt) accB[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, accB[ntl][rt]);
+                                // slice sl = (c, ntl): one hidden unit per upper row tile, element (sl >> 2, sl & 3)
+                                const int sl = c * 2 + ntl;                    // 0..7
+#pragma unroll
+                                for (int rt = 0; rt < RH; ++rt) ga[rt][sl] = apply_act16<ACT>(accA[sl >> 2][RH + rt][sl & 3]);
+                                __builtin_amdgcn_sched_barrier(0);
+                            }
+#pragma unroll
+                        for (int rt = 0; rt < RH; ++rt)
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) hidA[RH + rt].w[w] = pack2<DT>(ga[rt][2 * w], ga[rt][2 * w + 1]);
+                    }
+                    {   // phase 2
+                        ADVANCE(0);
+                        LOAD_STAGE(0, w2);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w2[nt], hidA[rt].v, x[rt][nt]);
+#pragma unroll
+                            for (int rt = 0; rt < RH; ++rt) ga[rt][nt] = apply_act16<ACT>(accB[nt >> 2][rt][nt & 3]);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+#pragma unroll
+                        for (int rt = 0; rt < RH; ++rt)
+#pragma unroll
+                            for (int w = 0; w < 4; ++w) hidB[rt].w[w] = pack2<DT>(ga[rt][2 * w], ga[rt][2 * w + 1]);
+                    }
 #pragma unroll
                     for (int ntl = 0; ntl < 2; ++ntl)
 #pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) acc[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, acc[ntl][rt]);
-            };
-            auto ffn_act = [&](const f32x4 (&acc)[2][RT], Frag8 (&hid)[RT]) {
+                        for (int rt = 0; rt < RT; ++rt) accA[ntl][rt] = accB[ntl][rt];
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
+                    for (int rt = 0; rt < RH; ++rt) hidA[rt] = hidB[rt];
+                }
+                {   // epilogue: last chunk's upper-half activation, then its down-projection
 #pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        hid[rt].w[ntl * 2] = pack2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
-                        hid[rt].w[ntl * 2 + 1] = pack2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
-                    }
-            };
-            auto ffn_down = [&](const s16x8 (&w2)[STAGE_FRAGS], const Frag8 (&hid)[RT]) {
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w2[nt], hid[rt].v, x[rt][nt]);
-            };
-            {
-                ADVANCE(0);
-                LOAD_STAGE(0, w1);
-                ffn_up(w1, 0, accA);
-            }
-            for (int ch = 0; ch < nch - 1; ++ch) {
-                Frag8 hid[RT];
-                f32x4 accB[2][RT];
-                {
+                    for (int rt = RH; rt < RT; ++rt) { act4(accA[0][rt], hidA[rt], 0); act4(accA[1][rt], hidA[rt], 1); }
                     ADVANCE(1);
-                    LOAD_STAGE(1, w1);
-                    ffn_up(w1, ch + 1, accB);
-                    ffn_act(accA, hid);
-                }
-                {
-                    ADVANCE(0);
-                    LOAD_STAGE(0, w2);
-                    ffn_down(w2, hid);
-                }
+                    LOAD_STAGE(1, w2);
 #pragma unroll
-                for (int ntl = 0; ntl < 2; ++ntl)
+                    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) accA[ntl][rt] = accB[ntl][rt];
-            }
-            {
-                Frag8 hid[RT];
-                ffn_act(accA, hid);
-                ADVANCE(1);
-                LOAD_STAGE(1, w2);
-                ffn_down(w2, hid);
+                        for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w2[nt], hidA[rt].v, x[rt][nt]);
+                }
             }
         };
 
