@@ -234,7 +234,7 @@ class ConfigPolicy(nn.Module):
             x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                           # x + out(att)
             h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)
             fused = None
-            if dt is not torch.float32 and ops.ffn_fused_supported(d, self.ffn_dim, dt):
+            if dt is not torch.float32 and ops.ffn_fused_profitable(d, self.ffn_dim, dt):
                 fused = ops.ffn_fused(x, h2, w["w0"], w["b0"], w["w2"], w["b2"], act=self.act)
             if fused is not None:
                 x = fused[0]

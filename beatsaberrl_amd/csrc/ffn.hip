@@ -4,7 +4,9 @@
 // of the fp32 output accumulator (residual + b2 folded in) and its h2 operand
 // fragments in registers for the whole kernel.  The hidden layer is walked in
 // chunks of 32 units: the chunk's W0 rows and W2 columns are staged once per
-// workgroup in LDS in MFMA fragment order (W0 in plain k order - it meets h2
+// workgroup in LDS (two buffers; the next chunk is loaded into registers one
+// chunk ahead and parked while the current one is consumed, one barrier per
+// chunk) in MFMA fragment order (W0 in plain k order - it meets h2
 // as loaded from memory; W2 in the order in which the up-projection's
 // accumulator tiles pack into an operand: k = 4g..4g+3 then 16+4g..16+4g+3 for
 // lane group g), the up-projection runs on the matrix cores, bias + activation
@@ -34,12 +36,42 @@ template <typename DT> __device__ __forceinline__ uint32_t pk2(float a, float b)
 }
 
 template <typename DT, int D, int RT, int ACT>
-__global__ __launch_bounds__(256) void ffn_fused_kernel(FfnArgs a) {
+__global__ __launch_bounds__(256, (RT * D <= 384) ? 2 : 1) void ffn_fused_kernel(FfnArgs a) {
     constexpr int NT = D / 16, KC = D / 32, NFR = 2 * KC + NT;
-    __shared__ uint4 wl[NFR * 64];
+    constexpr int PER = (NFR + 3) / 4;             // fragments each wave stages per chunk
+    extern __shared__ uint4 wl_all[];              // 2 x NFR fragments: chunk ch lives in buffer ch & 1
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RT * 16);
+
+    // one chunk's weight fragments, straight from the nn.Linear layouts: W0 rows in plain k order,
+    // W2 columns in the accumulator-pack order (4g..4g+3, 16+4g..16+4g+3)
+    uint4 pre[PER];
+    auto gload = [&](int ch) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = wave + 4 * i;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (f < 2 * KC) {
+                const int ntl = f / KC, c = f % KC;
+                v = *reinterpret_cast<const uint4*>(a.w0 + (int64_t)(32 * ch + 16 * ntl + r16) * D + 32 * c + 8 * g);
+            } else if (f < NFR) {
+                const u16* p = a.w2 + (int64_t)(16 * (f - 2 * KC) + r16) * a.F + 32 * ch + 4 * g;
+                const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 16);
+                v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
+            pre[i] = v;
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = wave + 4 * i;
+            if (f < NFR) wl_all[(buf * NFR + f) * 64 + lane] = pre[i];
+        }
+    };
+    const int nch = a.F / 32;
+    gload(0);
 
     f32x4 xa[RT][NT];
     union { s16x8 v; uint4 u; uint32_t w[4]; } hf[RT][KC];
@@ -56,22 +88,15 @@ __global__ __launch_bounds__(256) void ffn_fused_kernel(FfnArgs a) {
                                  DT::to_f((u16)(xv.y & 0xffff)) + b.z, DT::to_f((u16)(xv.y >> 16)) + b.w};
         }
     }
-    const int nch = a.F / 32;
+    lstore(0);
+    if (nch > 1) gload(1);
     for (int ch = 0; ch < nch; ++ch) {
-        __syncthreads();                       // the previous chunk's fragments are no longer read
-        for (int f = wave; f < NFR; f += 4) {
-            uint4 v;
-            if (f < 2 * KC) {
-                const int ntl = f / KC, c = f % KC;
-                v = *reinterpret_cast<const uint4*>(a.w0 + (int64_t)(32 * ch + 16 * ntl + r16) * D + 32 * c + 8 * g);
-            } else {
-                const u16* p = a.w2 + (int64_t)(16 * (f - 2 * KC) + r16) * a.F + 32 * ch + 4 * g;
-                const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 16);
-                v = make_uint4(lo.x, lo.y, hi.x, hi.y);
-            }
-            wl[f * 64 + lane] = v;
+        const uint4* wl = wl_all + (ch & 1) * NFR * 64;
+        __syncthreads();        // chunk ch is complete in buffer ch & 1; buffer (ch + 1) & 1 is no longer read
+        if (ch + 1 < nch) {
+            lstore((ch + 1) & 1);                  // chunk ch + 1 (loaded one chunk ago) -> the free buffer
+            if (ch + 2 < nch) gload(ch + 2);       // in flight during this chunk's MFMAs
         }
-        __syncthreads();
         f32x4 acc[2][RT];
 #pragma unroll
         for (int ntl = 0; ntl < 2; ++ntl) {
@@ -138,20 +163,30 @@ __global__ __launch_bounds__(256) void ffn_fused_kernel(FfnArgs a) {
     }
 }
 
-template <typename DT, int D, int RT>
-void launch(const FfnArgs& a, int act, hipStream_t st) {
+template <typename DT, int D, int RT, int ACT>
+bool launch_act(const FfnArgs& a, hipStream_t st) {
+    constexpr size_t lds = 2 * (size_t)(D / 8) * 64 * sizeof(uint4);       // two chunk buffers
+    auto kern = ffn_fused_kernel<DT, D, RT, ACT>;
+    if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return false;
     const unsigned grid = (unsigned)((a.rows + 64 * RT - 1) / (64 * RT));
-    if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_RELU>), dim3(grid), dim3(256), 0, st, a);
-    else if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_GELU>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((ffn_fused_kernel<DT, D, RT, BSRL_ACT_NONE>), dim3(grid), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+    return true;
+}
+template <typename DT, int D, int RT>
+bool launch(const FfnArgs& a, int act, hipStream_t st) {
+    if (act == BSRL_ACT_RELU) return launch_act<DT, D, RT, BSRL_ACT_RELU>(a, st);
+    if (act == BSRL_ACT_GELU) return launch_act<DT, D, RT, BSRL_ACT_GELU>(a, st);
+    return launch_act<DT, D, RT, BSRL_ACT_NONE>(a, st);
 }
 
 template <typename DT>
-void dispatch(const FfnArgs& a, int64_t d, int act, hipStream_t st) {
-    if (d == 128) launch<DT, 128, 4>(a, act, st);
-    else if (d == 192) launch<DT, 192, 2>(a, act, st);
-    else if (d == 256) launch<DT, 256, 2>(a, act, st);
-    else launch<DT, 384, 1>(a, act, st);
+bool dispatch(const FfnArgs& a, int64_t d, int act, hipStream_t st) {
+    if (d == 128) return launch<DT, 128, 2>(a, act, st);
+    if (d == 192) return launch<DT, 192, 2>(a, act, st);
+    if (d == 256) return launch<DT, 256, 2>(a, act, st);
+    return launch<DT, 384, 1>(a, act, st);
 }
 
 }  // namespace
@@ -177,8 +212,8 @@ extern "C" int bsrl_ffn_fused(const void* x, const void* h2, const void* w0, con
               static_cast<const u16*>(w2), b0, b2, ln_w, ln_b, static_cast<u16*>(xo), static_cast<u16*>(ho),
               rows, (int)F, eps};
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == BSRL_F16) dispatch<F16>(a, d, act, st);
-    else dispatch<BF16>(a, d, act, st);
+    const bool ok = dtype == BSRL_F16 ? dispatch<F16>(a, d, act, st) : dispatch<BF16>(a, d, act, st);
+    if (!ok) return BSRL_UNSUPPORTED;
     BSRL_CHECK_LAUNCH("bsrl_ffn_fused");
     return BSRL_OK;
 }

@@ -16,20 +16,9 @@
 // Replaces the vendor GEMM calls of the reference's op layer
 // (python/fp16_linear.py:134-181) and the bias+ReLU epilogues of
 // python/beat_arena_env/csrc/fp16_gemm.cu:77-111, 404-497.
-#include "bsrl_common.h"
+#include "linear_args.h"
 
 namespace {
-
-struct LinArgs {
-    const void* x; int64_t ldx;
-    const void* w;
-    const float* bias;
-    const void* res; int64_t ldr;
-    void* y; int64_t ldy;
-    void* y2; int64_t ldy2; int64_t split;
-    int64_t rows; int K; int M;
-    int out_f32;
-};
 
 // 8 consecutive k of one row, zero beyond K.  FAST: 16-byte aligned rows.
 template <bool FAST>
@@ -262,7 +251,9 @@ extern "C" int bsrl_linear(const void* x, int64_t ldx, const void* w, const floa
         const bool vec = fast && !y2 && M % 4 == 0 && ldy % 4 == 0 && bsrl_aligned(y, 4 * osz) &&
                          (!bias || bsrl_aligned(bias, 16)) &&
                          (!residual || (ldr % 4 == 0 && bsrl_aligned(residual, 8)));
-        if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
+        if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
+            // large, aligned, 16-bit-out problems: the LDS-tiled kernel
+        } else if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
         else launch16<BF16>(a, act, fast, vec, st);
     }
     BSRL_CHECK_LAUNCH("bsrl_linear");

@@ -191,14 +191,15 @@ def attn29_qkv(q, kv, attn_bias, n_heads=4):
 # ---- fused FFN --------------------------------------------------------------------------
 def fused_ffn_ok(x, ffn, ln=None) -> bool:
     """Can `fused_ffn` run on this input? (reference :1143-1174): the fusion is on,
-    16-bit contiguous rows, a Linear-ReLU/GELU-Linear Sequential of a supported width."""
+    16-bit contiguous rows, a Linear-ReLU/GELU-Linear Sequential of a width at which the
+    fused kernel is the faster route (ops.ffn_fused_profitable)."""
     if _ffn_mode == "off" or x.dtype not in (torch.float16, torch.bfloat16) or not x.is_cuda:
         return False
     if len(ffn) != 3 or not isinstance(ffn[0], nn.Linear) or not isinstance(ffn[2], nn.Linear):
         return False
     if not isinstance(ffn[1], (nn.ReLU, nn.GELU)):
         return False
-    return ops.ffn_fused_supported(ffn[0].in_features, ffn[0].out_features, x.dtype)
+    return ops.ffn_fused_profitable(ffn[0].in_features, ffn[0].out_features, x.dtype)
 
 
 def fused_ffn(x, h2, ffn, ln=None):

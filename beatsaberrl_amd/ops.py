@@ -188,6 +188,14 @@ def ffn_fused_supported(d, F, dtype) -> bool:
     return bool(_lib.load().bsrl_ffn_fused_supported(d, F, dt_code(dtype)))
 
 
+def ffn_fused_profitable(d, F, dtype) -> bool:
+    """Is the fused FFN kernel the faster route?  Measured on MI355X (fp16, GELU, 0.26M-3.1M rows):
+    d = 128: 0.17 ms fused vs 0.28 ms for the two linears; d = 192: 0.76 vs 0.98; d = 256: 4.0 vs 2.7;
+    d = 384: 44 vs 16.5 - at d >= 256 the per-workgroup row tile that fits in registers is too small
+    for the weight stream, so the unfused pair (LDS-tiled linears, hidden through HBM) wins."""
+    return d <= 192 and ffn_fused_supported(d, F, dtype)
+
+
 def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5):
     """xo = x + act(h2 w0^T + b0) w2^T + b2; ho = LN(xo) when ln_w is given.
     Returns (xo, ho) (ho None without LN), or None when unsupported."""

@@ -140,6 +140,25 @@ def test_linear_strided_views_split_and_packing(dtype):
         assert torch.equal(packed[..., i * d:(i + 1) * d], ops.linear(tok, ws[i], bs[i]))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,K,M", [(4096, 128, 128), (5000, 128, 384), (4097, 384, 1152), (8192, 1536, 384),
+                                      (6000, 192, 576), (4100, 40, 192), (9000, 256, 1024), (4099, 128, 136)])
+@pytest.mark.parametrize("act,use_res", [(None, False), ("gelu", False), ("relu", True), (None, True)])
+def test_linear_large_row_counts_take_the_tiled_kernel(dtype, rows, K, M, act, use_res):
+    """rows >= 4096 with aligned shapes run the LDS-tiled kernel: same closed form, and the same
+    BITS as the direct-from-global kernel on a slice (both accumulate k in the same order)."""
+    x = _rand(rows, K, dtype=dtype, seed=rows)
+    w = _rand(M, K, dtype=dtype, seed=K + M, scale=1 / math.sqrt(K))
+    b = _rand(M, seed=M)
+    res = _rand(rows, M, dtype=dtype, seed=7) if use_res else None
+    y = ops.linear(x, w, b, act=act, residual=res)
+    ref = _lin_ref(x, w, b, act, res)
+    assert (y.double() - ref).abs().max().item() <= 1.2 * EPS16[dtype] * ref.abs().max().item()
+    for lo, hi in ((0, 300), (rows - 257, rows)):
+        small = ops.linear(x[lo:hi], w, b, act=act, residual=None if res is None else res[lo:hi])
+        assert torch.equal(small, y[lo:hi])
+
+
 def test_linear_rows_are_batch_invariant():
     """A row's bits do not depend on the batch it sits in or on its tile phase
     (the reference holds its kernels to this: tests/test_fused_ffn.py:332-353)."""
