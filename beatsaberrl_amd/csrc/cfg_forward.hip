@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     const float* vlds = reinterpret_cast<const float*>(vlds4);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
-    const float scale = 0.17677669529663688110f;      // 1 / sqrt(32)
+    const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
     constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? 16 : 1;     // envs per 16-row MFMA tile
     constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
     const int64_t ntiles = (a.B + ENVS_PER_WG - 1) / ENVS_PER_WG;
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
-        int nv[RT];
+        float kmask[RT][4];     // additive key mask for keys 4g..4g+3 of each env: 0 (attendable) or -inf
         f32x4 x[RT][NT];
         Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
         Frag8 of[RT][KC];       // attention output fragments (chunk == head)
@@ -155,25 +155,26 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             for (int rt = 0; rt < RT; ++rt) {
                 float mean = 0.f, rstd = 1.f;
                 if (normalise) {
-                    float s = 0.f;
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) s += (x[rt][nt][0] + x[rt][nt][1]) + (x[rt][nt][2] + x[rt][nt][3]);
-                    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
-                    mean = s * (1.0f / D);
-                    float q = 0.f;
+                    // one pass: var = E[x^2] - mean^2, clamped at 0 (the reference kernel's formula,
+                    // python/beat_arena_env/csrc/layer_norm.cu:14-21); both sums ride one butterfly
+                    float s = 0.f, q = 0.f;
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) { const float t = x[rt][nt][i] - mean; q = fmaf(t, t, q); }
-                    q += __shfl_xor(q, 16, WAVE); q += __shfl_xor(q, 32, WAVE);
-                    rstd = rsqrtf(q * (1.0f / D) + 1e-5f);
+                        for (int i = 0; i < 4; ++i) { s += x[rt][nt][i]; q = fmaf(x[rt][nt][i], x[rt][nt][i], q); }
+                    s += __shfl_xor(s, 16, WAVE); q += __shfl_xor(q, 16, WAVE);
+                    s += __shfl_xor(s, 32, WAVE); q += __shfl_xor(q, 32, WAVE);
+                    mean = s * (1.0f / D);
+                    rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q * (1.0f / D)), 0.f) + 1e-5f);
                 }
+                const float shift = -mean * rstd;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const float y0 = fmaf((x[rt][nt][0] - mean) * rstd, gm[nt].x, bt[nt].x);
-                    const float y1 = fmaf((x[rt][nt][1] - mean) * rstd, gm[nt].y, bt[nt].y);
-                    const float y2 = fmaf((x[rt][nt][2] - mean) * rstd, gm[nt].z, bt[nt].z);
-                    const float y3 = fmaf((x[rt][nt][3] - mean) * rstd, gm[nt].w, bt[nt].w);
+                    // (x - mean) * rstd as one fma, then the affine
+                    const float y0 = fmaf(fmaf(x[rt][nt][0], rstd, shift), gm[nt].x, bt[nt].x);
+                    const float y1 = fmaf(fmaf(x[rt][nt][1], rstd, shift), gm[nt].y, bt[nt].y);
+                    const float y2 = fmaf(fmaf(x[rt][nt][2], rstd, shift), gm[nt].z, bt[nt].z);
+                    const float y3 = fmaf(fmaf(x[rt][nt][3], rstd, shift), gm[nt].w, bt[nt].w);
                     dst[rt][nt >> 1].w[(nt & 1) * 2] = pack2<DT>(y0, y1);
                     dst[rt][nt >> 1].w[(nt & 1) * 2 + 1] = pack2<DT>(y2, y3);
                 }
@@ -235,14 +236,16 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
                     f32x4 sc = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                    // raw scores + additive key mask (0 / -inf); softmax of (scale * s) = exp2((s - max) * scale*log2e)
                     float sv[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) sv[i] = (4 * g + i) <= nv[rt] ? sc[i] * scale : -INFINITY;
+                    for (int i = 0; i < 4; ++i) sv[i] = sc[i] + kmask[rt][i];
                     float m = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
                     m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
+                    const float ms = -m * scale_l2e;
                     float sum = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) { sv[i] = __expf(sv[i] - m); sum += sv[i]; }
+                    for (int i = 0; i < 4; ++i) { sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_l2e, ms)); sum += sv[i]; }
                     sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
                     const float inv = __builtin_amdgcn_rcpf(sum);
                     Frag4 pf;
@@ -447,7 +450,9 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
-                nv[rt] = a.n_valid ? a.n_valid[env] : T - 1;
+                const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
                 float ev[KC][8];
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
@@ -536,7 +541,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 int64_t env = env0 + rt * 16 + r16; env = env < a.B ? env : a.B - 1;
-                nv[rt] = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) kmask[rt][i] = 0.f;
                 const uint4* src = reinterpret_cast<const uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) x[rt][nt] = __builtin_bit_cast(f32x4, src[nt]);
