@@ -19,6 +19,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+# HBM bytes per forward of the headline workload (config[1], B = 16384, fp16, fused route with the final
+# block pruned: the HEAD + TAIL launch pair), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
+# dispatch) scaled by what the same counters read for a plain 256 MiB device copy (--calib-copy 256):
+# FETCH_SIZE reads 131084.7 for 262144 KiB fetched (factor 2.000), WRITE_SIZE reads 262144.0 (factor 1.000).
+#   fetched: HEAD 13400.4 x 2.000 + TAIL 7792.0 x 2.000 KiB; written: HEAD 12288.0 + TAIL 13559.7 KiB
+# (profiles/cfg_forward_config1_b16384_f16.txt).  Other workloads report null.
+TRAFFIC_BYTES_CFG1_FUSED_PRUNED = int(((13400.4 + 7792.0) * 2.000 + 12288.0 + 13559.7) * 1024)
 HBM_PEAK_GBS = 8000.0
 
 
@@ -67,6 +74,10 @@ def main():
     ap.add_argument("--no-eager", action="store_true", help="skip the torch-ROCm eager leg")
     ap.add_argument("--no-prune", action="store_true",
                     help="fused route: one persistent kernel computing every token of the last block")
+    ap.add_argument("--calib-copy", type=int, default=0, metavar="MIB",
+                    help="counter calibration only: run 5 plain device copies of MIB MiB (reads MIB, writes MIB "
+                         "per dispatch) and exit; FETCH_SIZE / WRITE_SIZE of these dispatches give the scale "
+                         "factor applied to the forward kernels' counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures ONE GPU: the forward is embarrassingly data-parallel (env rows are "
@@ -74,6 +85,16 @@ def main():
                  "run with --gpus 1.")
 
     import torch
+    if args.calib_copy:
+        n = args.calib_copy << 20
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calib_copy_bytes_read": n, "calib_copy_bytes_written": n, "dispatches": 5}))
+        return
     from beatsaberrl_amd import _lib
     from beatsaberrl_amd.config_policy import ConfigPolicy
     from oracle import config_model as cm     # checker / CPU baseline only
@@ -133,7 +154,9 @@ def main():
     kname = ("cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
              "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else "launch train (per-op route)")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": None, "kernel": kname,
+                "frac": round(achieved / peak, 4),
+                "traffic": TRAFFIC_BYTES_CFG1_FUSED_PRUNED if (pruned and args.config == 1 and B == 16384) else None,
+                "kernel": kname,
                 "launch_ms_avg": round(dev_ms_avg, 4), "launch_ms_p50": round(dev_ms[len(dev_ms) // 2], 4),
                 "flop_per_launch": exec_flops, "dense_flop_per_forward": dense_flops,
                 "dense_equivalent_frac": round(dense_flops / (dev_ms_avg * 1e-3) / 1e12 / peak, 4)}
