@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -51,6 +51,9 @@ SIGNATURES = {
     "bsrl_cfg_pack": (_i32, [C.POINTER(CfgDesc), C.POINTER(CfgParams), _p, _p]),
     "bsrl_cfg_workspace_size": (_i64, [C.POINTER(CfgDesc), _i64]),
     "bsrl_cfg_forward": (_i32, [C.POINTER(CfgDesc), _p, _p, _i64, _i32, _p, _p, _p, _i64, _p, _i64, _p]),
+    "bsrl_note_frontend": (_i32, [_p, _i64, _i32, _p, _p, _i32, _i32, _f, _p, _p, _p, _p, _p, _i64, _i32, _p]),
+    "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _i32,
+                                 _p, _p, _p, _p, _p, _p]),
 }
 
 _lib = None

@@ -235,3 +235,64 @@ def cfg_embed(obs, wp, bp, wo, bo, T, dtype):
     if not _lib.check(rc, "bsrl_cfg_embed"):
         raise Unsupported(f"cfg_embed T={T} d={d}")
     return tokens
+
+
+def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z_asinh=8.0):
+    """obs (B, 630) fp32 or `dtype` -> (saber_in (B, 2, 49), torso_in (B, 29), leg_in (B, 2, 34),
+    note_in (B, 24, 18 | 40), key_bias (B, 29)), all in `dtype`: the forward's preamble in one
+    kernel (obs rounding, lane gathers, note-geometry lanes, one-hots, key bias)."""
+    _need_cuda(obs, saber_idx, body_idx)
+    if obs.dim() != 2 or obs.shape[1] != 630 or obs.stride(1) != 1:
+        raise RuntimeError(f"note_frontend: obs must be (B, 630) with unit last stride, got {tuple(obs.shape)}")
+    if obs.dtype is not torch.float32 and obs.dtype is not dtype:
+        raise TypeError("note_frontend: obs must be fp32 or already in the stream dtype")
+    if saber_idx.dtype is not torch.int32 or body_idx.dtype is not torch.int32 or saber_idx.numel() != 94 \
+            or body_idx.numel() != 93 or not (saber_idx.is_contiguous() and body_idx.is_contiguous()):
+        raise TypeError("note_frontend: saber_idx (94) / body_idx (93) must be contiguous int32 tables")
+    B = obs.shape[0]
+    mk = lambda *s: torch.empty(*s, device=obs.device, dtype=dtype)
+    saber_in, torso_in, leg_in = mk(B, 2, 49), mk(B, 29), mk(B, 2, 34)
+    note_in, key_bias = mk(B, 24, 40 if note_geo else 18), mk(B, 29)
+    with torch.cuda.device(obs.device):
+        rc = _lib.load().bsrl_note_frontend(obs.data_ptr(), obs.stride(0), dt_code(obs.dtype), saber_idx.data_ptr(),
+                                            body_idx.data_ptr(), int(bool(note_geo)), int(bool(flux)), float(z_asinh),
+                                            saber_in.data_ptr(), torso_in.data_ptr(), leg_in.data_ptr(),
+                                            note_in.data_ptr(), key_bias.data_ptr(), B, dt_code(dtype), _stream(obs))
+    _lib.check(rc, "bsrl_note_frontend")
+    return saber_in, torso_in, leg_in, note_in, key_bias
+
+
+def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, action=None,
+                 need_entropy=True, want_ent_h=False, want_noise=False):
+    """Action epilogue on fp32 logits (B, n_heads, K).  action=None samples (Gumbel-max with the
+    caller's Exp(1) draws `exp_noise`, or the kernel's Philox stream keyed by (seed, offset));
+    otherwise evaluates the given (B, n_heads) int64 / uint8 actions.
+    Returns (action int64, logprob, entropy | None, ent_h | None, noise | None)."""
+    _need_cuda(logits, head_sizes, exp_noise, action)
+    if logits.dtype is not torch.float32 or logits.dim() != 3 or not logits.is_contiguous():
+        raise TypeError("sample_heads: logits must be a contiguous fp32 (B, n_heads, K) tensor")
+    B, NH, K = logits.shape
+    if head_sizes is not None and (head_sizes.dtype is not torch.int32 or head_sizes.numel() != NH
+                                   or not head_sizes.is_contiguous()):
+        raise TypeError("sample_heads: head_sizes must be a contiguous int32 (n_heads,) tensor")
+    if exp_noise is not None and (exp_noise.dtype is not torch.float32 or exp_noise.shape != logits.shape
+                                  or not exp_noise.is_contiguous()):
+        raise TypeError("sample_heads: exp_noise must be contiguous fp32 of the logits' shape")
+    u8 = 0
+    if action is not None:
+        if action.shape != (B, NH) or action.dtype not in (torch.int64, torch.uint8) or not action.is_contiguous():
+            raise TypeError("sample_heads: action must be a contiguous (B, n_heads) int64 or uint8 tensor")
+        u8 = int(action.dtype is torch.uint8)
+    dev = logits.device
+    act_out = torch.empty(B, NH, device=dev, dtype=torch.int64)
+    logprob = torch.empty(B, device=dev, dtype=torch.float32)
+    entropy = torch.empty(B, device=dev, dtype=torch.float32) if need_entropy else None
+    ent_h = torch.empty(B, NH, device=dev, dtype=torch.float32) if want_ent_h else None
+    noise = torch.empty_like(logits) if (want_noise and action is None) else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().bsrl_sample_heads(logits.data_ptr(), B, NH, K, _ptr(head_sizes), _ptr(exp_noise),
+                                           int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1), _ptr(action), u8,
+                                           act_out.data_ptr(), logprob.data_ptr(), _ptr(entropy), _ptr(ent_h),
+                                           _ptr(noise), _stream(logits))
+    _lib.check(rc, "bsrl_sample_heads")
+    return act_out, logprob, entropy, ent_h, noise

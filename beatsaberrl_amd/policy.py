@@ -9,10 +9,12 @@ same state_dict and checkpoints) and the same `forward_stacked(obs) -> (logits
     projections with the residual add in the epilogue, FFNs - fused with the next
     block's LayerNorm when `fused_ffn` is on -, SimBa trunk, packed heads, critic
     projections and MLP), every LayerNorm, every attention (blocks, the final block's
-    5 lead queries, the critic's single query);
-  * in torch on the GPU (data movement and O(B x 24) elementwise work): the obs lane
-    gathers, the 22 note-geometry lanes, token concatenation, the key-bias build, the
-    ragged-head scatter and the 101-bin value expectation.
+    5 lead queries, the critic's single query), the forward's preamble (obs rounding,
+    lane gathers, the 22 note-geometry lanes, one-hots, key bias: one front-end kernel)
+    and the action epilogue (log-softmax, Gumbel-max sampling, log-prob, entropy: one
+    kernel);
+  * in torch on the GPU (pure data movement): token concatenation, the ragged-head
+    scatter and the 101-bin value expectation.
 
 Stream dtype: `policy.fp16 = True` runs the 16-bit stream (fp16; set `stream_dtype =
 torch.bfloat16` for bf16) exactly as the reference's switch does (python/policy.py:
@@ -253,6 +255,12 @@ class NotePolicy(nn.Module):
                              persistent=False)
         self.register_buffer("_body_idx", torch.tensor(L.BODY3_IDX, dtype=torch.long), persistent=False)
         self.register_buffer("_hand_id", torch.eye(2), persistent=False)
+        # int32 copies of the lane tables and the per-head gear counts for the kernels
+        self.register_buffer("_saber_idx32", self._saber_idx.to(torch.int32), persistent=False)
+        self.register_buffer("_body_idx32", self._body_idx.to(torch.int32), persistent=False)
+        self.register_buffer("_head_sizes32", torch.tensor(self.head_sizes, dtype=torch.int32), persistent=False)
+        self.sampler = "kernel"                 # "kernel": in-kernel Philox stream; "torch": torch's generator
+        self._sample_calls = 0
         self.fp16 = False                       # True: 16-bit stream (python/policy.py:1085-1090)
         self.stream_dtype = torch.float16       # the 16-bit type used when fp16 is on
         self.fp16_accum = fp16_accum
@@ -313,20 +321,20 @@ class NotePolicy(nn.Module):
     def _forward_stacked(self, obs):
         dt = self.stream_dtype if self.fp16 else torch.float32
         B, d = obs.shape[0], self.embed
-        obs = obs.to(dt)                       # the 16-bit stream consumes the ROUNDED obs (policy.py:1200-1209)
-        sabers, body, notes, note_mask = self._split(obs)
-        sab3 = sabers.reshape(B, 2, SABER_FEAT)
-        if self.note_geo:
-            geo = note_geo(notes.float(), sab3.float(), self.z_asinh, self.game == "flux", obs[:, L.OBS_HEAD_Z].float())
-            notes = torch.cat([notes, geo.to(dt)], dim=-1)                 # (B, 24, 40)
-        hand_id = self._hand_id.to(dt).expand(B, 2, 2)
-        tok_saber = _seq(self.saber_mlp, torch.cat([sab3, hand_id], dim=-1))
-        tok_torso = _seq(self.torso_mlp, body[:, :TORSO_FEAT].contiguous()).unsqueeze(1)
-        legs = torch.cat([body[:, TORSO_FEAT:].reshape(B, 2, LEG_FEAT), hand_id], dim=-1)
-        tok_leg = _seq(self.leg_mlp, legs)
-        tok_note = _seq(self.note_mlp, notes.contiguous())
+        # preamble in one kernel: the obs is rounded once to the stream dtype (policy.py:1200-1209),
+        # gathered into the four encoder inputs (+ note-geometry lanes, one-hots) and the key bias
+        if obs.dtype is not torch.float32 and obs.dtype is not dt:
+            obs = obs.float()
+        if obs.stride(1) != 1:
+            obs = obs.contiguous()
+        sab_in, torso_in, leg_in, note_in, attn_bias = ops.note_frontend(
+            obs, self._saber_idx32, self._body_idx32, dt, note_geo=self.note_geo, flux=self.game == "flux",
+            z_asinh=self.z_asinh)
+        tok_saber = _seq(self.saber_mlp, sab_in)
+        tok_torso = _seq(self.torso_mlp, torso_in).unsqueeze(1)
+        tok_leg = _seq(self.leg_mlp, leg_in)
+        tok_note = _seq(self.note_mlp, note_in)
         x = torch.cat([tok_saber, tok_torso, tok_leg, tok_note], dim=1)   # (B, 29, d)
-        attn_bias = F.pad((note_mask - 1.0) * MASK_BIAS, (self.n_lead, 0)).contiguous()   # (B, 29)
         if self.emb_ln is not None:
             x = self.emb_ln(x)
         h = None
@@ -376,25 +384,31 @@ class NotePolicy(nn.Module):
 
     @torch.no_grad()
     def get_action_and_value(self, obs, action=None, need_entropy=True):
-        """log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) on the
-        kernel forward's logits (reference python/policy.py:1467-1516); this epilogue is
-        plain torch on the (B, 29, K) fp32 logits."""
+        """log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) in one kernel on
+        the forward's fp32 logits (reference python/policy.py:1467-1516).  `self.sampler`:
+        "kernel" draws inside the kernel (Philox keyed by torch's seed and a per-module call
+        counter); "torch" feeds the kernel Exp(1) draws from torch's default generator, the
+        stream the reference rides (use it under graph capture: a captured launch would replay
+        the same in-kernel counter)."""
         logits, value = self.forward_stacked(obs)
-        logsm = torch.log_softmax(logits, dim=-1)
-        if action is None:
-            score = logsm - torch.empty_like(logsm).exponential_().log()
-            if self._gear_valid is not None:
-                score = score.masked_fill(~self._gear_valid, -math.inf)
-            action = score.argmax(-1)
-        elif action.dtype is not torch.long:
+        logits = logits.contiguous()
+        if action is not None and action.dtype not in (torch.int64, torch.uint8):
             action = action.long()
-        logprob = logsm.gather(-1, action.unsqueeze(-1)).squeeze(-1).sum(-1)
-        entropy = None
+        noise = None
+        if action is None and self.sampler == "torch":
+            noise = torch.empty_like(logits).exponential_()
+        elif action is None and self.sampler != "kernel":
+            raise ValueError(f"sampler must be 'kernel' or 'torch', got {self.sampler!r}")
+        sizes = self._head_sizes32 if self._gear_valid is not None else None
+        act, logprob, entropy, ent_h, _ = ops.sample_heads(
+            logits, head_sizes=sizes, exp_noise=noise, seed=torch.initial_seed(), offset=self._sample_calls,
+            action=None if action is None else action.contiguous(), need_entropy=need_entropy,
+            want_ent_h=need_entropy)
+        if action is None:
+            self._sample_calls += 1
         if need_entropy:
-            ent_h = -(logsm.exp() * logsm).sum(-1)
             self._ent_h = ent_h
-            entropy = ent_h.sum(-1)
-        return action, logprob, entropy, value
+        return act, logprob, entropy, value
 
 
 def load_policy(ckpt, game: str = "standard") -> NotePolicy:

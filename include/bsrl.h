@@ -166,6 +166,47 @@ int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      int64_t B, void* workspace, int64_t workspace_bytes,
                      bsrl_stream stream);
 
+/* ---- NotePolicy front end --------------------------------------------------
+ * One pass over the (B, 630) observation that writes every encoder input and
+ * the additive key bias.  Replaces the preamble of the reference forward
+ * (python/policy.py:1199-1260): the one-time rounding of the obs to the stream
+ * dtype (:1199-1209), NotePolicy._split (:1099-1105), _note_geo (:329-404,
+ * fp32 arithmetic on the rounded lanes, one rounding on store), the hand / side
+ * one-hot concatenations (:1231-1246) and the key-bias build (:1257-1260).
+ * obs (B, obs_ld) in obs_dtype = F32 or `dtype`; saber_idx: 94 obs lanes (left
+ * hand's 47, right hand's 47; the reference's `_saber_idx` buffer), body_idx:
+ * 93 obs lanes (torso 29, left leg 32, right leg 32; `_body_idx`), both int32 on
+ * the device.  Outputs, contiguous, in `dtype`: saber_in (B, 2, 49), torso_in
+ * (B, 29), leg_in (B, 2, 34), note_in (B, 24, note_geo ? 40 : 18), key_bias
+ * (B, 29) = 0 for the 5 lead tokens, (mask - 1) * 16384 for the 24 slots. */
+int bsrl_note_frontend(const void* obs, int64_t obs_ld, int obs_dtype,
+                       const int32_t* saber_idx, const int32_t* body_idx,
+                       int note_geo, int flux, float z_asinh,
+                       void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
+                       int64_t B, int dtype, bsrl_stream stream);
+
+/* ---- Action epilogue ---------------------------------------------------------
+ * log-softmax + Gumbel-max sampling + summed log-probability + per-head entropy
+ * on the fp32 logits (B, n_heads, K), K <= 8, n_heads <= 32.  Replaces the tail
+ * of get_action_and_value (python/policy.py:1467-1516).
+ * Sampling (action_in == NULL): action = argmax_k(logsm[k] - log E[k]); lanes
+ * k >= head_sizes[h] (int32 (n_heads), NULL = all K) score -inf
+ * (python/policy.py:1487-1491).  E (B, n_heads, K) fp32 Exp(1) draws come from
+ * exp_noise, or, when it is NULL, from Philox4x32-10 with key = seed and
+ * counter = (row, 2 * offset + block) inside the kernel (row = env * n_heads +
+ * head; draw k of a row is word k & 3 of block k >> 2, mapped to
+ * E = -log(((word >> 8) + 1) * 2^-24)); noise_out, if not NULL, receives the E
+ * used.  Evaluation (action_in != NULL, int64 or uint8 when action_in_u8):
+ * no sampling; action_out may be NULL.
+ * Outputs: action_out (B, n_heads) int64; logprob (B); entropy (B) or NULL;
+ * ent_h (B, n_heads) or NULL. */
+int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads, int64_t K,
+                      const int32_t* head_sizes, const float* exp_noise,
+                      uint64_t seed, uint64_t offset,
+                      const void* action_in, int action_in_u8,
+                      int64_t* action_out, float* logprob, float* entropy, float* ent_h,
+                      float* noise_out, bsrl_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

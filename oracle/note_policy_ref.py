@@ -159,6 +159,25 @@ def _attend(q, k, v, bias, n_heads, r):
 
 
 @torch.no_grad()
+def frontend(obs, note_geo_on=False, flux=False, z_asinh=8.0, emulate=None):
+    """The forward's preamble on its own (reference python/policy.py:1199-1260): obs rounded once
+    to the stream dtype, then (saber_in (B,2,49), torso_in (B,29), leg_in (B,2,34),
+    note_in (B,24,18|40), key_bias (B,29)), every output rounded to the stream dtype."""
+    r = lambda x: _round(x, emulate)
+    B = obs.shape[0]
+    obs = r(obs.float())
+    sab = torch.stack([obs[:, SABER_L], obs[:, SABER_R]], 1)
+    notes = obs[:, OFF_NOTES:OFF_MASK].reshape(B, N_SLOTS, NOTE_FEAT)
+    mask = obs[:, OFF_MASK:OFF_MASK + N_SLOTS]
+    if note_geo_on:
+        notes = r(torch.cat([notes, note_geo(notes, sab, float(z_asinh), flux, obs[:, OBS_HEAD_Z])], -1))
+    eye = torch.eye(2).expand(B, 2, 2)
+    legs = torch.stack([obs[:, LEG_L], obs[:, LEG_R]], 1)
+    bias = F.pad((mask - 1.0) * MASK_BIAS, (N_LEAD, 0))
+    return torch.cat([sab, eye], -1), obs[:, TORSO], torch.cat([legs, eye], -1), notes, r(bias)
+
+
+@torch.no_grad()
 def forward(sd, arch, obs, emulate=None, return_parts=False):
     """obs (B, 630) -> logits (B, 29, k_max) fp32, value (B,) fp32."""
     net = _Net(sd, emulate)
