@@ -34,6 +34,14 @@ class CfgParams(C.Structure):
                 + [(n, C.c_void_p) for n in ("final_ln_w", "final_ln_b", "heads_w", "heads_b")])
 
 
+class BlocksDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "n_heads", "ffn", "T", "act", "n_queries", "dtype")]
+
+
+class BlocksParams(C.Structure):
+    _fields_ = [("blk", _Blk * MAX_LAYERS)]
+
+
 # name -> (restype, argtypes); must list every symbol include/bsrl.h declares
 SIGNATURES = {
     "bsrl_version": (_i32, []),
@@ -51,6 +59,9 @@ SIGNATURES = {
     "bsrl_cfg_pack": (_i32, [C.POINTER(CfgDesc), C.POINTER(CfgParams), _p, _p]),
     "bsrl_cfg_workspace_size": (_i64, [C.POINTER(CfgDesc), _i64]),
     "bsrl_cfg_forward": (_i32, [C.POINTER(CfgDesc), _p, _p, _i64, _i32, _p, _p, _p, _i64, _p, _i64, _p]),
+    "bsrl_blocks_pack_size": (_i64, [C.POINTER(BlocksDesc)]),
+    "bsrl_blocks_pack": (_i32, [C.POINTER(BlocksDesc), C.POINTER(BlocksParams), _p, _p]),
+    "bsrl_blocks_forward": (_i32, [C.POINTER(BlocksDesc), _p, _p, _p, _p, _p, _i64, _p]),
     "bsrl_note_frontend": (_i32, [_p, _i64, _i32, _p, _p, _i32, _i32, _f, _p, _p, _p, _p, _p, _i64, _i32, _p]),
     "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _i32,
                                  _p, _p, _p, _p, _p, _p]),

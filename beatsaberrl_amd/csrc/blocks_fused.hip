@@ -1,0 +1,518 @@
+// The transformer block stack of the policy in ONE persistent kernel for gfx950.
+//
+// Shape class: up to 32 tokens per env (NotePolicy: 29), d = 128 or 192 as 4 heads of 32 or
+// 48, FFN width a multiple of 32, ReLU or GELU, fp16 or bf16 operands with fp32 accumulate.
+// Replaces, for the block stack of NotePolicy._forward_stacked (python/policy.py:1262-1306),
+// the per-block launch train of Block.forward (python/policy.py:524-715): LayerNorm, packed
+// q|k|v projection, attention, output projection + residual, LayerNorm, FFN + residual,
+// with the final block restricted to its first n_queries rows (the reference's n_queries
+// path, python/policy.py:533-539: exact, masking is key-side only).
+//
+// Mapping.  One wave64 owns one 16-row MFMA tile of one env (rows 16*rt .. 16*rt + 15) and
+// carries that tile's fp32 residual stream in registers through every block (d/16 feature
+// tiles x 4 VGPRs).  An env is a wave pair; a workgroup of 8 waves owns 4 envs.  Everything
+// row-local (LayerNorm, projections, FFN with the hidden kept in registers) is wave-local,
+// with the activation always the MFMA operand whose free index is the token, so an output
+// fragment (4 consecutive features per lane) packs straight into the next GEMM's operand;
+// the k order this implies is baked into the weight image.  Only attention crosses the two
+// row tiles: each wave parks its K and V^T fragments of the current head in LDS, and after
+// the next stage barrier reads both tiles' fragments back (scores^T = K Q^T, 8 keys per
+// lane for one query; softmax by in-lane + two cross-lane steps; P V as 16x16x32 MFMAs
+// over the 32 keys).
+//
+// Weights stream from L2 through a 2-slot LDS ring in stages of 2 * (d/32) fragments
+// (8 or 12 KB) shared by the 8 waves: loads issued three stages ahead into registers,
+// written to LDS one stage ahead, one barrier per stage.  All fp32 vectors (biases,
+// LayerNorm affine) of all blocks stay resident in LDS.  HBM traffic is the token stream in
+// and the stream(s) out.
+#include "bsrl_common.h"
+
+namespace {
+
+struct BlkArgs {
+    const uint2* frags; const float* vec;
+    const u16* x_in; const u16* key_bias; u16* x_res; u16* x_out;
+    int64_t B; int n_layers, F, T, n_queries, total_stages;
+};
+
+template <typename DT> __device__ __forceinline__ uint32_t bpack2(float a, float b) {
+    return (uint32_t)DT::from_f(a) | ((uint32_t)DT::from_f(b) << 16);
+}
+template <> __device__ __forceinline__ uint32_t bpack2<F16>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+union BFrag8 { s16x8 v; uint32_t w[4]; uint2 h[2]; uint4 u; };
+union BFrag4 { s16x4 v; uint32_t w[2]; uint2 h; };
+
+__device__ __forceinline__ void blk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int D> struct Geo {
+    static constexpr int NT = D / 16, KC = D / 32, SF = 2 * KC;          // feature tiles, k chunks, fragments per stage
+    static constexpr int STAGE_U2 = SF * 128;                             // uint2 per stage
+    static constexpr int U2PT = STAGE_U2 / 512;                           // uint2 per thread per stage (2 or 3)
+    __host__ __device__ static constexpr int layer_stages(int F) { return 3 * NT / 2 + NT / 2 + 2 * (F / 32); }
+    // per-block fp32 vector region (floats)
+    static constexpr int LN1G = 0, LN1B = D, BQ = 2 * D, BK = 3 * D, BV = 4 * D, BOUT = 5 * D, LN2G = 6 * D, LN2B = 7 * D, B1 = 8 * D;
+    __host__ __device__ static constexpr int b2(int F) { return 8 * D + F; }
+    __host__ __device__ static constexpr int lv_size(int F) { return 9 * D + F; }
+};
+
+// Weight-stage pipeline: stage s lives in ring slot s & 1; its global loads were issued three
+// stage-steps earlier into the register set of the same parity.  The registers are plain named
+// locals (an indexed array would live in scratch and force a wait right after each load).
+#define BADVANCE_P(P, RA, RB, RC) do { \
+        blk_barrier();                                   /* stage s complete in slot P; slot 1-P free */ \
+        ring[1 - (P)][tid] = RA; \
+        ring[1 - (P)][tid + 512] = RB; \
+        if (G::U2PT == 3) ring[1 - (P)][tid + 1024] = RC; \
+        const uint2* src_ = img + (int64_t)pnext * G::STAGE_U2 + tid; \
+        RA = src_[0]; \
+        RB = src_[512]; \
+        if (G::U2PT == 3) RC = src_[1024]; \
+        pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1; \
+    } while (0)
+#define BADVANCE(par) do { if (par) BADVANCE_P(1, pr0a, pr0b, pr0c); else BADVANCE_P(0, pr1a, pr1b, pr1c); } while (0)
+#define BWFRAG(par, f) (__builtin_bit_cast(s16x8, reinterpret_cast<const uint4*>(ring[par])[(f) * 64 + lane]))
+// every fragment of the current stage -> registers in one burst of LDS reads (one wait instead of one per MFMA)
+#define BLOAD_STAGE(par, W) s16x8 W[G::SF]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF; ++f_) W[f_] = BWFRAG(par, f_)
+
+template <typename DT, int D, int DH, int ACT>
+__global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
+    typedef Geo<D> G;
+    constexpr int NT = G::NT, KC = G::KC, H = D / DH, TPH = DH / 16;     // TPH: 16-feature tiles per head (2 or 3)
+    __shared__ __align__(16) uint2 ring[2][G::STAGE_U2];
+    __shared__ uint2 kx[4][2][TPH][64];       // [env][row tile][feature tile of the head][lane]: K fragments
+    __shared__ uint2 vx[4][2][TPH][64];       // V^T half fragments (this row tile's 4 keys per lane)
+    extern __shared__ float4 bvl4[];          // fp32 vectors of every block
+    const float* vlds = reinterpret_cast<const float*>(bvl4);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int el = wave >> 1, rt = wave & 1;
+    const float scale_l2e = (DH == 32 ? 0.17677669529663688110f : 0.14433756729740644113f) * 1.44269504088896340736f;
+    const int64_t ntiles = (a.B + 3) / 4;
+
+    const uint2* img = a.frags;
+    uint2 pr0a, pr0b, pr0c = make_uint2(0, 0), pr1a, pr1b, pr1c = make_uint2(0, 0);
+    int pnext;
+    {   // prologue: stage 0 -> ring slot 0; stages 1 and 2 in flight (every block has an even stage count >= 4)
+        const uint2 s0a = img[tid], s0b = img[tid + 512];
+        uint2 s0c = make_uint2(0, 0);
+        if (G::U2PT == 3) s0c = img[tid + 1024];
+        pr1a = img[G::STAGE_U2 + tid]; pr1b = img[G::STAGE_U2 + tid + 512];
+        if (G::U2PT == 3) pr1c = img[G::STAGE_U2 + tid + 1024];
+        ring[0][tid] = s0a; ring[0][tid + 512] = s0b;
+        if (G::U2PT == 3) ring[0][tid + 1024] = s0c;
+        pr0a = img[2 * G::STAGE_U2 + tid]; pr0b = img[2 * G::STAGE_U2 + tid + 512];
+        if (G::U2PT == 3) pr0c = img[2 * G::STAGE_U2 + tid + 1024];
+        pnext = 3 % a.total_stages;
+        const int nv4 = a.n_layers * G::lv_size(a.F) / 4;
+        for (int i = tid; i < nv4; i += 512) bvl4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        blk_barrier();
+    }
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t env = tile * 4 + el;
+        const int64_t envc = env < a.B ? env : a.B - 1;
+        const int row = 16 * rt + r16;
+        const bool row_ok = row < a.T;
+        f32x4 x[NT];
+        BFrag8 hf[KC];       // LayerNorm output as operand fragments
+        BFrag8 of[KC];       // attention output fragments
+        float kmask[2][4];   // additive key bias * log2(e) for keys 16*kt + 4g + i; -inf past T
+        {
+            const u16* xr = a.x_in + (envc * a.T + (row_ok ? row : 0)) * D;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint2 v = *reinterpret_cast<const uint2*>(xr + 16 * nt + 4 * g);
+                x[nt][0] = row_ok ? DT::to_f((u16)(v.x & 0xffff)) : 0.f;
+                x[nt][1] = row_ok ? DT::to_f((u16)(v.x >> 16)) : 0.f;
+                x[nt][2] = row_ok ? DT::to_f((u16)(v.y & 0xffff)) : 0.f;
+                x[nt][3] = row_ok ? DT::to_f((u16)(v.y >> 16)) : 0.f;
+            }
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = 16 * kt + 4 * g + i;
+                    kmask[kt][i] = key < a.T ? DT::to_f(a.key_bias[envc * a.T + key]) * 1.44269504088896340736f : -INFINITY;
+                }
+        }
+
+        auto norm_to_frags = [&](const float* gptr, const float* bptr) {
+            // one pass: var = E[x^2] - mean^2 clamped at 0 (python/beat_arena_env/csrc/layer_norm.cu:14-21)
+            float s = 0.f, q = 0.f;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { s += x[nt][i]; q = fmaf(x[nt][i], x[nt][i], q); }
+            s += __shfl_xor(s, 16, WAVE); q += __shfl_xor(q, 16, WAVE);
+            s += __shfl_xor(s, 32, WAVE); q += __shfl_xor(q, 32, WAVE);
+            const float mean = s * (1.0f / D);
+            const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q * (1.0f / D)), 0.f) + 1e-5f);
+            const float shift = -mean * rstd;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 gm = *reinterpret_cast<const float4*>(gptr + 16 * nt + 4 * g);
+                const float4 bt = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+                const float y0 = fmaf(fmaf(x[nt][0], rstd, shift), gm.x, bt.x);
+                const float y1 = fmaf(fmaf(x[nt][1], rstd, shift), gm.y, bt.y);
+                const float y2 = fmaf(fmaf(x[nt][2], rstd, shift), gm.z, bt.z);
+                const float y3 = fmaf(fmaf(x[nt][3], rstd, shift), gm.w, bt.w);
+                hf[nt >> 1].w[(nt & 1) * 2] = bpack2<DT>(y0, y1);
+                hf[nt >> 1].w[(nt & 1) * 2 + 1] = bpack2<DT>(y2, y3);
+            }
+        };
+        auto add_bias = [&](const float* bptr) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 b = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+                x[nt][0] += b.x; x[nt][1] += b.y; x[nt][2] += b.z; x[nt][3] += b.w;
+            }
+        };
+        auto store_rows = [&](u16* dst, int rows_per_env, int nrows_valid) {
+            // this wave's rows < nrows_valid of its env, 4 consecutive features (8 bytes) per lane and tile
+            if (env < a.B && row < nrows_valid) {
+                u16* o = dst + (env * rows_per_env + row) * D;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    uint2 v;
+                    v.x = bpack2<DT>(x[nt][0], x[nt][1]); v.y = bpack2<DT>(x[nt][2], x[nt][3]);
+                    *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                }
+            }
+        };
+
+        for (int l = 0; l < a.n_layers; ++l) {
+            const float* lv = vlds + l * G::lv_size(a.F);
+            const bool pruned = a.n_queries > 0 && l == a.n_layers - 1;
+            const bool active = !pruned || rt == 0;          // wave-uniform: the pruned block's queries sit in row tile 0
+            if (pruned && a.x_res) store_rows(a.x_res, a.T, a.T);
+
+            norm_to_frags(lv + G::LN1G, lv + G::LN1B);
+
+            uint2 q[2][TPH];                                  // Q fragments, double-buffered by head parity
+
+            // attention of head hd for this wave's 16 queries over the env's 32 key slots
+            auto attention = [&](int hd) {
+                if (!active) return;
+                f32x4 sc[2];
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    BFrag8 kf, qf;
+                    kf.h[0] = kx[el][kt][0][lane]; kf.h[1] = kx[el][kt][1][lane];
+                    qf.h[0] = q[hd & 1][0]; qf.h[1] = q[hd & 1][1];
+                    sc[kt] = DT::mfma32(kf.v, qf.v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                    if (TPH == 3) {
+                        // features 32..47: a K = 16 MFMA into its OWN accumulator (chaining it onto the
+                        // 16x16x32 accumulator loses the first product on this hardware), summed on the VALU
+                        BFrag4 k2, q2;
+                        k2.h = kx[el][kt][TPH - 1][lane]; q2.h = q[hd & 1][TPH - 1];
+                        const f32x4 s2 = DT::mfma16(k2.v, q2.v, (f32x4){0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sc[kt][i] += s2[i];
+                    }
+                }
+                float sv[2][4];
+                float m = -INFINITY;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[kt][i] = fmaf(sc[kt][i], scale_l2e, kmask[kt][i]); m = fmaxf(m, sv[kt][i]); }
+                m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
+                float sum = 0.f;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[kt][i] = __builtin_amdgcn_exp2f(sv[kt][i] - m); sum += sv[kt][i]; }
+                sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
+                const float inv = __builtin_amdgcn_rcpf(sum);
+                BFrag8 pf;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    pf.w[2 * kt] = bpack2<DT>(sv[kt][0] * inv, sv[kt][1] * inv);
+                    pf.w[2 * kt + 1] = bpack2<DT>(sv[kt][2] * inv, sv[kt][3] * inv);
+                }
+#pragma unroll
+                for (int t = 0; t < TPH; ++t) {
+                    BFrag8 vf;
+                    vf.h[0] = vx[el][0][t][lane]; vf.h[1] = vx[el][1][t][lane];
+                    const float4 bv = *reinterpret_cast<const float4*>(lv + G::BV + DH * hd + 16 * t + 4 * g);
+                    const f32x4 o = DT::mfma32(vf.v, pf.v, (f32x4){bv.x, bv.y, bv.z, bv.w});
+                    const int nt = hd * TPH + t;
+                    of[nt >> 1].w[(nt & 1) * 2] = bpack2<DT>(o[0], o[1]);
+                    of[nt >> 1].w[(nt & 1) * 2 + 1] = bpack2<DT>(o[2], o[3]);
+                }
+            };
+
+            // ---- packed q|k|v projection: 3 * NT feature tiles in head-major order
+            //      [q tiles | k tiles | v tiles] per head, two tiles per stage ----
+#pragma unroll
+            for (int st = 0; st < 3 * NT / 2; ++st) {
+                BADVANCE(st & 1);
+                // a head whose last tile was computed in an earlier stage is complete in LDS after this barrier
+                if (st > 0) {
+                    const int done = (2 * st) / (3 * TPH);            // heads complete before this stage's first tile
+                    const int done_prev = (2 * st - 2) / (3 * TPH);
+                    if (done > done_prev) attention(done - 1);
+                }
+                BLOAD_STAGE(st & 1, wf);
+                f32x4 acc[2];
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
+                    float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? G::BQ : G::BK) + DH * hd + 16 * t + 4 * g);
+                    acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
+                }
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
+                        if (part == 0 && !active) continue;            // the pruned block needs no queries from row tile 1
+                        const s16x8 w = wf[ntl * KC + c];
+                        if (part < 2) acc[ntl] = DT::mfma32(w, hf[c].v, acc[ntl]);
+                        else acc[ntl] = DT::mfma32(hf[c].v, w, acc[ntl]);   // V^T: operand roles swapped
+                    }
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
+                    uint2 pk;
+                    pk.x = bpack2<DT>(acc[ntl][0], acc[ntl][1]); pk.y = bpack2<DT>(acc[ntl][2], acc[ntl][3]);
+                    if (part == 0) q[hd & 1][t] = pk;
+                    else if (part == 1) kx[el][rt][t][lane] = pk;
+                    else vx[el][rt][t][lane] = pk;
+                }
+            }
+
+            // ---- output projection onto the residual (NT / 2 stages) ----
+            if (active) add_bias(lv + G::BOUT);
+#pragma unroll
+            for (int st = 0; st < NT / 2; ++st) {
+                BADVANCE((3 * NT / 2 + st) & 1);
+                if (st == 0) attention(H - 1);                         // the last head completed in the previous stage
+                BLOAD_STAGE((3 * NT / 2 + st) & 1, wf);
+                if (active) {
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl)
+                            x[2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], of[c].v, x[2 * st + ntl]);
+                }
+            }
+
+            // ---- LayerNorm + FFN: stage order W1(0), {W1(ch+1), W2(ch)}..., W2(last); the hidden of a
+            //      32-unit chunk lives in two accumulators, activated and packed into one operand fragment ----
+            constexpr int P0 = (3 * NT / 2 + NT / 2) & 1;              // stage parity at FFN entry (0: 2 * NT is even)
+            static_assert(P0 == 0, "FFN stages start on an even stage");
+            if (active) { norm_to_frags(lv + G::LN2G, lv + G::LN2B); add_bias(lv + G::b2(a.F)); }
+            const int nch = a.F / 32;
+            f32x4 accA[2];
+            auto up = [&](int par, int ch, f32x4 (&acc)[2]) {
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const float4 b = *reinterpret_cast<const float4*>(lv + G::B1 + 32 * ch + 16 * ntl + 4 * g);
+                    acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
+                }
+                BLOAD_STAGE(par, wf);
+                if (active) {
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) acc[ntl] = DT::mfma32(wf[ntl * KC + c], hf[c].v, acc[ntl]);
+                }
+            };
+            BADVANCE(0);
+            up(0, 0, accA);
+            for (int ch = 0; ch < nch; ++ch) {
+                BFrag8 hid;
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    hid.w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(accA[ntl][0]), apply_act16<ACT>(accA[ntl][1]));
+                    hid.w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(accA[ntl][2]), apply_act16<ACT>(accA[ntl][3]));
+                }
+                if (ch + 1 < nch) {
+                    BADVANCE(1);
+                    up(1, ch + 1, accA);
+                    BADVANCE(0);
+                    BLOAD_STAGE(0, w2);
+                    if (active) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) x[nt] = DT::mfma32(w2[nt], hid.v, x[nt]);
+                    }
+                } else {
+                    BADVANCE(1);
+                    BLOAD_STAGE(1, w2);
+                    if (active) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) x[nt] = DT::mfma32(w2[nt], hid.v, x[nt]);
+                    }
+                }
+            }
+        }
+        if (a.n_queries > 0) { if (rt == 0) store_rows(a.x_out, a.n_queries, a.n_queries); }
+        else store_rows(a.x_out, a.T, a.T);
+    }
+}
+
+// ---- weight image ------------------------------------------------------------------
+struct BlkPackArgs {
+    bsrl_blocks_params p;
+    void* frags; float* vec;
+    int n_layers, F;
+};
+__device__ __forceinline__ int bperm_k(int c, int gg, int j) { return 32 * c + 4 * gg + (j & 3) + (j >> 2) * 16; }
+
+// one wave per fragment, one lane per 16-byte slot
+template <typename DT, int D, int DH>
+__global__ __launch_bounds__(256) void blocks_pack_frags_kernel(BlkPackArgs a) {
+    typedef Geo<D> G;
+    constexpr int NT = G::NT, KC = G::KC, SF = G::SF, TPH = DH / 16;
+    const int lane = threadIdx.x & 63;
+    const int lfr = G::layer_stages(a.F) * SF;                 // fragments per block
+    const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= a.n_layers * lfr) return;
+    const int n16 = lane & 15, gg = lane >> 4;
+    const int l = f / lfr, r = f % lfr;
+    const auto& b = a.p.blk[l];
+    const float* src; int ld, n, kbase = 0, c;
+    if (r < 3 * NT * KC) {
+        const int j = r / KC, hd = j / (3 * TPH), rr = j % (3 * TPH), part = rr / TPH, t = rr % TPH;
+        src = part == 0 ? b.q_w : part == 1 ? b.k_w : b.v_w;
+        ld = D; n = DH * hd + 16 * t + n16; c = r % KC;
+    } else if (r < 4 * NT * KC) {
+        const int r2 = r - 3 * NT * KC;
+        src = b.out_w; ld = D; n = 16 * (r2 / KC) + n16; c = r2 % KC;
+    } else {
+        const int r3 = r - 4 * NT * KC, s3 = r3 / SF, i = r3 % SF, nch = a.F / 32;
+        bool upw; int ch;
+        if (s3 == 0) { upw = true; ch = 0; }
+        else if (s3 == 2 * nch - 1) { upw = false; ch = nch - 1; }
+        else { upw = ((s3 - 1) & 1) == 0; ch = (s3 - 1) / 2 + (upw ? 1 : 0); }
+        if (upw) { src = b.ffn0_w; ld = D; n = 32 * ch + 16 * (i / KC) + n16; c = i % KC; }
+        else { src = b.ffn2_w; ld = a.F; n = 16 * i + n16; c = 0; kbase = 32 * ch; }
+    }
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + bperm_k(c, gg, j)];
+    uint4 o;
+    o.x = bpack2<DT>(v[0], v[1]); o.y = bpack2<DT>(v[2], v[3]); o.z = bpack2<DT>(v[4], v[5]); o.w = bpack2<DT>(v[6], v[7]);
+    static_cast<uint4*>(a.frags)[(int64_t)f * 64 + lane] = o;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void blocks_pack_vec_kernel(BlkPackArgs a) {
+    typedef Geo<D> G;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int lvs = G::lv_size(a.F);
+    if (i >= a.n_layers * lvs) return;
+    const int l = i / lvs, r = i % lvs;
+    const auto& b = a.p.blk[l];
+    float v;
+    if (r < G::B1) {
+        const float* srcs[8] = {b.ln_attn_w, b.ln_attn_b, b.q_b, b.k_b, b.v_b, b.out_b, b.ln_ffn_w, b.ln_ffn_b};
+        v = srcs[r / D][r % D];
+    } else if (r < G::b2(a.F)) v = b.ffn0_b[r - G::B1];
+    else v = b.ffn2_b[r - G::b2(a.F)];
+    a.vec[i] = v;
+}
+
+constexpr int LDS_STATIC_MAX = 2 * 12 * 1024 + 2 * 4 * 2 * 3 * 64 * 8;      // ring + K/V exchange at d = 192
+constexpr int LDS_BUDGET = 160 * 1024;
+
+bool blocks_shape_ok(const bsrl_blocks_desc* d) {
+    if (!d) return false;
+    const bool geo = (d->d == 128 && d->n_heads == 4) || (d->d == 192 && d->n_heads == 4);
+    if (!geo || d->T < 1 || d->T > 32 || d->ffn <= 0 || d->ffn % 32 != 0 || d->ffn < 64 || d->n_layers < 1 ||
+        d->n_layers > BSRL_MAX_LAYERS || (d->dtype != BSRL_F16 && d->dtype != BSRL_BF16) ||
+        (d->act != BSRL_ACT_RELU && d->act != BSRL_ACT_GELU) || d->n_queries < 0 || d->n_queries > 16 || d->n_queries > d->T)
+        return false;
+    const int64_t vec_bytes = (int64_t)d->n_layers * (9 * d->d + d->ffn) * 4;
+    return vec_bytes + LDS_STATIC_MAX <= LDS_BUDGET;
+}
+int64_t blocks_stages(const bsrl_blocks_desc* d) {
+    return (int64_t)d->n_layers * (d->d == 128 ? Geo<128>::layer_stages(d->ffn) : Geo<192>::layer_stages(d->ffn));
+}
+int64_t blocks_frag_bytes(const bsrl_blocks_desc* d) { return blocks_stages(d) * (d->d / 16) * 1024; }
+
+template <typename DT, int D, int DH>
+void pack_launch(const BlkPackArgs& pa, int64_t nfrags, hipStream_t st) {
+    hipLaunchKernelGGL((blocks_pack_frags_kernel<DT, D, DH>), dim3((unsigned)((nfrags + 3) / 4)), dim3(256), 0, st, pa);
+    const int nvec = pa.n_layers * Geo<D>::lv_size(pa.F);
+    hipLaunchKernelGGL(blocks_pack_vec_kernel<D>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, st, pa);
+}
+
+template <typename DT, int D, int DH, int ACT>
+int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
+    const size_t dyn = (size_t)a.n_layers * Geo<D>::lv_size(a.F) * sizeof(float);
+    auto kern = blocks_kernel<DT, D, DH, ACT>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+        return BSRL_UNSUPPORTED;
+    const int64_t ntiles = (a.B + 3) / 4;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(512), dyn, st, a);
+    return BSRL_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t bsrl_blocks_pack_size(const bsrl_blocks_desc* d) {
+    if (!blocks_shape_ok(d)) return 0;
+    return blocks_frag_bytes(d) + (int64_t)d->n_layers * (9 * d->d + d->ffn) * 4;
+}
+
+extern "C" int bsrl_blocks_pack(const bsrl_blocks_desc* d, const bsrl_blocks_params* p, void* packed, bsrl_stream stream) {
+    if (!d || !p || !packed) BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_pack: null pointer");
+    if (!blocks_shape_ok(d)) return BSRL_UNSUPPORTED;
+    if (!bsrl_aligned(packed, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_pack: image must be 16-byte aligned");
+    for (int l = 0; l < d->n_layers; ++l) {
+        const float* const* ptrs = reinterpret_cast<const float* const*>(&p->blk[l]);
+        for (int i = 0; i < 16; ++i)
+            if (!ptrs[i]) BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_pack: null parameter pointer in block %d", l);
+    }
+    BlkPackArgs pa;
+    pa.p = *p; pa.frags = packed;
+    pa.vec = reinterpret_cast<float*>(static_cast<char*>(packed) + blocks_frag_bytes(d));
+    pa.n_layers = d->n_layers; pa.F = d->ffn;
+    const int64_t nfrags = blocks_stages(d) * (d->d / 16);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (d->d == 128) { if (d->dtype == BSRL_F16) pack_launch<F16, 128, 32>(pa, nfrags, st); else pack_launch<BF16, 128, 32>(pa, nfrags, st); }
+    else { if (d->dtype == BSRL_F16) pack_launch<F16, 192, 48>(pa, nfrags, st); else pack_launch<BF16, 192, 48>(pa, nfrags, st); }
+    BSRL_CHECK_LAUNCH("bsrl_blocks_pack");
+    return BSRL_OK;
+}
+
+extern "C" int bsrl_blocks_forward(const bsrl_blocks_desc* d, const void* packed, const void* x_in, const void* key_bias,
+                                   void* x_res, void* x_out, int64_t B, bsrl_stream stream) {
+    if (!d || !packed || !x_in || !key_bias || !x_out) BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_forward: null pointer");
+    if (!blocks_shape_ok(d)) return BSRL_UNSUPPORTED;
+    if (B < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_forward: B < 0");
+    if (!bsrl_aligned(packed, 16) || !bsrl_aligned(x_in, 8) || !bsrl_aligned(x_out, 8) || (x_res && !bsrl_aligned(x_res, 8)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_blocks_forward: image must be 16-byte, token streams 8-byte aligned");
+    if (B == 0) return BSRL_OK;
+    BlkArgs a;
+    a.frags = static_cast<const uint2*>(packed);
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(packed) + blocks_frag_bytes(d));
+    a.x_in = static_cast<const u16*>(x_in); a.key_bias = static_cast<const u16*>(key_bias);
+    a.x_res = static_cast<u16*>(x_res); a.x_out = static_cast<u16*>(x_out);
+    a.B = B; a.n_layers = d->n_layers; a.F = d->ffn; a.T = d->T; a.n_queries = d->n_queries;
+    a.total_stages = (int)blocks_stages(d);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    int rc;
+    const bool relu = d->act == BSRL_ACT_RELU, f16 = d->dtype == BSRL_F16;
+    if (d->d == 128) {
+        if (f16) rc = relu ? fwd_launch<F16, 128, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<F16, 128, 32, BSRL_ACT_GELU>(a, cus, st);
+        else rc = relu ? fwd_launch<BF16, 128, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<BF16, 128, 32, BSRL_ACT_GELU>(a, cus, st);
+    } else {
+        if (f16) rc = relu ? fwd_launch<F16, 192, 48, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<F16, 192, 48, BSRL_ACT_GELU>(a, cus, st);
+        else rc = relu ? fwd_launch<BF16, 192, 48, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<BF16, 192, 48, BSRL_ACT_GELU>(a, cus, st);
+    }
+    if (rc != BSRL_OK) return rc;
+    BSRL_CHECK_LAUNCH("bsrl_blocks_forward");
+    return BSRL_OK;
+}

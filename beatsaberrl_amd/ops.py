@@ -296,3 +296,56 @@ def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, acti
                                            _ptr(noise), _stream(logits))
     _lib.check(rc, "bsrl_sample_heads")
     return act_out, logprob, entropy, ent_h, noise
+
+
+# ---- fused transformer block stack ----------------------------------------------------
+def _blocks_desc(n_layers, d, n_heads, ffn, T, act, n_queries, dtype):
+    return _lib.BlocksDesc(n_layers=n_layers, d=d, n_heads=n_heads, ffn=ffn, T=T, act=_ACT[act],
+                           n_queries=n_queries, dtype=dt_code(dtype))
+
+
+def blocks_pack_size(n_layers, d, n_heads, ffn, T, act, n_queries, dtype) -> int:
+    """Bytes of the fused block stack's weight image; 0 = this shape has no fused kernel."""
+    desc = _blocks_desc(n_layers, d, n_heads, ffn, T, act, n_queries, dtype)
+    return int(_lib.load().bsrl_blocks_pack_size(desc))
+
+
+_BLK_FIELDS = ("ln_attn_w", "ln_attn_b", "q_w", "q_b", "k_w", "k_b", "v_w", "v_b", "out_w", "out_b",
+               "ln_ffn_w", "ln_ffn_b", "ffn0_w", "ffn0_b", "ffn2_w", "ffn2_b")
+
+
+def blocks_pack(block_params, image, d, n_heads, ffn, T, act, n_queries, dtype):
+    """block_params: per block, the 16 fp32 master tensors in `_BLK_FIELDS` order (contiguous,
+    on the device).  Writes the MFMA-fragment-major image into `image` (uint8 tensor of
+    blocks_pack_size bytes, 16-byte aligned)."""
+    desc = _blocks_desc(len(block_params), d, n_heads, ffn, T, act, n_queries, dtype)
+    params = _lib.BlocksParams()
+    for l, tensors in enumerate(block_params):
+        if len(tensors) != 16:
+            raise ValueError("blocks_pack: 16 tensors per block expected")
+        for name, t in zip(_BLK_FIELDS, tensors):
+            _need_cuda(t)
+            setattr(params.blk[l], name, _f32c(t.detach(), name).data_ptr())
+    with torch.cuda.device(image.device):
+        rc = _lib.load().bsrl_blocks_pack(desc, params, image.data_ptr(), _stream(image))
+    if not _lib.check(rc, "bsrl_blocks_pack"):
+        raise Unsupported("blocks_pack: shape not covered by the fused block stack")
+
+
+def blocks_forward(image, x, key_bias, n_layers, n_heads, ffn, act, n_queries, want_res=True):
+    """x (B, T, d) 16-bit tokens, key_bias (B, T) same dtype -> (x_out, x_res | None): the whole
+    block stack in one launch; x_out is (B, n_queries, d) when n_queries > 0 else (B, T, d)."""
+    _need_cuda(image, x, key_bias)
+    if x.dim() != 3 or not x.is_contiguous() or not key_bias.is_contiguous() or key_bias.dtype is not x.dtype \
+            or key_bias.shape != x.shape[:2]:
+        raise RuntimeError("blocks_forward: x (B, T, d) and key_bias (B, T) must be contiguous and of one dtype")
+    B, T, d = x.shape
+    desc = _blocks_desc(n_layers, d, n_heads, ffn, T, act, n_queries, x.dtype)
+    out = torch.empty(B, n_queries if n_queries else T, d, device=x.device, dtype=x.dtype)
+    res = torch.empty_like(x) if (want_res and n_queries) else None
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_blocks_forward(desc, image.data_ptr(), x.data_ptr(), key_bias.data_ptr(), _ptr(res),
+                                             out.data_ptr(), B, _stream(x))
+    if not _lib.check(rc, "bsrl_blocks_forward"):
+        raise Unsupported("blocks_forward: shape not covered by the fused block stack")
+    return out, res

@@ -132,13 +132,17 @@ typedef struct {
     int32_t prop_dim, obj_dim, dtype, reserved;
 } bsrl_cfg_desc;
 
+/* fp32 master parameter pointers of one transformer block, in the reference's
+ * registration order (python/policy.py:492-522); device memory. */
+typedef struct {
+    const float *ln_attn_w, *ln_attn_b, *q_w, *q_b, *k_w, *k_b, *v_w, *v_b,
+        *out_w, *out_b, *ln_ffn_w, *ln_ffn_b, *ffn0_w, *ffn0_b, *ffn2_w, *ffn2_b;
+} bsrl_block_params;
+
 /* fp32 master parameter pointers in state_dict order (device memory). */
 typedef struct {
     const float *prop_w, *prop_b, *obj_w, *obj_b;
-    struct {
-        const float *ln_attn_w, *ln_attn_b, *q_w, *q_b, *k_w, *k_b, *v_w, *v_b,
-            *out_w, *out_b, *ln_ffn_w, *ln_ffn_b, *ffn0_w, *ffn0_b, *ffn2_w, *ffn2_b;
-    } blk[BSRL_MAX_LAYERS];
+    bsrl_block_params blk[BSRL_MAX_LAYERS];
     const float *final_ln_w, *final_ln_b, *heads_w, *heads_b;
 } bsrl_cfg_params;
 
@@ -206,6 +210,36 @@ int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads, int64_t K
                       const void* action_in, int action_in_u8,
                       int64_t* action_out, float* logprob, float* entropy, float* ent_h,
                       float* noise_out, bsrl_stream stream);
+
+/* ---- Transformer block stack in one persistent kernel ------------------------
+ * Replaces the block loop of NotePolicy._forward_stacked (python/policy.py:
+ * 1262-1306): every Block.forward (python/policy.py:524-715) of the stack -
+ * LayerNorm, q|k|v projection, attention with the additive key bias, output
+ * projection + residual, LayerNorm, FFN + residual - with the residual stream
+ * held in fp32 registers from the first block to the last.
+ * Shapes: T <= 32 tokens per env, d = 128 (4 heads x 32) or 192 (4 x 48), ffn a
+ * multiple of 32, act RELU or GELU, dtype F16 or BF16.  n_queries > 0 restricts
+ * the LAST block to its first n_queries (<= 16) rows, the reference's n_queries
+ * path (python/policy.py:533-539; exact: masking is key-side only).
+ * `packed` = image written by bsrl_blocks_pack for the same desc (rebuild after
+ * each optimizer step; the address must not move under a captured graph).
+ * x_in (B, T, d), key_bias (B, T) in `dtype`, contiguous.  x_out: (B, n_queries, d)
+ * when n_queries > 0, else (B, T, d).  x_res (B, T, d) or NULL: with n_queries > 0,
+ * the stream entering the last block (what the reference's critic reads,
+ * python/policy.py:1296-1301). */
+typedef struct {
+    int32_t n_layers, d, n_heads, ffn, T, act, n_queries, dtype;
+} bsrl_blocks_desc;
+typedef struct {
+    bsrl_block_params blk[BSRL_MAX_LAYERS];
+} bsrl_blocks_params;
+/* Bytes of the packed image, or 0 if the shape is unsupported. */
+int64_t bsrl_blocks_pack_size(const bsrl_blocks_desc* desc);
+int bsrl_blocks_pack(const bsrl_blocks_desc* desc, const bsrl_blocks_params* params,
+                     void* packed, bsrl_stream stream);
+int bsrl_blocks_forward(const bsrl_blocks_desc* desc, const void* packed,
+                        const void* x_in, const void* key_bias,
+                        void* x_res, void* x_out, int64_t B, bsrl_stream stream);
 
 #ifdef __cplusplus
 }

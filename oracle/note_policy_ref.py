@@ -158,6 +158,41 @@ def _attend(q, k, v, bias, n_heads, r):
     return (r(torch.softmax(s, -1)) @ vh).transpose(1, 2).reshape(B, Tq, d)
 
 
+def _blocks(net, arch, x, bias, round_residual=True):
+    """The block stack (reference python/policy.py:1262-1306, Block.forward :524-715): blocks
+    0..L-2 over all T rows, the final block on the N_LEAD lead rows only.  Returns (lead (B,5,d),
+    x_res (B,T,d) = the stream entering the final block).  round_residual=False keeps the
+    residual stream unrounded between blocks (a kernel that carries it in fp32 registers)."""
+    r = net.r
+    rr = r if round_residual else (lambda t: t)
+    H, L = arch["n_heads"], arch["n_blocks"]
+
+    def block(i, x, n_q):
+        p = f"blocks.{i}."
+        h = r(net.ln(p + "ln_attn", x))
+        k, v = r(net.lin(p + "k_proj", h)), r(net.lin(p + "v_proj", h))
+        x_full = x
+        if n_q:
+            x, h = x[:, :n_q], h[:, :n_q]
+        q = r(net.lin(p + "q_proj", h))
+        att = r(_attend(q, k, v, bias, H, r))
+        x = rr(x + net.lin(p + "out_proj", att))
+        h2 = r(net.ln(p + "ln_ffn", x))
+        x = rr(x + net.mlp2(p + "ffn", h2))
+        return x, x_full
+
+    for i in range(L - 1):
+        x, _ = block(i, x, 0)
+    lead, x_res = block(L - 1, x, N_LEAD)
+    return r(lead), r(x_res)
+
+
+@torch.no_grad()
+def blocks_forward(sd, arch, x, bias, emulate=None, round_residual=True):
+    """Public form of the block stack for kernel tests: x (B,T,d) tokens, bias (B,T) additive key bias."""
+    return _blocks(_Net(sd, emulate), arch, _round(x.float(), emulate), bias.float(), round_residual)
+
+
 @torch.no_grad()
 def frontend(obs, note_geo_on=False, flux=False, z_asinh=8.0, emulate=None):
     """The forward's preamble on its own (reference python/policy.py:1199-1260): obs rounded once
@@ -203,23 +238,7 @@ def forward(sd, arch, obs, emulate=None, return_parts=False):
     if arch.get("emb_ln", False):
         x = r(net.ln("emb_ln", x))
 
-    def block(i, x, n_q):
-        p = f"blocks.{i}."
-        h = r(net.ln(p + "ln_attn", x))
-        k, v = r(net.lin(p + "k_proj", h)), r(net.lin(p + "v_proj", h))
-        x_full = x
-        if n_q:
-            x, h = x[:, :n_q], h[:, :n_q]
-        q = r(net.lin(p + "q_proj", h))
-        att = r(_attend(q, k, v, bias, H, r))
-        x = r(x + net.lin(p + "out_proj", att))
-        h2 = r(net.ln(p + "ln_ffn", x))
-        x = r(x + net.mlp2(p + "ffn", h2))
-        return x, x_full
-
-    for i in range(L - 1):
-        x, _ = block(i, x, 0)
-    lead, x_res = block(L - 1, x, N_LEAD)
+    lead, x_res = _blocks(net, arch, x, bias)
     if arch.get("final_ln", False):
         lead = r(net.ln("final_ln", lead))
     # SimBa readout trunk

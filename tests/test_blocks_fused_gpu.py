@@ -1,0 +1,105 @@
+"""GPU parity of the fused transformer block stack (one persistent kernel, C ABI) against the CPU
+oracle's block stack (oracle/note_policy_ref.py::blocks_forward, the part of the NotePolicy oracle
+that the reference's golden vectors pin).
+
+Gates (the class-relative form used for every whole-stack 16-bit comparison in this suite): with
+e_emul = max |emulated-16-bit oracle - fp32 oracle| and e_mine = max |kernel - fp32 oracle|,
+e_mine <= max(1.25 * e_emul, floor) and |kernel - emulated oracle| <= 2.5 * max(e_emul, floor)
+(the triangle bound of the first gate; floor = 2e-3 for fp16, 1.6e-2 = one bf16 ulp at 2 for bf16): the
+kernel keeps its residual stream in fp32 registers, so it must sit inside the error class of a
+16-bit-stream forward, not reproduce one particular rounding order."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from beatsaberrl_amd import ops  # noqa: E402
+from oracle import note_policy_ref as nr  # noqa: E402
+
+DEV = "cuda"
+TDT = {"f16": torch.float16, "bf16": torch.bfloat16}
+FIELDS = ("ln_attn.weight", "ln_attn.bias", "q_proj.weight", "q_proj.bias", "k_proj.weight", "k_proj.bias",
+          "v_proj.weight", "v_proj.bias", "out_proj.weight", "out_proj.bias", "ln_ffn.weight", "ln_ffn.bias",
+          "ffn.0.weight", "ffn.0.bias", "ffn.2.weight", "ffn.2.bias")
+
+
+def _weights(L, d, F, seed):
+    g = torch.Generator().manual_seed(seed)
+    sd = {}
+    for i in range(L):
+        p = f"blocks.{i}."
+        for n in ("ln_attn", "ln_ffn"):
+            sd[p + n + ".weight"] = 1.0 + 0.1 * torch.randn(d, generator=g)
+            sd[p + n + ".bias"] = 0.1 * torch.randn(d, generator=g)
+        for n, (o, k) in (("q_proj", (d, d)), ("k_proj", (d, d)), ("v_proj", (d, d)), ("out_proj", (d, d)),
+                          ("ffn.0", (F, d)), ("ffn.2", (d, F))):
+            sd[p + n + ".weight"] = torch.randn(o, k, generator=g) * (1.0 / k ** 0.5)
+            sd[p + n + ".bias"] = 0.1 * torch.randn(o, generator=g)
+    return sd
+
+
+def _inputs(B, T, d, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, T, d, generator=g)
+    mask = (torch.rand(B, T, generator=g) < 0.6).float()
+    mask[:, :5] = 1.0
+    mask[0, 5:] = 0.0
+    return x, (mask - 1.0) * 16384.0
+
+
+def _run(sd, L, d, F, T, dtype, x, bias, n_queries):
+    tdt = TDT[dtype]
+    nbytes = ops.blocks_pack_size(L, d, 4, F, T, "relu", n_queries, tdt)
+    assert nbytes > 0
+    image = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    params = [[sd[f"blocks.{i}.{f}"].to(DEV).contiguous() for f in FIELDS] for i in range(L)]
+    ops.blocks_pack(params, image, d, 4, F, T, "relu", n_queries, tdt)
+    return ops.blocks_forward(image, x.to(DEV).to(tdt).contiguous(), bias.to(DEV).to(tdt).contiguous(), L, 4, F,
+                              "relu", n_queries)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("d,L,B", [(128, 1, 5), (192, 1, 5), (128, 3, 37), (192, 3, 37), (192, 6, 64)])
+def test_block_stack_matches_oracle(dtype, d, L, B):
+    T, F = 29, 4 * d
+    sd = _weights(L, d, F, 10 + L + d)
+    x, bias = _inputs(B, T, d, 3 + B)
+    arch = {"n_heads": 4, "n_blocks": L}
+    lead32, res32 = nr.blocks_forward(sd, arch, x.to(TDT[dtype]), bias)          # fp32 math on the rounded tokens
+    lead_em, res_em = nr.blocks_forward(sd, arch, x, bias, emulate=dtype)
+    out, res = _run(sd, L, d, F, T, dtype, x, bias, 5)
+    out, res = out.float().cpu(), res.float().cpu()
+    assert out.shape == (B, 5, d) and res.shape == (B, T, d)
+    for mine, ref, em, name in ((out, lead32, lead_em, "lead"), (res, res32, res_em, "x_res")):
+        e_emul = (em - ref).abs().max().item()
+        e_mine = (mine - ref).abs().max().item()
+        floor = 2e-3 if dtype == "f16" else 1.6e-2
+        assert e_mine <= max(1.25 * e_emul, floor), (name, e_mine, e_emul)
+        assert (mine - em).abs().max().item() <= 2.5 * max(e_emul, floor), name
+
+
+def test_unpruned_stack_and_invariants():
+    d, L, B, T, F = 192, 2, 21, 29, 768
+    sd = _weights(L, d, F, 77)
+    x, bias = _inputs(B, T, d, 8)
+    full, none = _run(sd, L, d, F, T, "f16", x, bias, 0)
+    assert none is None and full.shape == (B, T, d)
+    lead, res = _run(sd, L, d, F, T, "f16", x, bias, 5)
+    # pruning the final block to the lead rows is exact up to the reduction order inside the kernel
+    assert (full[:, :5].float() - lead.float()).abs().max().item() <= 2e-3
+    # junk in masked slots cannot change anything attendable: lead rows bitwise equal
+    x2 = x.clone()
+    x2[bias < 0] = 7.0
+    lead2, _ = _run(sd, L, d, F, T, "f16", x2, bias, 5)
+    assert torch.equal(lead, lead2)
+    # batch-slice invariance and run-to-run reproducibility (bitwise)
+    lead3, res3 = _run(sd, L, d, F, T, "f16", x[3:11], bias[3:11], 5)
+    assert torch.equal(lead3, lead[3:11]) and torch.equal(res3, res[3:11])
+    lead4, res4 = _run(sd, L, d, F, T, "f16", x, bias, 5)
+    assert torch.equal(lead4, lead) and torch.equal(res4, res)
+
+
+def test_unsupported_shapes_are_reported():
+    assert ops.blocks_pack_size(2, 256, 8, 1024, 32, "relu", 0, torch.float16) == 0
+    assert ops.blocks_pack_size(2, 192, 4, 768, 48, "relu", 0, torch.float16) == 0
+    assert ops.blocks_pack_size(2, 192, 4, 768, 29, "relu", 5, torch.float32 if False else torch.float16) > 0
