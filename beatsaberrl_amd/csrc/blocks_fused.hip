@@ -26,6 +26,7 @@
 // LayerNorm affine) of all blocks stay resident in LDS.  HBM traffic is the token stream in
 // and the stream(s) out.
 #include "bsrl_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -48,6 +49,12 @@ union BFrag8 { s16x8 v; uint32_t w[4]; uint2 h[2]; uint4 u; };
 union BFrag4 { s16x4 v; uint32_t w[2]; uint2 h; };
 
 __device__ __forceinline__ void blk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// compile-time loop: the body sees its index as a constant (the loop unroller gives up on the
+// larger bodies, and register arrays indexed by the loop variable would then live in scratch)
+template <int I, int N, typename Fn> __device__ __forceinline__ void static_for(Fn&& fn) {
+    if constexpr (I < N) { fn(std::integral_constant<int, I>{}); static_for<I + 1, N>(fn); }
+}
 
 template <int D> struct Geo {
     static constexpr int NT = D / 16, KC = D / 32, SF = 2 * KC;          // feature tiles, k chunks, fragments per stage
@@ -77,7 +84,12 @@ template <int D> struct Geo {
 #define BADVANCE(par) do { if (par) BADVANCE_P(1, pr0a, pr0b, pr0c); else BADVANCE_P(0, pr1a, pr1b, pr1c); } while (0)
 #define BWFRAG(par, f) (__builtin_bit_cast(s16x8, reinterpret_cast<const uint4*>(ring[par])[(f) * 64 + lane]))
 // every fragment of the current stage -> registers in one burst of LDS reads (one wait instead of one per MFMA)
-#define BLOAD_STAGE(par, W) s16x8 W[G::SF]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF; ++f_) W[f_] = BWFRAG(par, f_)
+// half a stage (SF / 2 fragments) -> registers in one burst of LDS reads (one wait instead of one per MFMA).
+// BLOAD_HALF: k chunks [half * KC/2, +KC/2) of both feature tiles, W[ntl * KC/2 + ci]; BLOAD_RANGE: fragments
+// [first, first + SF/2).
+#define BLOAD_HALF(par, W, half) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) \
+        W[f_] = BWFRAG(par, (f_ / (G::KC / 2)) * G::KC + (half) * (G::KC / 2) + f_ % (G::KC / 2))
+#define BLOAD_RANGE(par, W, first) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) W[f_] = BWFRAG(par, (first) + f_)
 
 template <typename DT, int D, int DH, int ACT>
 __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
@@ -196,7 +208,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
             uint2 q[2][TPH];                                  // Q fragments, double-buffered by head parity
 
             // attention of head hd for this wave's 16 queries over the env's 32 key slots
-            auto attention = [&](int hd) {
+            auto attention = [&](auto hd_) {
+                constexpr int hd = decltype(hd_)::value;
                 if (!active) return;
                 f32x4 sc[2];
 #pragma unroll
@@ -249,16 +262,15 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 
             // ---- packed q|k|v projection: 3 * NT feature tiles in head-major order
             //      [q tiles | k tiles | v tiles] per head, two tiles per stage ----
-#pragma unroll
-            for (int st = 0; st < 3 * NT / 2; ++st) {
+            static_for<0, 3 * NT / 2>([&](auto st_) {
+                constexpr int st = decltype(st_)::value;
                 BADVANCE(st & 1);
                 // a head whose last tile was computed in an earlier stage is complete in LDS after this barrier
-                if (st > 0) {
-                    const int done = (2 * st) / (3 * TPH);            // heads complete before this stage's first tile
-                    const int done_prev = (2 * st - 2) / (3 * TPH);
-                    if (done > done_prev) attention(done - 1);
+                if constexpr (st > 0) {
+                    constexpr int done = (2 * st) / (3 * TPH);        // heads complete before this stage's first tile
+                    constexpr int done_prev = (2 * st - 2) / (3 * TPH);
+                    if constexpr (done > done_prev) attention(std::integral_constant<int, done - 1>{});
                 }
-                BLOAD_STAGE(st & 1, wf);
                 f32x4 acc[2];
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
@@ -268,15 +280,20 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
                 }
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
+                for (int half = 0; half < 2; ++half) {
+                    BLOAD_HALF(st & 1, wf, half);                      // k chunks [half * KC/2, +KC/2) of both tiles
 #pragma unroll
-                    for (int ntl = 0; ntl < 2; ++ntl) {
-                        const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
-                        if (part == 0 && !active) continue;            // the pruned block needs no queries from row tile 1
-                        const s16x8 w = wf[ntl * KC + c];
-                        if (part < 2) acc[ntl] = DT::mfma32(w, hf[c].v, acc[ntl]);
-                        else acc[ntl] = DT::mfma32(hf[c].v, w, acc[ntl]);   // V^T: operand roles swapped
-                    }
+                    for (int ci = 0; ci < KC / 2; ++ci)
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) {
+                            const int c = half * (KC / 2) + ci;
+                            const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
+                            if (part == 0 && !active) continue;        // the pruned block needs no queries from row tile 1
+                            const s16x8 w = wf[ntl * (KC / 2) + ci];
+                            if (part < 2) acc[ntl] = DT::mfma32(w, hf[c].v, acc[ntl]);
+                            else acc[ntl] = DT::mfma32(hf[c].v, w, acc[ntl]);   // V^T: operand roles swapped
+                        }
+                }
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
                     const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
@@ -286,21 +303,24 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     else if (part == 1) kx[el][rt][t][lane] = pk;
                     else vx[el][rt][t][lane] = pk;
                 }
-            }
+            });
 
             // ---- output projection onto the residual (NT / 2 stages) ----
             if (active) add_bias(lv + G::BOUT);
 #pragma unroll
             for (int st = 0; st < NT / 2; ++st) {
                 BADVANCE((3 * NT / 2 + st) & 1);
-                if (st == 0) attention(H - 1);                         // the last head completed in the previous stage
-                BLOAD_STAGE((3 * NT / 2 + st) & 1, wf);
-                if (active) {
+                if (st == 0) attention(std::integral_constant<int, H - 1>{});                         // the last head completed in the previous stage
 #pragma unroll
-                    for (int c = 0; c < KC; ++c)
+                for (int half = 0; half < 2; ++half) {
+                    BLOAD_HALF((3 * NT / 2 + st) & 1, wf, half);
+                    if (active) {
 #pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl)
-                            x[2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], of[c].v, x[2 * st + ntl]);
+                        for (int ci = 0; ci < KC / 2; ++ci)
+#pragma unroll
+                            for (int ntl = 0; ntl < 2; ++ntl)
+                                x[2 * st + ntl] = DT::mfma32(wf[ntl * (KC / 2) + ci], of[half * (KC / 2) + ci].v, x[2 * st + ntl]);
+                    }
                 }
             }
 
@@ -317,12 +337,16 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     const float4 b = *reinterpret_cast<const float4*>(lv + G::B1 + 32 * ch + 16 * ntl + 4 * g);
                     acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
                 }
-                BLOAD_STAGE(par, wf);
-                if (active) {
 #pragma unroll
-                    for (int c = 0; c < KC; ++c)
+                for (int half = 0; half < 2; ++half) {
+                    BLOAD_HALF(par, wf, half);
+                    if (active) {
 #pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl) acc[ntl] = DT::mfma32(wf[ntl * KC + c], hf[c].v, acc[ntl]);
+                        for (int ci = 0; ci < KC / 2; ++ci)
+#pragma unroll
+                            for (int ntl = 0; ntl < 2; ++ntl)
+                                acc[ntl] = DT::mfma32(wf[ntl * (KC / 2) + ci], hf[half * (KC / 2) + ci].v, acc[ntl]);
+                    }
                 }
             };
             BADVANCE(0);
@@ -338,17 +362,23 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     BADVANCE(1);
                     up(1, ch + 1, accA);
                     BADVANCE(0);
-                    BLOAD_STAGE(0, w2);
-                    if (active) {
 #pragma unroll
-                        for (int nt = 0; nt < NT; ++nt) x[nt] = DT::mfma32(w2[nt], hid.v, x[nt]);
+                    for (int half = 0; half < 2; ++half) {
+                        BLOAD_RANGE(0, w2, half * (NT / 2));
+                        if (active) {
+#pragma unroll
+                            for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
+                        }
                     }
                 } else {
                     BADVANCE(1);
-                    BLOAD_STAGE(1, w2);
-                    if (active) {
 #pragma unroll
-                        for (int nt = 0; nt < NT; ++nt) x[nt] = DT::mfma32(w2[nt], hid.v, x[nt]);
+                    for (int half = 0; half < 2; ++half) {
+                        BLOAD_RANGE(1, w2, half * (NT / 2));
+                        if (active) {
+#pragma unroll
+                            for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
+                        }
                     }
                 }
             }

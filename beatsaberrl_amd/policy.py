@@ -260,6 +260,10 @@ class NotePolicy(nn.Module):
         self.register_buffer("_body_idx32", self._body_idx.to(torch.int32), persistent=False)
         self.register_buffer("_head_sizes32", torch.tensor(self.head_sizes, dtype=torch.int32), persistent=False)
         self.sampler = "kernel"                 # "kernel": in-kernel Philox stream; "torch": torch's generator
+        # "auto": the 16-bit stream runs the whole block stack as one persistent kernel when the
+        # shape has one (ops.blocks_pack_size > 0); "off": always the per-op launch train
+        self.fused_blocks = "auto"
+        self._blocks_image = None               # [weights version, dtype, uint8 image]
         self._sample_calls = 0
         self.fp16 = False                       # True: 16-bit stream (python/policy.py:1085-1090)
         self.stream_dtype = torch.float16       # the 16-bit type used when fp16 is on
@@ -276,12 +280,48 @@ class NotePolicy(nn.Module):
         recast in place per weights version, so only the replicas are (re)built."""
         self.refresh_fp16_caches()
 
+    def _blocks_desc(self, dt):
+        b0 = self.blocks[0]
+        act = "gelu" if isinstance(b0.ffn[1], nn.GELU) else "relu"
+        return dict(d=self.embed, n_heads=self.n_heads, ffn=b0.ffn[0].out_features, T=self.n_lead + N_NOTE_SLOTS,
+                    act=act, n_queries=self.n_lead, dtype=dt)
+
+    def fused_blocks_ok(self, dt) -> bool:
+        """True when the block stack of this architecture has a fused kernel in dtype dt."""
+        if self.fused_blocks == "off" or dt is torch.float32:
+            return False
+        if self.fused_blocks != "auto":
+            raise ValueError(f"fused_blocks must be 'auto' or 'off', got {self.fused_blocks!r}")
+        return ops.blocks_pack_size(len(self.blocks), **self._blocks_desc(dt)) > 0
+
+    def blocks_image(self, dt):
+        """The fused block stack's weight image for the current weights version: rebuilt IN PLACE
+        (one cast + permute launch pair) when `bump_weights_version` has been called, so its
+        address is stable under a captured graph - the contract of the reference's flat replica
+        buffer (python/fp16_linear.py:249-346, :367-375)."""
+        desc = self._blocks_desc(dt)
+        c = self._blocks_image
+        dev = self.blocks[0].q_proj.weight.device
+        if c is None or c[1] is not dt or c[2].device != dev:
+            nbytes = ops.blocks_pack_size(len(self.blocks), **desc)
+            c = self._blocks_image = [-1, dt, torch.empty(nbytes, dtype=torch.uint8, device=dev)]
+        if c[0] != _fl._weights_version:
+            params = [[blk.ln_attn.weight, blk.ln_attn.bias, blk.q_proj.weight, blk.q_proj.bias, blk.k_proj.weight,
+                       blk.k_proj.bias, blk.v_proj.weight, blk.v_proj.bias, blk.out_proj.weight, blk.out_proj.bias,
+                       blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ffn[0].weight, blk.ffn[0].bias, blk.ffn[2].weight,
+                       blk.ffn[2].bias] for blk in self.blocks]
+            ops.blocks_pack(params, c[2], **desc)
+            c[0] = _fl._weights_version
+        return c[2]
+
     def refresh_fp16_caches(self):
         """Force every 16-bit replica up to date for the current weights version
         (python/policy.py:1448-1461): call after optimizer steps under a captured graph."""
         if not self.fp16:
             return
         dt = self.stream_dtype
+        if self.fused_blocks_ok(dt):
+            self.blocks_image(dt)
         for m in self.modules():
             if isinstance(m, nn.Linear):
                 _fl._replica(m.weight, dt)
@@ -337,12 +377,19 @@ class NotePolicy(nn.Module):
         x = torch.cat([tok_saber, tok_torso, tok_leg, tok_note], dim=1)   # (B, 29, d)
         if self.emb_ln is not None:
             x = self.emb_ln(x)
-        h = None
-        nb = len(self.blocks)
-        for i in range(nb - 1):
-            x, h = self.blocks[i](x, attn_bias, h=h, next_ln=self.blocks[i + 1].ln_attn)
-        x_res = x                                                          # the stream entering the final block
-        lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead)
+        if self.fused_blocks_ok(dt):
+            # the whole stack in one persistent kernel; x_res = the stream entering the final block
+            b0 = self.blocks[0]
+            lead, x_res = ops.blocks_forward(self.blocks_image(dt), x.contiguous(), attn_bias, len(self.blocks),
+                                             self.n_heads, b0.ffn[0].out_features,
+                                             "gelu" if isinstance(b0.ffn[1], nn.GELU) else "relu", self.n_lead)
+        else:
+            h = None
+            nb = len(self.blocks)
+            for i in range(nb - 1):
+                x, h = self.blocks[i](x, attn_bias, h=h, next_ln=self.blocks[i + 1].ln_attn)
+            x_res = x                                                      # the stream entering the final block
+            lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead)
         if self.final_ln is not None:
             lead = self.final_ln(lead)
         hfeat = self._trunk(lead.reshape(B, self.n_lead * d))

@@ -70,15 +70,23 @@ def _big(seed, **kw):
     return m, sd
 
 
-@pytest.mark.parametrize("kw,dtype,ffn", [
-    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "on"),
-    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "off"),
-    (dict(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4), "f16", "on"),
-    (dict(embed=128, trunk_dim=256, n_blocks=2, n_heads=4, n_gears=7, ffn_mult=2, emb_ln=True, final_ln=True,
-          note_geo=True, head_gears=tuple(7 if j in (8, 15) else 5 for j in range(29))), "bf16", "on"),
-    (dict(embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f32", "off"),
+_RAGGED = dict(embed=128, trunk_dim=256, n_blocks=2, n_heads=4, n_gears=7, ffn_mult=2, emb_ln=True, final_ln=True,
+               note_geo=True, head_gears=tuple(7 if j in (8, 15) else 5 for j in range(29)))
+
+
+# blocks = "auto": the block stack runs as one persistent kernel; "off": the per-op launch train
+@pytest.mark.parametrize("kw,dtype,ffn,blocks", [
+    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "on", "off"),
+    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "off", "off"),
+    (dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "off", "auto"),
+    (dict(embed=192, trunk_dim=384, n_blocks=6, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f16", "off", "auto"),
+    (dict(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4), "f16", "on", "off"),
+    (dict(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4), "f16", "off", "auto"),
+    (_RAGGED, "bf16", "on", "off"),
+    (_RAGGED, "bf16", "off", "auto"),
+    (dict(embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f32", "off", "auto"),
 ])
-def test_production_shapes_against_the_oracle(kw, dtype, ffn):
+def test_production_shapes_against_the_oracle(kw, dtype, ffn, blocks):
     m, sd = _big(5, **kw)
     m = m.to(DEV)
     obs = _make_obs(96, 7)
@@ -94,13 +102,15 @@ def test_production_shapes_against_the_oracle(kw, dtype, ffn):
     m.fp16 = True
     m.stream_dtype = torch.float16 if dtype == "f16" else torch.bfloat16
     m.fused_ffn = ffn
+    m.fused_blocks = blocks
+    assert m.fused_blocks_ok(m.stream_dtype) == (blocks == "auto")
     lg, v = m.forward_stacked(obs.to(DEV))
     lg, v = lg.cpu(), v.cpu()
     em_lg, em_v = nr.forward(sd, m.arch, obs, emulate=dtype)
     e_mine = (lg[live] - ref_lg[live]).abs().max().item()
     e_emul = (em_lg[live] - ref_lg[live]).abs().max().item()
     e_class = (lg[live] - em_lg[live]).abs().max().item()
-    print(f"\n[{dtype} ffn={ffn}] mine-vs-fp32 {e_mine:.2e}  emulated-vs-fp32 {e_emul:.2e}  mine-vs-emulated {e_class:.2e}")
+    print(f"\n[{dtype} ffn={ffn} blocks={blocks}] mine-vs-fp32 {e_mine:.2e}  emulated-vs-fp32 {e_emul:.2e}  mine-vs-emulated {e_class:.2e}")
     assert torch.equal(lg[~live], ref_lg[~live])
     assert e_mine <= max(1.25 * e_emul, 2e-3) and e_class <= max(e_emul, 2e-3)
     assert (v - ref_v).abs().max().item() <= max(1.25 * (em_v - ref_v).abs().max().item(), e_emul, 2e-3)
@@ -111,11 +121,13 @@ def test_production_shapes_against_the_oracle(kw, dtype, ffn):
         assert bool(((lg.argmax(-1) == ref_lg.argmax(-1)) | ~decided).all())
 
 
-def test_invariants_and_sampling_epilogue():
+@pytest.mark.parametrize("blocks", ["auto", "off"])
+def test_invariants_and_sampling_epilogue(blocks):
     m, sd = _big(9, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,
                  head_gears=tuple(7 if j == 4 else 5 for j in range(29)))
     m = m.to(DEV)
     m.fp16, m.fused_ffn = True, "on"
+    m.fused_blocks = blocks
     obs = _make_obs(50, 3)
     od = obs.to(DEV)
     lg, v = m.forward_stacked(od)
