@@ -100,7 +100,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
     __shared__ uint2 vx[4][2][TPH][64];       // V^T half fragments (this row tile's 4 keys per lane)
     extern __shared__ float4 bvl4[];          // fp32 vectors of every block
     const float* vlds = reinterpret_cast<const float*>(bvl4);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in an SGPR: branches on it are scalar
     const int r16 = lane & 15, g = lane >> 4;
     const int el = wave >> 1, rt = wave & 1;
     const float scale_l2e = (DH == 32 ? 0.17677669529663688110f : 0.14433756729740644113f) * 1.44269504088896340736f;
@@ -313,8 +314,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                 if (st == 0) attention(std::integral_constant<int, H - 1>{});                         // the last head completed in the previous stage
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
-                    BLOAD_HALF((3 * NT / 2 + st) & 1, wf, half);
-                    if (active) {
+                    if (active) {            // idle waves of the pruned block leave the LDS bandwidth to the others
+                        BLOAD_HALF((3 * NT / 2 + st) & 1, wf, half);
 #pragma unroll
                         for (int ci = 0; ci < KC / 2; ++ci)
 #pragma unroll
@@ -339,8 +340,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                 }
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
-                    BLOAD_HALF(par, wf, half);
                     if (active) {
+                        BLOAD_HALF(par, wf, half);
 #pragma unroll
                         for (int ci = 0; ci < KC / 2; ++ci)
 #pragma unroll
@@ -364,8 +365,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     BADVANCE(0);
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
-                        BLOAD_RANGE(0, w2, half * (NT / 2));
                         if (active) {
+                            BLOAD_RANGE(0, w2, half * (NT / 2));
 #pragma unroll
                             for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
                         }
@@ -374,8 +375,8 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     BADVANCE(1);
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
-                        BLOAD_RANGE(1, w2, half * (NT / 2));
                         if (active) {
+                            BLOAD_RANGE(1, w2, half * (NT / 2));
 #pragma unroll
                             for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
                         }
