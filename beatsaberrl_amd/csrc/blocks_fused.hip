@@ -20,6 +20,14 @@
 // lane for one query; softmax by in-lane + two cross-lane steps; P V as 16x16x32 MFMAs
 // over the 32 keys).
 //
+// What bounds it: every weight fragment (1 KB) read from LDS feeds ONE MFMA of the reading wave,
+// so a CU asks its LDS for 4 x 1 KB per 16 cycles = 256 B/clk against 128 B/clk delivered
+// (measured): the stack runs at the LDS read rate, ~750 cycles per 12 KB stage.  Giving a wave both
+// row tiles of an env halves that traffic but needs ~450 registers, i.e. one wave per SIMD; built
+// and measured (3-slot ring, fragment reads prefetched across the barrier), it came out level at
+// d = 128 and slower at d = 192 (register spills), each stage then waiting on the L2 latency of the
+// weight stream (~1500 cycles) with no second wave to cover it.
+//
 // Weights stream from L2 through a 2-slot LDS ring in stages of 2 * (d/32) fragments
 // (8 or 12 KB) shared by the 8 waves: loads issued three stages ahead into registers,
 // written to LDS one stage ahead, one barrier per stage.  All fp32 vectors (biases,
@@ -88,7 +96,7 @@ template <int D> struct Geo {
 // BLOAD_HALF: k chunks [half * KC/2, +KC/2) of both feature tiles, W[ntl * KC/2 + ci]; BLOAD_RANGE: fragments
 // [first, first + SF/2).
 #define BLOAD_HALF(par, W, half) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) \
-        W[f_] = BWFRAG(par, (f_ / (G::KC / 2)) * G::KC + (half) * (G::KC / 2) + f_ % (G::KC / 2))
+        W[f_] = BWFRAG(par, (half) * (G::SF / 2) + f_)
 #define BLOAD_RANGE(par, W, first) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) W[f_] = BWFRAG(par, (first) + f_)
 
 template <typename DT, int D, int DH, int ACT>
@@ -198,10 +206,12 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
             }
         };
 
-        for (int l = 0; l < a.n_layers; ++l) {
+        // one block; in the pruned final block only row tile 0 carries queries.  `pruned` is a compile-time
+        // constant so that the full blocks carry no branches around their MFMAs.
+        auto layer = [&](int l, auto pruned_) {
+            constexpr bool pruned = decltype(pruned_)::value;
             const float* lv = vlds + l * G::lv_size(a.F);
-            const bool pruned = a.n_queries > 0 && l == a.n_layers - 1;
-            const bool active = !pruned || rt == 0;          // wave-uniform: the pruned block's queries sit in row tile 0
+            const bool active = !pruned || rt == 0;          // wave-uniform
             if (pruned && a.x_res) store_rows(a.x_res, a.T, a.T);
 
             norm_to_frags(lv + G::LN1G, lv + G::LN1B);
@@ -383,11 +393,15 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     }
                 }
             }
-        }
+        };
+        const int n_full = a.n_queries > 0 ? a.n_layers - 1 : a.n_layers;
+        for (int l = 0; l < n_full; ++l) layer(l, std::false_type{});
+        if (a.n_queries > 0) layer(a.n_layers - 1, std::true_type{});
         if (a.n_queries > 0) { if (rt == 0) store_rows(a.x_out, a.n_queries, a.n_queries); }
         else store_rows(a.x_out, a.T, a.T);
     }
 }
+
 
 // ---- weight image ------------------------------------------------------------------
 struct BlkPackArgs {
@@ -410,20 +424,28 @@ __global__ __launch_bounds__(256) void blocks_pack_frags_kernel(BlkPackArgs a) {
     const int l = f / lfr, r = f % lfr;
     const auto& b = a.p.blk[l];
     const float* src; int ld, n, kbase = 0, c;
+    // inside a stage of two feature tiles the fragments are ordered (k half, tile, k chunk of the half),
+    // so the first SF / 2 fragments are what a consumer needs first
+    auto split = [&](int i, int& ntl, int& cc) {
+        const int half = i / (SF / 2), rem = i % (SF / 2);
+        ntl = rem / (KC / 2); cc = half * (KC / 2) + rem % (KC / 2);
+    };
     if (r < 3 * NT * KC) {
-        const int j = r / KC, hd = j / (3 * TPH), rr = j % (3 * TPH), part = rr / TPH, t = rr % TPH;
+        int ntl; split(r % SF, ntl, c);
+        const int j = 2 * (r / SF) + ntl, hd = j / (3 * TPH), rr = j % (3 * TPH), part = rr / TPH, t = rr % TPH;
         src = part == 0 ? b.q_w : part == 1 ? b.k_w : b.v_w;
-        ld = D; n = DH * hd + 16 * t + n16; c = r % KC;
+        ld = D; n = DH * hd + 16 * t + n16;
     } else if (r < 4 * NT * KC) {
         const int r2 = r - 3 * NT * KC;
-        src = b.out_w; ld = D; n = 16 * (r2 / KC) + n16; c = r2 % KC;
+        int ntl; split(r2 % SF, ntl, c);
+        src = b.out_w; ld = D; n = 16 * (2 * (r2 / SF) + ntl) + n16;
     } else {
         const int r3 = r - 4 * NT * KC, s3 = r3 / SF, i = r3 % SF, nch = a.F / 32;
         bool upw; int ch;
         if (s3 == 0) { upw = true; ch = 0; }
         else if (s3 == 2 * nch - 1) { upw = false; ch = nch - 1; }
         else { upw = ((s3 - 1) & 1) == 0; ch = (s3 - 1) / 2 + (upw ? 1 : 0); }
-        if (upw) { src = b.ffn0_w; ld = D; n = 32 * ch + 16 * (i / KC) + n16; c = i % KC; }
+        if (upw) { int ntl; split(i, ntl, c); src = b.ffn0_w; ld = D; n = 32 * ch + 16 * ntl + n16; }
         else { src = b.ffn2_w; ld = a.F; n = 16 * i + n16; c = 0; kbase = 32 * ch; }
     }
     float v[8];
@@ -479,11 +501,12 @@ void pack_launch(const BlkPackArgs& pa, int64_t nfrags, hipStream_t st) {
 template <typename DT, int D, int DH, int ACT>
 int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
     const size_t dyn = (size_t)a.n_layers * Geo<D>::lv_size(a.F) * sizeof(float);
+    const int64_t ntiles = (a.B + 3) / 4;
+    const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));
     auto kern = blocks_kernel<DT, D, DH, ACT>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
         return BSRL_UNSUPPORTED;
-    const int64_t ntiles = (a.B + 3) / 4;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(512), dyn, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(512), dyn, st, a);
     return BSRL_OK;
 }
 
