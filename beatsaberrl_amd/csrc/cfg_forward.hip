@@ -90,6 +90,17 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
         pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1; \
     } while (0)
 #define ADVANCE(par) do { if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
+// TAIL launch: a workgroup streams its 44 stages for ONE tile with little arithmetic per stage, so the
+// step time is the L2 latency of the weight stream divided by the stages in flight.  Four register
+// sets (q0..q3) keep four stages in flight instead of two: ADVANCE4(Q), Q = index of the stage about to
+// be consumed modulo 4, writes stage s+1 (set (Q+1) & 3) to the free slot and requests stage s+5 into it.
+#define ADVANCE4(Q) do { \
+        if ((Q) == 0) ADVANCE_P(0, q1a, q1b); else if ((Q) == 1) ADVANCE_P(1, q2a, q2b); \
+        else if ((Q) == 2) ADVANCE_P(0, q3a, q3b); else ADVANCE_P(1, q0a, q0b); \
+    } while (0)
+// ADV(sidx): sidx = stage index counted from the start of the block (HEAD / FULL: only its parity
+// matters) or from the start of the TAIL launch's own stage range (its value modulo 4 matters)
+#define ADV(sidx) do { if (MODE == MODE_TAIL) ADVANCE4((sidx) & 3); else ADVANCE((sidx) & 1); } while (0)
 #define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[par][(f) * 64 + lane]))
 // all 8 fragments of the current stage -> registers in one burst of LDS reads (one wait instead of 8)
 #define LOAD_STAGE(par, W) s16x8 W[STAGE_FRAGS]; _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = WFRAG(par, f_)
@@ -118,14 +129,23 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 
     const uint4* img = a.frags;
     uint4 pr0a, pr0b, pr1a, pr1b;
+    uint4 q0a, q0b, q1a, q1b, q2a, q2b, q3a, q3b;       // TAIL launch only
     int pnext;
-    {   // prologue: first stage -> LDS slot 0; the next two in flight (stage counts per mode are even)
+    {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
         const int s0 = a.s_begin;
         const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
-        pr1a = img[(int64_t)(s0 + 1) * STAGE_U4 + tid]; pr1b = img[(int64_t)(s0 + 1) * STAGE_U4 + tid + 256];
+        if (MODE == MODE_TAIL) {
+            q1a = img[(int64_t)(s0 + 1) * STAGE_U4 + tid]; q1b = img[(int64_t)(s0 + 1) * STAGE_U4 + tid + 256];
+            q2a = img[(int64_t)(s0 + 2) * STAGE_U4 + tid]; q2b = img[(int64_t)(s0 + 2) * STAGE_U4 + tid + 256];
+            q3a = img[(int64_t)(s0 + 3) * STAGE_U4 + tid]; q3b = img[(int64_t)(s0 + 3) * STAGE_U4 + tid + 256];
+            q0a = img[(int64_t)(s0 + 4) * STAGE_U4 + tid]; q0b = img[(int64_t)(s0 + 4) * STAGE_U4 + tid + 256];
+        } else {
+            pr1a = img[(int64_t)(s0 + 1) * STAGE_U4 + tid]; pr1b = img[(int64_t)(s0 + 1) * STAGE_U4 + tid + 256];
+        }
         lds[0][tid] = s0a; lds[0][tid + 256] = s0b;
-        pr0a = img[(int64_t)(s0 + 2) * STAGE_U4 + tid]; pr0b = img[(int64_t)(s0 + 2) * STAGE_U4 + tid + 256];
-        pnext = s0 + 3 >= a.s_end ? a.s_begin + (s0 + 3 - a.s_end) : s0 + 3;
+        if (MODE != MODE_TAIL) { pr0a = img[(int64_t)(s0 + 2) * STAGE_U4 + tid]; pr0b = img[(int64_t)(s0 + 2) * STAGE_U4 + tid + 256]; }
+        constexpr int AHEAD = MODE == MODE_TAIL ? 5 : 3;
+        pnext = s0 + AHEAD >= a.s_end ? a.s_begin + (s0 + AHEAD - a.s_end) : s0 + AHEAD;
         // No global load other than the weight pipeline may sit in the steady state: vmcnt retires
         // in order, so waiting on a late bias load would also drain the prefetches issued before it.
         const int nv4 = vec_floats(a.n_layers, a.F) / 4;
@@ -264,7 +284,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             add_bias(lv + LV_BOUT);
 #pragma unroll
             for (int st = 0; st < NT / 2; ++st) {
-                ADVANCE(st & 1);            // 12 stages precede in the block: parity restarts even
+                ADV(st);                    // 12 stages precede in the block (parity restarts even); TAIL starts here
                 LOAD_STAGE(st & 1, wf);
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
@@ -301,8 +321,11 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             };
             if (RT == 1) {
                 // single row tile (TAIL launch): plain chunk loop, no split
+                // stage indices count from the TAIL launch's first stage: 4 output-projection stages precede,
+                // chunk ch's stages are W1(ch+1) = 5 + 2 ch and W2(ch) = 6 + 2 ch (the last chunk: W2 = 3 + 2 nch);
+                // the hidden width is a multiple of 64 here, so two chunks advance the index by 4
                 {
-                    ADVANCE(0);
+                    ADV(4);
                     LOAD_STAGE(0, w1);
                     up_init(0, accA);
 #pragma unroll
@@ -310,30 +333,34 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 #pragma unroll
                         for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
                 }
-                for (int ch = 0; ch < nch; ++ch) {
-                    act4(accA[0][0], hidA[0], 0); act4(accA[1][0], hidA[0], 1);
-                    if (ch + 1 < nch) {
-                        ADVANCE(1);
-                        LOAD_STAGE(1, w1);
-                        up_init(ch + 1, accA);
+                for (int ch2 = 0; ch2 < nch; ch2 += 2) {
 #pragma unroll
-                        for (int c = 0; c < KC; ++c)
+                    for (int o = 0; o < 2; ++o) {
+                        const int ch = ch2 + o;
+                        act4(accA[0][0], hidA[0], 0); act4(accA[1][0], hidA[0], 1);
+                        if (ch + 1 < nch) {
+                            ADV(5 + 2 * o);
+                            LOAD_STAGE(1, w1);
+                            up_init(ch + 1, accA);
 #pragma unroll
-                            for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
-                        ADVANCE(0);
-                    } else {
-                        ADVANCE(1);
+                            for (int c = 0; c < KC; ++c)
+#pragma unroll
+                                for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
+                            ADV(6 + 2 * o);
+                        } else {
+                            ADV(3);             // o == 1: the last chunk's down-projection stage, index 3 + 2 nch
+                        }
+                        s16x8 w2[STAGE_FRAGS];
+                        if (ch + 1 < nch) {
+#pragma unroll
+                            for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(0, f);
+                        } else {
+#pragma unroll
+                            for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(1, f);
+                        }
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
                     }
-                    s16x8 w2[STAGE_FRAGS];
-                    if (ch + 1 < nch) {
-#pragma unroll
-                        for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(0, f);
-                    } else {
-#pragma unroll
-                        for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(1, f);
-                    }
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
                 }
             } else {
                 {   // prologue: up-projection of chunk 0, activation of its lower row tiles
@@ -418,7 +445,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             constexpr int NR = sizeof(rf) / sizeof(rf[0]);
 #pragma unroll
             for (int st = 0; st < HEAD_STAGES; ++st) {
-                ADVANCE(st & 1);            // an even number of stages precedes the readout
+                ADV(st);                    // a multiple of 4 stages precedes the readout in the TAIL launch, an even number otherwise
                 LOAD_STAGE(st & 1, wf);
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
@@ -739,7 +766,8 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
     a.ws = static_cast<uint32_t*>(workspace);
-    const bool pruned = workspace && workspace_bytes >= bsrl_cfg_workspace_size(d, B);
+    // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
+    const bool pruned = workspace && workspace_bytes >= bsrl_cfg_workspace_size(d, B) && d->ffn % 64 == 0;
     if (workspace && !bsrl_aligned(workspace, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: workspace must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
