@@ -443,6 +443,10 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
         //      row r16 of tile i being env env_base + i * 16 + r16 (stored when r16 < rows_valid) ----
         auto heads = [&](auto& rf, int64_t env_base, int rows_valid, const float* fvp) {
             constexpr int NR = sizeof(rf) / sizeof(rf[0]);
+            // The outputs stay in registers until the last stage has been consumed: stores count in the same
+            // in-order vmcnt queue as the weight prefetches, so a store issued inside the stage loop would make
+            // the next stage's wait sit out an HBM write.
+            f32x4 res[HEAD_TILES][NR];
 #pragma unroll
             for (int st = 0; st < HEAD_STAGES; ++st) {
                 ADV(st);                    // a multiple of 4 stages precedes the readout in the TAIL launch, an even number otherwise
@@ -456,13 +460,29 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         f32x4 acc = {b.x, b.y, b.z, b.w};
 #pragma unroll
                         for (int c = 0; c < KC; ++c) acc = DT::mfma32(wf[ntl * KC + c], rf[i][c].v, acc);
-                        const int64_t env = env_base + i * 16 + r16;
-                        if (r16 < rows_valid && env < a.B) {
+                        res[nt][i] = acc;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int64_t env = env_base + i * 16 + r16;
+                if (r16 < rows_valid && env < a.B) {
+                    // a lane holds 4 consecutive outputs of its row: one 4-dword store (rows are only dword-aligned:
+                    // the type says so and the compiler picks the widest store the target allows at that alignment)
+                    typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+                    float* lrow = a.logits + env * a.n_logits;
+#pragma unroll
+                    for (int nt = 0; nt < HEAD_TILES; ++nt) {
+                        const int col0 = 16 * nt + 4 * g;
+                        if (col0 + 3 < a.n_logits) {
+                            *reinterpret_cast<f32x4_a4*>(lrow + col0) = (f32x4_a4){res[nt][i][0], res[nt][i][1], res[nt][i][2], res[nt][i][3]};
+                        } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
-                                const int col = 16 * nt + 4 * g + e;
-                                if (col < a.n_logits) a.logits[env * a.n_logits + col] = acc[e];
-                                else if (col == a.n_logits) a.value[env] = acc[e];
+                                const int col = col0 + e;
+                                if (col < a.n_logits) lrow[col] = res[nt][i][e];
+                                else if (col == a.n_logits) a.value[env] = res[nt][i][e];
                             }
                         }
                     }
