@@ -113,6 +113,9 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 //   workspace; TAIL re-tiles those rows 16 envs per MFMA tile and runs the last block's
 //   output projection + FFN and the 29*K + 1 output projection on them.
 enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
+// Envs per 16-row MFMA tile in the TAIL launch.  Measured: 8 (twice the waves in flight, twice the weight stream)
+// takes 30 us against 24 us with full tiles at B = 16384.
+constexpr int TAIL_ENVS = 16;
 constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
 
 template <typename DT, int RT, int ACT, int MODE>
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
-    constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? 16 : 1;     // envs per 16-row MFMA tile
+    constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? TAIL_ENVS : 1;     // envs per 16-row MFMA tile
     constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
     const int64_t ntiles = (a.B + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
@@ -587,7 +590,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             const float* lv = vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                int64_t env = env0 + rt * 16 + r16; env = env < a.B ? env : a.B - 1;
+                int64_t env = env0 + rt * TAIL_ENVS + r16; env = env < a.B ? env : a.B - 1;     // rows >= TAIL_ENVS: never stored
 #pragma unroll
                 for (int i = 0; i < 4; ++i) kmask[rt][i] = 0.f;
                 const uint4* src = reinterpret_cast<const uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             proj_and_ffn(lv);
             Frag8 yf[RT][KC];
             norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
-            heads(yf, env0, 16, fv);
+            heads(yf, env0, TAIL_ENVS, fv);
         }
     }
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
@@ -708,7 +711,7 @@ int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
     }
-    const int64_t per_wg = 4 * RT * (MODE == MODE_TAIL ? 16 : 1);
+    const int64_t per_wg = 4 * RT * (MODE == MODE_TAIL ? TAIL_ENVS : 1);
     const int64_t ntiles = (a.B + per_wg - 1) / per_wg;
     const int64_t resident = (int64_t)cus * (RT <= 2 ? 2 : 1);
     hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < resident ? ntiles : resident)), dim3(256), dyn, st, a);
