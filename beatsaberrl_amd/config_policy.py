@@ -9,13 +9,17 @@ architecture is the textbook pre-LN transformer of the benchmark configs:
 one Linear per token type, L blocks, one packed (29*K + 1, d) output matrix
 whose last row is the value.
 
-Two routes, both entirely on the C-ABI kernels:
-  * "ops":   one kernel per op (tokenizer, LayerNorm, packed QKV linear,
-             attention, out-proj + residual, LayerNorm, FFN up + act,
-             FFN down + residual, heads) - any supported shape and dtype;
-  * "fused": the whole forward in one persistent kernel reading a packed
-             weight image (16-bit dtypes, shapes the kernel is built for).
-`route="auto"` takes "fused" when the library supports the shape."""
+Three routes, all entirely on the C-ABI kernels:
+  * "ops":    one kernel per op (tokenizer, LayerNorm, packed QKV linear,
+              attention, out-proj + residual, LayerNorm, FFN up + act,
+              FFN down + residual, heads) - any supported shape and dtype;
+  * "fused":  the whole forward in one persistent kernel reading a packed
+              weight image (16-bit dtypes, T = 16 / d = 128);
+  * "blocks": tokenizer kernel, then the whole block stack in one persistent
+              kernel (final block pruned to token 0), then final LayerNorm and
+              heads on the B token-0 rows (16-bit dtypes, T <= 32, d = 128 / 256).
+`route="auto"` takes "fused", else "blocks", else "ops", by what the library
+supports for the shape."""
 from __future__ import annotations
 
 import ctypes
@@ -65,7 +69,8 @@ class ConfigPolicy(nn.Module):
         self.final_ln = FusedLayerNorm(d) if final_ln else None
         self.heads = nn.Linear(d, self.n_out)
         self.dtype = dtype            # stream dtype: "f32" | "f16" | "bf16"
-        self.route = route            # "auto" | "ops" | "fused"
+        self.route = route            # "auto" | "ops" | "fused" | "blocks"
+        self._blocks_image = None     # (key, uint8 image) of the fused block stack
         self._version = 0             # bumped by bump_weights_version()
         self._replica = None          # (version, dtype, device) -> 16-bit weight copies
         self._packed = None           # (version, dtype, device) -> fused-kernel weight image
@@ -123,6 +128,29 @@ class ConfigPolicy(nn.Module):
         if dt is torch.float32:
             return False
         return _lib.load().bsrl_cfg_pack_size(ctypes.byref(self._desc(dt))) > 0
+
+    def _blocks_shape(self, dt):
+        return dict(d=self.d, n_heads=self.n_heads, ffn=self.ffn_dim, T=self.T, act=self.act, n_queries=1, dtype=dt)
+
+    def blocks_supported(self, dt=None) -> bool:
+        dt = dt or _DTYPES[self.dtype]
+        if dt is torch.float32:
+            return False
+        return ops.blocks_pack_size(self.n_layers, **self._blocks_shape(dt)) > 0
+
+    def blocks_image(self, dt, device):
+        """Weight image of the fused block stack for the current weights version."""
+        key = (self._version, dt, str(device))
+        if self._blocks_image is not None and self._blocks_image[0] == key:
+            return self._blocks_image[1]
+        shape = self._blocks_shape(dt)
+        img = torch.empty(ops.blocks_pack_size(self.n_layers, **shape), dtype=torch.uint8, device=device)
+        params = [[b.ln_attn.weight, b.ln_attn.bias, b.q_proj.weight, b.q_proj.bias, b.k_proj.weight, b.k_proj.bias,
+                   b.v_proj.weight, b.v_proj.bias, b.out_proj.weight, b.out_proj.bias, b.ln_ffn.weight, b.ln_ffn.bias,
+                   b.ffn[0].weight, b.ffn[0].bias, b.ffn[2].weight, b.ffn[2].bias] for b in self.blocks]
+        ops.blocks_pack(params, img, **shape)
+        self._blocks_image = (key, img)
+        return img
 
     def packed_image(self, dt, device):
         """The fused kernel's weight image for the current weights version
@@ -184,11 +212,13 @@ class ConfigPolicy(nn.Module):
         dt = _DTYPES[self.dtype]
         route = route or self.route
         if route == "auto":
-            route = "fused" if self.fused_supported(dt) else "ops"
+            route = "fused" if self.fused_supported(dt) else "blocks" if self.blocks_supported(dt) else "ops"
         if route == "fused":
             return self._forward_fused(obs, n_valid, dt)
+        if route == "blocks":
+            return self._forward_blocks(obs, n_valid, dt)
         if route != "ops":
-            raise ValueError(f"route must be auto/ops/fused, got {route!r}")
+            raise ValueError(f"route must be auto/ops/fused/blocks, got {route!r}")
         return self._forward_ops(obs, n_valid, dt)
 
     def forward(self, obs, n_valid=None):
@@ -220,6 +250,27 @@ class ConfigPolicy(nn.Module):
         if not _lib.check(rc, "bsrl_cfg_forward"):
             raise ops.Unsupported("bsrl_cfg_forward")
         return logits.view(B, N_ACTION_HEADS, self.n_gears), value
+
+    def _forward_blocks(self, obs, n_valid, dt):
+        B, T = obs.shape[0], self.T
+        r = self._replicas(dt, obs.device)
+        if obs.dtype not in (torch.float32, dt):
+            obs = obs.float()
+        x = ops.cfg_embed(obs, r["prop_w"], r["prop_b"], r["obj_w"], r["obj_b"], T, dt)       # (B, T, d)
+        # additive key bias of the padding mask: tokens 0..n_valid attendable (exp(-16384) == 0 in fp32)
+        if n_valid is None:
+            bias = torch.zeros(B, T, device=obs.device, dtype=dt)
+        else:
+            pos = torch.arange(T, device=obs.device, dtype=torch.int32)
+            bias = ((pos[None, :] > n_valid[:, None]).to(dt) * -16384.0).contiguous()
+        h, _ = ops.blocks_forward(self.blocks_image(dt, obs.device), x, bias, self.n_layers, self.n_heads, self.ffn_dim,
+                                  self.act, 1, want_res=False)                                 # (B, 1, d)
+        h = h.view(B, self.d)
+        if self.final_ln is not None:
+            h = ops.ln_fwd(h, self.final_ln.weight, self.final_ln.bias, self.final_ln.eps)
+        n_log = N_ACTION_HEADS * self.n_gears
+        logits, value = ops.linear(h, r["heads_w"], r["heads_b"], out_dtype=torch.float32, split=n_log)
+        return logits.view(B, N_ACTION_HEADS, self.n_gears), value.view(B)
 
     def _forward_ops(self, obs, n_valid, dt):
         B, T, d = obs.shape[0], self.T, self.d

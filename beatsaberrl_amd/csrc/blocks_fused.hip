@@ -1,7 +1,7 @@
 // The transformer block stack of the policy in ONE persistent kernel for gfx950.
 //
-// Shape class: up to 32 tokens per env (NotePolicy: 29), d = 128 or 192 as 4 heads of 32 or
-// 48, FFN width a multiple of 32, ReLU or GELU, fp16 or bf16 operands with fp32 accumulate.
+// Shape class: up to 32 tokens per env (NotePolicy: 29), d = 128 / 192 / 256 as 4 x 32, 4 x 48 or
+// 8 x 32 heads, FFN width a multiple of 32, ReLU or GELU, fp16 or bf16 operands with fp32 accumulate.
 // Replaces, for the block stack of NotePolicy._forward_stacked (python/policy.py:1262-1306),
 // the per-block launch train of Block.forward (python/policy.py:524-715): LayerNorm, packed
 // q|k|v projection, attention, output projection + residual, LayerNorm, FFN + residual,
@@ -60,12 +60,15 @@ __device__ __forceinline__ void blk_barrier() { asm volatile("s_waitcnt lgkmcnt(
 
 // compile-time loop: the body sees its index as a constant (the loop unroller gives up on the
 // larger bodies, and register arrays indexed by the loop variable would then live in scratch)
-template <int I, int N, typename Fn> __device__ __forceinline__ void static_for(Fn&& fn) {
+template <int I, int N, typename Fn> __device__ __forceinline__ void static_for(Fn&& fn) {   // fn: an always_inline lambda
     if constexpr (I < N) { fn(std::integral_constant<int, I>{}); static_for<I + 1, N>(fn); }
 }
 
 template <int D> struct Geo {
     static constexpr int NT = D / 16, KC = D / 32, SF = 2 * KC;          // feature tiles, k chunks, fragments per stage
+    // a stage is consumed in NB bursts of FB fragments (KB k chunks of both feature tiles): one burst of LDS
+    // reads, then its MFMAs; bursts are sized to keep the fragment registers at 16-24 VGPRs
+    static constexpr int NB = SF > 12 ? 4 : 2, FB = SF / NB, KB = KC / NB;
     static constexpr int STAGE_U2 = SF * 128;                             // uint2 per stage
     static constexpr int U2PT = STAGE_U2 / 512;                           // uint2 per thread per stage (2 or 3)
     __host__ __device__ static constexpr int layer_stages(int F) { return 3 * NT / 2 + NT / 2 + 2 * (F / 32); }
@@ -78,31 +81,33 @@ template <int D> struct Geo {
 // Weight-stage pipeline: stage s lives in ring slot s & 1; its global loads were issued three
 // stage-steps earlier into the register set of the same parity.  The registers are plain named
 // locals (an indexed array would live in scratch and force a wait right after each load).
-#define BADVANCE_P(P, RA, RB, RC) do { \
+#define BADVANCE_P(P, RA, RB, RC, RD) do { \
         blk_barrier();                                   /* stage s complete in slot P; slot 1-P free */ \
         ring[1 - (P)][tid] = RA; \
         ring[1 - (P)][tid + 512] = RB; \
-        if (G::U2PT == 3) ring[1 - (P)][tid + 1024] = RC; \
+        if (G::U2PT >= 3) ring[1 - (P)][tid + 1024] = RC; \
+        if (G::U2PT == 4) ring[1 - (P)][tid + 1536] = RD; \
         const uint2* src_ = img + (int64_t)pnext * G::STAGE_U2 + tid; \
         RA = src_[0]; \
         RB = src_[512]; \
-        if (G::U2PT == 3) RC = src_[1024]; \
+        if (G::U2PT >= 3) RC = src_[1024]; \
+        if (G::U2PT == 4) RD = src_[1536]; \
         pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1; \
     } while (0)
-#define BADVANCE(par) do { if (par) BADVANCE_P(1, pr0a, pr0b, pr0c); else BADVANCE_P(0, pr1a, pr1b, pr1c); } while (0)
+#define BADVANCE(par) do { if (par) BADVANCE_P(1, pr0a, pr0b, pr0c, pr0d); else BADVANCE_P(0, pr1a, pr1b, pr1c, pr1d); } while (0)
 #define BWFRAG(par, f) (__builtin_bit_cast(s16x8, reinterpret_cast<const uint4*>(ring[par])[(f) * 64 + lane]))
 // every fragment of the current stage -> registers in one burst of LDS reads (one wait instead of one per MFMA)
-// half a stage (SF / 2 fragments) -> registers in one burst of LDS reads (one wait instead of one per MFMA).
-// BLOAD_HALF: k chunks [half * KC/2, +KC/2) of both feature tiles, W[ntl * KC/2 + ci]; BLOAD_RANGE: fragments
-// [first, first + SF/2).
-#define BLOAD_HALF(par, W, half) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) \
-        W[f_] = BWFRAG(par, (half) * (G::SF / 2) + f_)
-#define BLOAD_RANGE(par, W, first) s16x8 W[G::SF / 2]; _Pragma("unroll") for (int f_ = 0; f_ < G::SF / 2; ++f_) W[f_] = BWFRAG(par, (first) + f_)
+// one burst of a stage (FB fragments) -> registers in one run of LDS reads (one wait instead of one per MFMA).
+// BLOAD_BURST: burst b of a two-tile stage, W[ntl * KB + ci] = k chunk b * KB + ci of tile ntl;
+// BLOAD_RANGE: fragments [first, first + FB).
+#define BLOAD_BURST(par, W, b) s16x8 W[G::FB]; _Pragma("unroll") for (int f_ = 0; f_ < G::FB; ++f_) W[f_] = BWFRAG(par, (b) * G::FB + f_)
+#define BLOAD_RANGE(par, W, first) s16x8 W[G::FB]; _Pragma("unroll") for (int f_ = 0; f_ < G::FB; ++f_) W[f_] = BWFRAG(par, (first) + f_)
 
 template <typename DT, int D, int DH, int ACT>
 __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
     typedef Geo<D> G;
     constexpr int NT = G::NT, KC = G::KC, H = D / DH, TPH = DH / 16;     // TPH: 16-feature tiles per head (2 or 3)
+    constexpr int NB = G::NB, KB = G::KB, FB = G::FB;
     __shared__ __align__(16) uint2 ring[2][G::STAGE_U2];
     __shared__ uint2 kx[4][2][TPH][64];       // [env][row tile][feature tile of the head][lane]: K fragments
     __shared__ uint2 vx[4][2][TPH][64];       // V^T half fragments (this row tile's 4 keys per lane)
@@ -116,18 +121,18 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
     const int64_t ntiles = (a.B + 3) / 4;
 
     const uint2* img = a.frags;
-    uint2 pr0a, pr0b, pr0c = make_uint2(0, 0), pr1a, pr1b, pr1c = make_uint2(0, 0);
+    const uint2 z2 = make_uint2(0, 0);
+    uint2 pr0a, pr0b, pr0c = z2, pr0d = z2, pr1a, pr1b, pr1c = z2, pr1d = z2;
     int pnext;
     {   // prologue: stage 0 -> ring slot 0; stages 1 and 2 in flight (every block has an even stage count >= 4)
-        const uint2 s0a = img[tid], s0b = img[tid + 512];
-        uint2 s0c = make_uint2(0, 0);
-        if (G::U2PT == 3) s0c = img[tid + 1024];
+#pragma unroll
+        for (int u = 0; u < G::U2PT; ++u) ring[0][tid + 512 * u] = img[tid + 512 * u];
         pr1a = img[G::STAGE_U2 + tid]; pr1b = img[G::STAGE_U2 + tid + 512];
-        if (G::U2PT == 3) pr1c = img[G::STAGE_U2 + tid + 1024];
-        ring[0][tid] = s0a; ring[0][tid + 512] = s0b;
-        if (G::U2PT == 3) ring[0][tid + 1024] = s0c;
+        if (G::U2PT >= 3) pr1c = img[G::STAGE_U2 + tid + 1024];
+        if (G::U2PT == 4) pr1d = img[G::STAGE_U2 + tid + 1536];
         pr0a = img[2 * G::STAGE_U2 + tid]; pr0b = img[2 * G::STAGE_U2 + tid + 512];
-        if (G::U2PT == 3) pr0c = img[2 * G::STAGE_U2 + tid + 1024];
+        if (G::U2PT >= 3) pr0c = img[2 * G::STAGE_U2 + tid + 1024];
+        if (G::U2PT == 4) pr0d = img[2 * G::STAGE_U2 + tid + 1536];
         pnext = 3 % a.total_stages;
         const int nv4 = a.n_layers * G::lv_size(a.F) / 4;
         for (int i = tid; i < nv4; i += 512) bvl4[i] = reinterpret_cast<const float4*>(a.vec)[i];
@@ -162,7 +167,7 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                 }
         }
 
-        auto norm_to_frags = [&](const float* gptr, const float* bptr) {
+        auto norm_to_frags = [&](const float* gptr, const float* bptr) __attribute__((always_inline)) {
             // one pass: var = E[x^2] - mean^2 clamped at 0 (python/beat_arena_env/csrc/layer_norm.cu:14-21)
             float s = 0.f, q = 0.f;
 #pragma unroll
@@ -186,14 +191,14 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                 hf[nt >> 1].w[(nt & 1) * 2 + 1] = bpack2<DT>(y2, y3);
             }
         };
-        auto add_bias = [&](const float* bptr) {
+        auto add_bias = [&](const float* bptr) __attribute__((always_inline)) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 b = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
                 x[nt][0] += b.x; x[nt][1] += b.y; x[nt][2] += b.z; x[nt][3] += b.w;
             }
         };
-        auto store_rows = [&](u16* dst, int rows_per_env, int nrows_valid) {
+        auto store_rows = [&](u16* dst, int rows_per_env, int nrows_valid) __attribute__((always_inline)) {
             // this wave's rows < nrows_valid of its env, 4 consecutive features (8 bytes) per lane and tile
             if (env < a.B && row < nrows_valid) {
                 u16* o = dst + (env * rows_per_env + row) * D;
@@ -208,7 +213,7 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 
         // one block; in the pruned final block only row tile 0 carries queries.  `pruned` is a compile-time
         // constant so that the full blocks carry no branches around their MFMAs.
-        auto layer = [&](int l, auto pruned_) {
+        auto layer = [&](int l, auto pruned_) __attribute__((always_inline)) {
             constexpr bool pruned = decltype(pruned_)::value;
             const float* lv = vlds + l * G::lv_size(a.F);
             const bool active = !pruned || rt == 0;          // wave-uniform
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
             uint2 q[2][TPH];                                  // Q fragments, double-buffered by head parity
 
             // attention of head hd for this wave's 16 queries over the env's 32 key slots
-            auto attention = [&](auto hd_) {
+            auto attention = [&](auto hd_) __attribute__((always_inline)) {
                 constexpr int hd = decltype(hd_)::value;
                 if (!active) return;
                 f32x4 sc[2];
@@ -273,7 +278,7 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 
             // ---- packed q|k|v projection: 3 * NT feature tiles in head-major order
             //      [q tiles | k tiles | v tiles] per head, two tiles per stage ----
-            static_for<0, 3 * NT / 2>([&](auto st_) {
+            static_for<0, 3 * NT / 2>([&](auto st_) __attribute__((always_inline)) {
                 constexpr int st = decltype(st_)::value;
                 BADVANCE(st & 1);
                 // a head whose last tile was computed in an earlier stage is complete in LDS after this barrier
@@ -291,16 +296,16 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
                 }
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    BLOAD_HALF(st & 1, wf, half);                      // k chunks [half * KC/2, +KC/2) of both tiles
+                for (int half = 0; half < NB; ++half) {
+                    BLOAD_BURST(st & 1, wf, half);                     // k chunks [half * KB, +KB) of both tiles
 #pragma unroll
-                    for (int ci = 0; ci < KC / 2; ++ci)
+                    for (int ci = 0; ci < KB; ++ci)
 #pragma unroll
                         for (int ntl = 0; ntl < 2; ++ntl) {
-                            const int c = half * (KC / 2) + ci;
+                            const int c = half * KB + ci;
                             const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
                             if (part == 0 && !active) continue;        // the pruned block needs no queries from row tile 1
-                            const s16x8 w = wf[ntl * (KC / 2) + ci];
+                            const s16x8 w = wf[ntl * KB + ci];
                             if (part < 2) acc[ntl] = DT::mfma32(w, hf[c].v, acc[ntl]);
                             else acc[ntl] = DT::mfma32(hf[c].v, w, acc[ntl]);   // V^T: operand roles swapped
                         }
@@ -318,22 +323,22 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 
             // ---- output projection onto the residual (NT / 2 stages) ----
             if (active) add_bias(lv + G::BOUT);
-#pragma unroll
-            for (int st = 0; st < NT / 2; ++st) {
+            static_for<0, NT / 2>([&](auto st_) __attribute__((always_inline)) {
+                constexpr int st = decltype(st_)::value;
                 BADVANCE((3 * NT / 2 + st) & 1);
-                if (st == 0) attention(std::integral_constant<int, H - 1>{});                         // the last head completed in the previous stage
+                if constexpr (st == 0) attention(std::integral_constant<int, H - 1>{});               // the last head completed in the previous stage
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int half = 0; half < NB; ++half) {
                     if (active) {            // idle waves of the pruned block leave the LDS bandwidth to the others
-                        BLOAD_HALF((3 * NT / 2 + st) & 1, wf, half);
+                        BLOAD_BURST((3 * NT / 2 + st) & 1, wf, half);
 #pragma unroll
-                        for (int ci = 0; ci < KC / 2; ++ci)
+                        for (int ci = 0; ci < KB; ++ci)
 #pragma unroll
                             for (int ntl = 0; ntl < 2; ++ntl)
-                                x[2 * st + ntl] = DT::mfma32(wf[ntl * (KC / 2) + ci], of[half * (KC / 2) + ci].v, x[2 * st + ntl]);
+                                x[2 * st + ntl] = DT::mfma32(wf[ntl * KB + ci], of[half * KB + ci].v, x[2 * st + ntl]);
                     }
                 }
-            }
+            });
 
             // ---- LayerNorm + FFN: stage order W1(0), {W1(ch+1), W2(ch)}..., W2(last); the hidden of a
             //      32-unit chunk lives in two accumulators, activated and packed into one operand fragment ----
@@ -342,21 +347,21 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
             if (active) { norm_to_frags(lv + G::LN2G, lv + G::LN2B); add_bias(lv + G::b2(a.F)); }
             const int nch = a.F / 32;
             f32x4 accA[2];
-            auto up = [&](int par, int ch, f32x4 (&acc)[2]) {
+            auto up = [&](int par, int ch, f32x4 (&acc)[2]) __attribute__((always_inline)) {
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
                     const float4 b = *reinterpret_cast<const float4*>(lv + G::B1 + 32 * ch + 16 * ntl + 4 * g);
                     acc[ntl] = (f32x4){b.x, b.y, b.z, b.w};
                 }
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int half = 0; half < NB; ++half) {
                     if (active) {
-                        BLOAD_HALF(par, wf, half);
+                        BLOAD_BURST(par, wf, half);
 #pragma unroll
-                        for (int ci = 0; ci < KC / 2; ++ci)
+                        for (int ci = 0; ci < KB; ++ci)
 #pragma unroll
                             for (int ntl = 0; ntl < 2; ++ntl)
-                                acc[ntl] = DT::mfma32(wf[ntl * (KC / 2) + ci], hf[half * (KC / 2) + ci].v, acc[ntl]);
+                                acc[ntl] = DT::mfma32(wf[ntl * KB + ci], hf[half * KB + ci].v, acc[ntl]);
                     }
                 }
             };
@@ -374,21 +379,21 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
                     up(1, ch + 1, accA);
                     BADVANCE(0);
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
+                    for (int half = 0; half < NB; ++half) {
                         if (active) {
-                            BLOAD_RANGE(0, w2, half * (NT / 2));
+                            BLOAD_RANGE(0, w2, half * FB);
 #pragma unroll
-                            for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
+                            for (int i = 0; i < FB; ++i) x[half * FB + i] = DT::mfma32(w2[i], hid.v, x[half * FB + i]);
                         }
                     }
                 } else {
                     BADVANCE(1);
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
+                    for (int half = 0; half < NB; ++half) {
                         if (active) {
-                            BLOAD_RANGE(1, w2, half * (NT / 2));
+                            BLOAD_RANGE(1, w2, half * FB);
 #pragma unroll
-                            for (int i = 0; i < NT / 2; ++i) x[half * (NT / 2) + i] = DT::mfma32(w2[i], hid.v, x[half * (NT / 2) + i]);
+                            for (int i = 0; i < FB; ++i) x[half * FB + i] = DT::mfma32(w2[i], hid.v, x[half * FB + i]);
                         }
                     }
                 }
@@ -424,11 +429,11 @@ __global__ __launch_bounds__(256) void blocks_pack_frags_kernel(BlkPackArgs a) {
     const int l = f / lfr, r = f % lfr;
     const auto& b = a.p.blk[l];
     const float* src; int ld, n, kbase = 0, c;
-    // inside a stage of two feature tiles the fragments are ordered (k half, tile, k chunk of the half),
-    // so the first SF / 2 fragments are what a consumer needs first
+    // inside a stage of two feature tiles the fragments are ordered (burst, tile, k chunk of the burst):
+    // consecutive runs of FB fragments are what a consumer reads together
     auto split = [&](int i, int& ntl, int& cc) {
-        const int half = i / (SF / 2), rem = i % (SF / 2);
-        ntl = rem / (KC / 2); cc = half * (KC / 2) + rem % (KC / 2);
+        const int burst = i / G::FB, rem = i % G::FB;
+        ntl = rem / G::KB; cc = burst * G::KB + rem % G::KB;
     };
     if (r < 3 * NT * KC) {
         int ntl; split(r % SF, ntl, c);
@@ -473,12 +478,12 @@ __global__ __launch_bounds__(256) void blocks_pack_vec_kernel(BlkPackArgs a) {
     a.vec[i] = v;
 }
 
-constexpr int LDS_STATIC_MAX = 2 * 12 * 1024 + 2 * 4 * 2 * 3 * 64 * 8;      // ring + K/V exchange at d = 192
+constexpr int LDS_STATIC_MAX = 2 * 16 * 1024 + 2 * 4 * 2 * 3 * 64 * 8;      // upper bound of ring + K/V exchange over the shapes
 constexpr int LDS_BUDGET = 160 * 1024;
 
 bool blocks_shape_ok(const bsrl_blocks_desc* d) {
     if (!d) return false;
-    const bool geo = (d->d == 128 && d->n_heads == 4) || (d->d == 192 && d->n_heads == 4);
+    const bool geo = (d->d == 128 && d->n_heads == 4) || (d->d == 192 && d->n_heads == 4) || (d->d == 256 && d->n_heads == 8);
     if (!geo || d->T < 1 || d->T > 32 || d->ffn <= 0 || d->ffn % 32 != 0 || d->ffn < 64 || d->n_layers < 1 ||
         d->n_layers > BSRL_MAX_LAYERS || (d->dtype != BSRL_F16 && d->dtype != BSRL_BF16) ||
         (d->act != BSRL_ACT_RELU && d->act != BSRL_ACT_GELU) || d->n_queries < 0 || d->n_queries > 16 || d->n_queries > d->T)
@@ -487,7 +492,7 @@ bool blocks_shape_ok(const bsrl_blocks_desc* d) {
     return vec_bytes + LDS_STATIC_MAX <= LDS_BUDGET;
 }
 int64_t blocks_stages(const bsrl_blocks_desc* d) {
-    return (int64_t)d->n_layers * (d->d == 128 ? Geo<128>::layer_stages(d->ffn) : Geo<192>::layer_stages(d->ffn));
+    return (int64_t)d->n_layers * (d->d == 128 ? Geo<128>::layer_stages(d->ffn) : d->d == 192 ? Geo<192>::layer_stages(d->ffn) : Geo<256>::layer_stages(d->ffn));
 }
 int64_t blocks_frag_bytes(const bsrl_blocks_desc* d) { return blocks_stages(d) * (d->d / 16) * 1024; }
 
@@ -533,6 +538,7 @@ extern "C" int bsrl_blocks_pack(const bsrl_blocks_desc* d, const bsrl_blocks_par
     const int64_t nfrags = blocks_stages(d) * (d->d / 16);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (d->d == 128) { if (d->dtype == BSRL_F16) pack_launch<F16, 128, 32>(pa, nfrags, st); else pack_launch<BF16, 128, 32>(pa, nfrags, st); }
+    else if (d->d == 256) { if (d->dtype == BSRL_F16) pack_launch<F16, 256, 32>(pa, nfrags, st); else pack_launch<BF16, 256, 32>(pa, nfrags, st); }
     else { if (d->dtype == BSRL_F16) pack_launch<F16, 192, 48>(pa, nfrags, st); else pack_launch<BF16, 192, 48>(pa, nfrags, st); }
     BSRL_CHECK_LAUNCH("bsrl_blocks_pack");
     return BSRL_OK;
@@ -562,6 +568,9 @@ extern "C" int bsrl_blocks_forward(const bsrl_blocks_desc* d, const void* packed
     if (d->d == 128) {
         if (f16) rc = relu ? fwd_launch<F16, 128, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<F16, 128, 32, BSRL_ACT_GELU>(a, cus, st);
         else rc = relu ? fwd_launch<BF16, 128, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<BF16, 128, 32, BSRL_ACT_GELU>(a, cus, st);
+    } else if (d->d == 256) {
+        if (f16) rc = relu ? fwd_launch<F16, 256, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<F16, 256, 32, BSRL_ACT_GELU>(a, cus, st);
+        else rc = relu ? fwd_launch<BF16, 256, 32, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<BF16, 256, 32, BSRL_ACT_GELU>(a, cus, st);
     } else {
         if (f16) rc = relu ? fwd_launch<F16, 192, 48, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<F16, 192, 48, BSRL_ACT_GELU>(a, cus, st);
         else rc = relu ? fwd_launch<BF16, 192, 48, BSRL_ACT_RELU>(a, cus, st) : fwd_launch<BF16, 192, 48, BSRL_ACT_GELU>(a, cus, st);

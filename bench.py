@@ -67,7 +67,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--route", default="auto", choices=("auto", "fused", "ops"))
+    ap.add_argument("--route", default="auto", choices=("auto", "fused", "blocks", "ops"))
     ap.add_argument("--config", type=int, default=1, help="benchmark config index (1 = headline)")
     ap.add_argument("--batch", type=int, default=0, help="override B (0 = the config's B)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -112,7 +112,7 @@ def main():
     obs, k = obs_cpu.to(dev), k_cpu.to(dev)
     route = args.route
     if route == "auto":
-        route = "fused" if m.fused_supported() else "ops"
+        route = "fused" if m.fused_supported() else "blocks" if m.blocks_supported() else "ops"
 
     def step():
         return m.forward_stacked(obs, k, route=route)
@@ -143,7 +143,7 @@ def main():
     # EXECUTED figure when the fused route prunes the final block to token 0 (the reference's
     # own n_queries path): the roofline fraction is quoted on executed work only.
     dense_flops = cm.flops_per_env(spec) * B
-    pruned = route == "fused" and m.prune_final
+    pruned = (route == "fused" and m.prune_final) or route == "blocks"
     exec_flops = dense_flops
     if pruned:
         d_, T_, F_ = spec.d, spec.T, spec.ffn
@@ -152,7 +152,9 @@ def main():
     achieved = exec_flops / (dev_ms_avg * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[dtype]
     kname = ("cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
-             "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else "launch train (per-op route)")
+             "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else
+             "cfg_embed_kernel + blocks_kernel (final block pruned to token 0) + heads" if route == "blocks" else
+             "launch train (per-op route)")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4),
                 "traffic": TRAFFIC_BYTES_CFG1_FUSED_PRUNED if (pruned and args.config == 1 and B == 16384) else None,

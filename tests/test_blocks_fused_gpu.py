@@ -47,24 +47,29 @@ def _inputs(B, T, d, seed):
     return x, (mask - 1.0) * 16384.0
 
 
+def _heads(d):
+    return 8 if d == 256 else 4
+
+
 def _run(sd, L, d, F, T, dtype, x, bias, n_queries):
-    tdt = TDT[dtype]
-    nbytes = ops.blocks_pack_size(L, d, 4, F, T, "relu", n_queries, tdt)
+    tdt, H = TDT[dtype], _heads(d)
+    nbytes = ops.blocks_pack_size(L, d, H, F, T, "relu", n_queries, tdt)
     assert nbytes > 0
     image = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
     params = [[sd[f"blocks.{i}.{f}"].to(DEV).contiguous() for f in FIELDS] for i in range(L)]
-    ops.blocks_pack(params, image, d, 4, F, T, "relu", n_queries, tdt)
-    return ops.blocks_forward(image, x.to(DEV).to(tdt).contiguous(), bias.to(DEV).to(tdt).contiguous(), L, 4, F,
+    ops.blocks_pack(params, image, d, H, F, T, "relu", n_queries, tdt)
+    return ops.blocks_forward(image, x.to(DEV).to(tdt).contiguous(), bias.to(DEV).to(tdt).contiguous(), L, H, F,
                               "relu", n_queries)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("d,L,B", [(128, 1, 5), (192, 1, 5), (128, 3, 37), (192, 3, 37), (192, 6, 64)])
-def test_block_stack_matches_oracle(dtype, d, L, B):
-    T, F = 29, 4 * d
+@pytest.mark.parametrize("d,L,B,T", [(128, 1, 5, 29), (192, 1, 5, 29), (128, 3, 37, 29), (192, 3, 37, 29),
+                                     (192, 6, 64, 29), (256, 2, 9, 32), (256, 4, 33, 17)])
+def test_block_stack_matches_oracle(dtype, d, L, B, T):
+    F = 4 * d
     sd = _weights(L, d, F, 10 + L + d)
     x, bias = _inputs(B, T, d, 3 + B)
-    arch = {"n_heads": 4, "n_blocks": L}
+    arch = {"n_heads": _heads(d), "n_blocks": L}
     lead32, res32 = nr.blocks_forward(sd, arch, x.to(TDT[dtype]), bias)          # fp32 math on the rounded tokens
     lead_em, res_em = nr.blocks_forward(sd, arch, x, bias, emulate=dtype)
     out, res = _run(sd, L, d, F, T, dtype, x, bias, 5)
@@ -100,6 +105,7 @@ def test_unpruned_stack_and_invariants():
 
 
 def test_unsupported_shapes_are_reported():
-    assert ops.blocks_pack_size(2, 256, 8, 1024, 32, "relu", 0, torch.float16) == 0
+    assert ops.blocks_pack_size(2, 384, 12, 1536, 32, "relu", 0, torch.float16) == 0
+    assert ops.blocks_pack_size(2, 256, 4, 1024, 32, "relu", 0, torch.float16) == 0
     assert ops.blocks_pack_size(2, 192, 4, 768, 48, "relu", 0, torch.float16) == 0
     assert ops.blocks_pack_size(2, 192, 4, 768, 29, "relu", 5, torch.float32 if False else torch.float16) > 0
