@@ -50,6 +50,8 @@ SIGNATURES = {
     "bsrl_ln_fwd_add": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f, _i32, _p]),
     "bsrl_linear": (_i32, [_p, _i64, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64,
                            _i32, _i32, _i32, _p]),
+    "bsrl_linear_grouped": (_i32, [_p, _i64, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64,
+                                   _i32, _i32, _i32, _i64, _i64, _p]),
     "bsrl_attn_fwd": (_i32, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p,
                              _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_ffn_fused": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _i64, _i64, _i64, _i32, _i32, _p]),

@@ -251,12 +251,23 @@ class ConfigPolicy(nn.Module):
             raise ops.Unsupported("bsrl_cfg_forward")
         return logits.view(B, N_ACTION_HEADS, self.n_gears), value
 
+    def _tokens(self, obs, r, dt):
+        """Tokenizer on the GEMM kernels: the obs is rounded once to the stream dtype
+        (python/policy.py:1200-1209), then one Linear per token type writes its rows of the
+        (B, T, d) stream directly (ops.cfg_embed is the same op as one VALU kernel)."""
+        B, T = obs.shape[0], self.T
+        o = obs.to(dt)
+        x = torch.empty(B, T, self.d, device=obs.device, dtype=dt)
+        ops.linear(o[:, :self.prop_dim], r["prop_w"], r["prop_b"], out=x[:, 0:1])
+        ops.linear(o[:, self.prop_dim:].reshape(B * (T - 1), self.obj_dim), r["obj_w"], r["obj_b"], out=x[:, 1:])
+        return x
+
     def _forward_blocks(self, obs, n_valid, dt):
         B, T = obs.shape[0], self.T
         r = self._replicas(dt, obs.device)
         if obs.dtype not in (torch.float32, dt):
             obs = obs.float()
-        x = ops.cfg_embed(obs, r["prop_w"], r["prop_b"], r["obj_w"], r["obj_b"], T, dt)       # (B, T, d)
+        x = self._tokens(obs, r, dt)                                                          # (B, T, d)
         # additive key bias of the padding mask: tokens 0..n_valid attendable (exp(-16384) == 0 in fp32)
         if n_valid is None:
             bias = torch.zeros(B, T, device=obs.device, dtype=dt)
@@ -277,7 +288,7 @@ class ConfigPolicy(nn.Module):
         r = self._replicas(dt, obs.device)
         if obs.dtype not in (torch.float32, dt):
             obs = obs.float()
-        x = ops.cfg_embed(obs, r["prop_w"], r["prop_b"], r["obj_w"], r["obj_b"], T, dt)       # (B, T, d)
+        x = self._tokens(obs, r, dt)                                                          # (B, T, d)
         for blk, w in zip(self.blocks, r["blk"]):
             h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
             qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                       # (B, T, 3d)

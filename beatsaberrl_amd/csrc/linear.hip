@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
                 if (res) o += DT::to_f(res[row * a.ldr + c]);
                 const bool second = a.y2 && c >= a.split;
                 void* dst = second ? a.y2 : a.y;
-                const int64_t off = second ? row * a.ldy2 + (c - a.split) : row * a.ldy + c;
+                const int64_t off = second ? row * a.ldy2 + (c - a.split) : lin_yoff(a, row) + c;
                 if (a.out_f32) static_cast<float*>(dst)[off] = o;
                 else static_cast<u16*>(dst)[off] = DT::from_f(o);
             }
@@ -149,12 +149,12 @@ __global__ __launch_bounds__(256) void linear_mfma_vec_kernel(LinArgs a) {
                 o[2] += DT::to_f((u16)(rv.y & 0xffff)); o[3] += DT::to_f((u16)(rv.y >> 16));
             }
             if (a.out_f32) {
-                *reinterpret_cast<float4*>(static_cast<float*>(a.y) + row * a.ldy + col) = make_float4(o[0], o[1], o[2], o[3]);
+                *reinterpret_cast<float4*>(static_cast<float*>(a.y) + lin_yoff(a, row) + col) = make_float4(o[0], o[1], o[2], o[3]);
             } else {
                 uint2 ov;
                 ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
                 ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
-                *reinterpret_cast<uint2*>(static_cast<u16*>(a.y) + row * a.ldy + col) = ov;
+                *reinterpret_cast<uint2*>(static_cast<u16*>(a.y) + lin_yoff(a, row) + col) = ov;
             }
         }
     }
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs a) {
             float o = apply_act<ACT>(acc[i][j] + (a.bias ? a.bias[c] : 0.f));
             if (res) o += res[row * a.ldr + c];
             if (a.y2 && c >= a.split) static_cast<float*>(a.y2)[row * a.ldy2 + (c - a.split)] = o;
-            else static_cast<float*>(a.y)[row * a.ldy + c] = o;
+            else static_cast<float*>(a.y)[lin_yoff(a, row) + c] = o;
         }
     }
 }
@@ -227,6 +227,14 @@ extern "C" int bsrl_linear(const void* x, int64_t ldx, const void* w, const floa
                            int64_t ldr, void* y, int64_t ldy, void* y2, int64_t ldy2, int64_t split,
                            int64_t rows, int64_t K, int64_t M, int act, int dtype, int out_dtype,
                            bsrl_stream stream) {
+    return bsrl_linear_grouped(x, ldx, w, bias, residual, ldr, y, ldy, y2, ldy2, split, rows, K, M, act, dtype, out_dtype,
+                               0, 0, stream);
+}
+
+extern "C" int bsrl_linear_grouped(const void* x, int64_t ldx, const void* w, const float* bias, const void* residual,
+                                   int64_t ldr, void* y, int64_t ldy, void* y2, int64_t ldy2, int64_t split,
+                                   int64_t rows, int64_t K, int64_t M, int act, int dtype, int out_dtype,
+                                   int64_t y_group_rows, int64_t y_group_stride, bsrl_stream stream) {
     if (!x || !w || !y) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: null pointer");
     if (rows < 0 || K <= 0 || M <= 0 || K > (1 << 20) || M > (1 << 20))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad shape rows=%lld K=%lld M=%lld", (long long)rows, (long long)K, (long long)M);
@@ -236,10 +244,14 @@ extern "C" int bsrl_linear(const void* x, int64_t ldx, const void* w, const floa
     if (act < 0 || act > 2) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad act %d", act);
     if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: bad dtype");
     if (out_dtype != dtype && out_dtype != BSRL_F32) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear: out_dtype must be dtype or F32");
+    if (y_group_rows < 0 || (y_group_rows > 0 && (y2 || rows % y_group_rows != 0 || y_group_rows > (1 << 20) ||
+                                                  y_group_stride < y_group_rows * ldy)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_grouped: groups need rows %% group == 0, group stride >= group * ldy, no split");
     if (rows == 0) return BSRL_OK;
     if ((rows + 127) / 128 > 65535 * 16) return BSRL_UNSUPPORTED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    LinArgs a{x, ldx, w, bias, residual, ldr, y, ldy, y2, ldy2, split, rows, (int)K, (int)M, out_dtype == BSRL_F32};
+    LinArgs a{x, ldx, w, bias, residual, ldr, y, ldy, y2, ldy2, split, rows, (int)K, (int)M, out_dtype == BSRL_F32,
+              (int)y_group_rows, y_group_stride};
     if (dtype == BSRL_F32) {
         dim3 grid((unsigned)((M + 63) / 64), (unsigned)((rows + 63) / 64));
         if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_RELU>), grid, dim3(256), 0, st, a);
@@ -248,7 +260,7 @@ extern "C" int bsrl_linear(const void* x, int64_t ldx, const void* w, const floa
     } else {
         const bool fast = K % 8 == 0 && ldx % 8 == 0 && bsrl_aligned(x, 16) && bsrl_aligned(w, 16);
         const int osz = out_dtype == BSRL_F32 ? 4 : 2;
-        const bool vec = fast && !y2 && M % 4 == 0 && ldy % 4 == 0 && bsrl_aligned(y, 4 * osz) &&
+        const bool vec = fast && !y2 && M % 4 == 0 && ldy % 4 == 0 && y_group_stride % 4 == 0 && bsrl_aligned(y, 4 * osz) &&
                          (!bias || bsrl_aligned(bias, 16)) &&
                          (!residual || (ldr % 4 == 0 && bsrl_aligned(residual, 8)));
         if (vec && bsrl_linear_tiled(a, act, dtype, st)) {

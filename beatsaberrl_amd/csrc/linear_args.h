@@ -11,7 +11,17 @@ struct LinArgs {
     void* y2; int64_t ldy2; int64_t split;
     int64_t rows; int K; int M;
     int out_f32;
+    // grouped output rows (0 = off): output row r lives at (r / y_group) * y_gstride + (r % y_group) * ldy,
+    // i.e. y is a (rows / y_group, y_group, M) view of a larger tensor (a token slice of a (B, T, d) stream)
+    int y_group; int64_t y_gstride;
 };
+
+// element offset of output row `row` in y (rows < 2^31 is checked on the host)
+__device__ __forceinline__ int64_t lin_yoff(const LinArgs& a, int64_t row) {
+    if (a.y_group == 0) return row * a.ldy;
+    const uint32_t r = (uint32_t)row, gq = r / (uint32_t)a.y_group;
+    return (int64_t)gq * a.y_gstride + (int64_t)(r - gq * (uint32_t)a.y_group) * a.ldy;
+}
 
 // LDS-tiled 16-bit kernel for large row counts (linear_tiled.hip); returns false when the
 // shape is outside what it covers (the caller then takes the direct-from-global kernel).

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
                 ov.y = (uint32_t)DT::from_f(v[2]) | ((uint32_t)DT::from_f(v[3]) << 16);
                 ov.z = (uint32_t)DT::from_f(v[4]) | ((uint32_t)DT::from_f(v[5]) << 16);
                 ov.w = (uint32_t)DT::from_f(v[6]) | ((uint32_t)DT::from_f(v[7]) << 16);
-                *reinterpret_cast<uint4*>(y + row * a.ldy + col) = ov;
+                *reinterpret_cast<uint4*>(y + lin_yoff(a, row) + col) = ov;
             }
         }
     }
@@ -145,7 +145,7 @@ bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st) {
     static_assert(16 * EP_LD * 4 * 4 <= LDS_U4 * 16, "epilogue staging must fit in the operand tiles");
     // worth it only when there are enough rows to fill the chip with 256-row tiles
     if (a.out_f32 || a.y2 || a.rows < 4096 || a.M % 8 != 0 || a.K % 8 != 0) return false;
-    if (a.ldy % 8 != 0 || !bsrl_aligned(a.y, 16) || (a.res && (a.ldr % 8 != 0 || !bsrl_aligned(a.res, 16)))) return false;
+    if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16) || (a.res && (a.ldr % 8 != 0 || !bsrl_aligned(a.res, 16)))) return false;
     if ((a.rows + BM - 1) / BM > 65535) return false;
     if (dtype == BSRL_F16) launch<F16>(a, act, st);
     else launch<BF16>(a, act, st);

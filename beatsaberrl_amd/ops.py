@@ -118,11 +118,14 @@ def _rows2d(t):
     return t, rows, ld
 
 
-def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None):
+def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None, out=None):
     """act(x @ w.T + bias) (+ residual).  x (..., K) in w's dtype, w (M, K)
     contiguous, bias fp32.  split=s returns (y[..., :s], y[..., s:]) as two
-    separately stored tensors."""
-    _need_cuda(x, w, bias, residual)
+    separately stored tensors.  out: a (N, G, M) view with unit last stride (e.g. a
+    token slice `stream[:, a:b, :]` of a (B, T, d) tensor) that receives the N * G
+    output rows in place of a fresh tensor - the kernel writes the slice directly, there
+    is no concatenation pass."""
+    _need_cuda(x, w, bias, residual, out)
     if x.dtype is not w.dtype:
         raise TypeError(f"linear: x is {x.dtype} but w is {w.dtype}")
     if not w.is_contiguous() or w.dim() != 2:
@@ -138,7 +141,15 @@ def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None)
         if residual.dtype is not x.dtype or residual.shape != (*lead, M):
             raise RuntimeError("linear: residual must be (..., M) in x's dtype")
         r2, _, ldr = _rows2d(residual)
-    if split is None:
+    group, gstride = 0, 0
+    if out is not None:
+        if split is not None or out.dim() != 3 or out.shape[2] != M or out.stride(2) != 1 or out.dtype is not out_dtype \
+                or out.shape[0] * out.shape[1] != rows:
+            raise RuntimeError("linear: out must be a (N, G, M) view with unit last stride holding all output rows")
+        y, y2, ld2, sp = out, None, 0, 0
+        group, gstride = out.shape[1], out.stride(0)
+        ldy = out.stride(1) if group > 1 else M
+    elif split is None:
         y = torch.empty(*lead, M, device=x.device, dtype=out_dtype)
         y2, ld2, sp = None, 0, 0
         ldy = M
@@ -147,9 +158,9 @@ def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None)
         y2 = torch.empty(*lead, M - split, device=x.device, dtype=out_dtype)
         ldy, ld2, sp = split, M - split, split
     with torch.cuda.device(x.device):
-        rc = _lib.load().bsrl_linear(x2.data_ptr(), ldx, w.data_ptr(), _ptr(_f32c(bias, "bias")), _ptr(r2), ldr,
-                                     y.data_ptr(), ldy, _ptr(y2), ld2, sp, rows, K, M, _ACT[act],
-                                     dt_code(x.dtype), dt_code(out_dtype), _stream(x))
+        rc = _lib.load().bsrl_linear_grouped(x2.data_ptr(), ldx, w.data_ptr(), _ptr(_f32c(bias, "bias")), _ptr(r2), ldr,
+                                             y.data_ptr(), ldy, _ptr(y2), ld2, sp, rows, K, M, _ACT[act],
+                                             dt_code(x.dtype), dt_code(out_dtype), group, gstride, _stream(x))
     if not _lib.check(rc, "bsrl_linear"):
         raise Unsupported(f"linear rows={rows} K={K} M={M} dtype={x.dtype}")
     return y if split is None else (y, y2)

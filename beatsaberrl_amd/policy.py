@@ -57,14 +57,15 @@ def _mlp(sizes, act=nn.ReLU):
     return nn.Sequential(*layers)
 
 
-def _lin(m: nn.Linear, x, act=None, residual=None):
+def _lin(m: nn.Linear, x, act=None, residual=None, out=None):
     """A Linear on the kernels in x's dtype (fp32 master weights, 16-bit replica when needed)."""
-    return ops.linear(x, _fl._replica(m.weight, x.dtype), _fl._bias32(m.bias), act=act, residual=residual)
+    return ops.linear(x, _fl._replica(m.weight, x.dtype), _fl._bias32(m.bias), act=act, residual=residual, out=out)
 
 
-def _seq(seq: nn.Sequential, x):
+def _seq(seq: nn.Sequential, x, out=None):
     """Linear (ReLU Linear)* with each ReLU in its producer's epilogue (reference
-    python/policy.py:76-145, `_seq` / `_run`)."""
+    python/policy.py:76-145, `_seq` / `_run`).  out: a (N, G, M) slice of the token stream that
+    receives the last Linear's rows directly."""
     ms = list(seq)
     i = 0
     while i < len(ms):
@@ -72,7 +73,8 @@ def _seq(seq: nn.Sequential, x):
         if not isinstance(m, nn.Linear):
             raise RuntimeError(f"unsupported module in Sequential: {type(m).__name__}")
         relu = i + 1 < len(ms) and isinstance(ms[i + 1], nn.ReLU)
-        x = _lin(m, x, act="relu" if relu else None)
+        last = i + (2 if relu else 1) >= len(ms)
+        x = _lin(m, x, act="relu" if relu else None, out=out if last else None)
         i += 2 if relu else 1
     return x
 
@@ -370,11 +372,13 @@ class NotePolicy(nn.Module):
         sab_in, torso_in, leg_in, note_in, attn_bias = ops.note_frontend(
             obs, self._saber_idx32, self._body_idx32, dt, note_geo=self.note_geo, flux=self.game == "flux",
             z_asinh=self.z_asinh)
-        tok_saber = _seq(self.saber_mlp, sab_in)
-        tok_torso = _seq(self.torso_mlp, torso_in).unsqueeze(1)
-        tok_leg = _seq(self.leg_mlp, leg_in)
-        tok_note = _seq(self.note_mlp, note_in)
-        x = torch.cat([tok_saber, tok_torso, tok_leg, tok_note], dim=1)   # (B, 29, d)
+        # every encoder writes its tokens straight into their rows of the (B, 29, d) stream
+        # [saber_L, saber_R, torso, leg_L, leg_R, notes...] (the reference concatenates, policy.py:1247-1249)
+        x = torch.empty(B, self.n_lead + N_NOTE_SLOTS, d, device=obs.device, dtype=dt)
+        _seq(self.saber_mlp, sab_in, out=x[:, 0:2])
+        _seq(self.torso_mlp, torso_in, out=x[:, 2:3])
+        _seq(self.leg_mlp, leg_in, out=x[:, 3:5])
+        _seq(self.note_mlp, note_in, out=x[:, 5:])
         if self.emb_ln is not None:
             x = self.emb_ln(x)
         if self.fused_blocks_ok(dt):

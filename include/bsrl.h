@@ -75,6 +75,18 @@ int bsrl_linear(const void* x, int64_t ldx, const void* w, const float* bias,
                 void* y2, int64_t ldy2, int64_t split,
                 int64_t rows, int64_t K, int64_t M, int act, int dtype,
                 int out_dtype, bsrl_stream stream);
+/* bsrl_linear whose output rows are grouped: output row r is written at
+ * y + (r / y_group_rows) * y_group_stride + (r % y_group_rows) * ldy (elements),
+ * i.e. y is a (rows / y_group_rows, y_group_rows, M) slice of a larger tensor -
+ * an encoder's tokens written straight into their rows of the (B, T, d) stream,
+ * which replaces the reference's torch.cat of the token groups
+ * (python/policy.py:1247-1249).  y_group_rows == 0: plain bsrl_linear.  No split
+ * output in grouped form. */
+int bsrl_linear_grouped(const void* x, int64_t ldx, const void* w, const float* bias,
+                        const void* residual, int64_t ldr, void* y, int64_t ldy,
+                        void* y2, int64_t ldy2, int64_t split,
+                        int64_t rows, int64_t K, int64_t M, int act, int dtype, int out_dtype,
+                        int64_t y_group_rows, int64_t y_group_stride, bsrl_stream stream);
 
 /* ---- Short-sequence masked multi-head attention ----------------------------
  * Replaces fp16_gemm.attn29_fwd (small_attn.cu:515-536) and the SDPA / fp32

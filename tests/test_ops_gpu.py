@@ -159,6 +159,30 @@ def test_linear_large_row_counts_take_the_tiled_kernel(dtype, rows, K, M, act, u
         assert torch.equal(small, y[lo:hi])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,G,K,M,T,t0", [(7, 2, 49, 192, 29, 0), (333, 1, 29, 192, 29, 2), (700, 24, 40, 192, 29, 5),
+                                          (64, 31, 16, 256, 32, 1), (3, 5, 128, 136, 8, 3)])
+@pytest.mark.parametrize("act", [None, "relu"])
+def test_linear_grouped_output_rows_write_a_token_slice(dtype, N, G, K, M, T, t0, act):
+    """out = stream[:, t0:t0+G, :] receives the N * G rows in place (direct, vectorised and LDS-tiled kernels):
+    the slice holds the same BITS as the plain call, the rest of the stream is untouched."""
+    x = _rand(N * G, K, dtype=dtype, seed=N + G)
+    w = _rand(M, K, dtype=dtype, seed=K + M, scale=1 / math.sqrt(K))
+    b = _rand(M, seed=M)
+    plain = ops.linear(x, w, b, act=act)
+    stream = torch.full((N, T, M), 7.0, device=DEV, dtype=dtype)
+    got = ops.linear(x, w, b, act=act, out=stream[:, t0:t0 + G])
+    assert got.data_ptr() == stream[:, t0:t0 + G].data_ptr()
+    assert torch.equal(stream[:, t0:t0 + G].reshape(N * G, M), plain)
+    rest = torch.ones(T, dtype=torch.bool)
+    rest[t0:t0 + G] = False
+    assert bool((stream[:, rest] == 7.0).all())
+    with pytest.raises(RuntimeError):
+        ops.linear(x, w, b, out=stream[:, t0:t0 + G, :M - 1])
+    with pytest.raises(RuntimeError):
+        ops.linear(x, w, b, out=stream[:, t0:t0 + G], split=8)
+
+
 def test_linear_rows_are_batch_invariant():
     """A row's bits do not depend on the batch it sits in or on its tile phase
     (the reference holds its kernels to this: tests/test_fused_ffn.py:332-353)."""
