@@ -46,6 +46,52 @@ def test_argument_errors_are_reported_without_a_device(lib):
     assert lib.bsrl_attn_fwd(16, 8, 8, 16, 8, 8, 16, 8, 8, None, None, 16, 2, 64, 64, 4, 32, _lib.F16, None) > 0
 
 
+def test_new_entry_points_reject_bad_arguments_without_a_device(lib):
+    C = ctypes
+    # front end: null pointers, short rows, obs dtype that is neither fp32 nor the stream dtype, bad z scale
+    args = [16, 630, _lib.F32, 16, 16, 1, 0, C.c_float(8.0), 16, 16, 16, 16, 16, 4, _lib.F16, None]
+    bad = list(args); bad[0] = None
+    assert lib.bsrl_note_frontend(*bad) == -1 and b"null" in lib.bsrl_last_error()
+    bad = list(args); bad[1] = 629
+    assert lib.bsrl_note_frontend(*bad) == -1
+    bad = list(args); bad[2] = _lib.BF16
+    assert lib.bsrl_note_frontend(*bad) == -1 and b"stream dtype" in lib.bsrl_last_error()
+    bad = list(args); bad[7] = C.c_float(0.0)
+    assert lib.bsrl_note_frontend(*bad) == -1
+    ok = list(args); ok[13] = 0
+    assert lib.bsrl_note_frontend(*ok) == 0                     # B == 0: nothing to do
+    # action epilogue: K and head-count limits, sampling without an output
+    assert lib.bsrl_sample_heads(16, 4, 29, 9, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 4, 33, 7, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 4, 29, 7, None, None, 0, 0, None, 0, None, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 0, 29, 7, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == 0
+    # grouped linear: the group must divide the rows, fit its stride and exclude a split output
+    g = lambda rows, grp, gs, y2=None, split=0: lib.bsrl_linear_grouped(
+        16, 8, 16, None, None, 0, 16, 8, y2, 8 if y2 else 0, split, rows, 8, 8, 0, _lib.F16, _lib.F16, grp, gs, None)
+    assert g(6, 4, 64) == -1 and b"group" in lib.bsrl_last_error()
+    assert g(8, 4, 16) == -1
+    assert g(8, 4, 64, y2=16, split=4) == -1
+    assert g(0, 4, 64) == 0
+
+
+def test_block_stack_shape_support_table(lib):
+    d = lambda **k: _lib.BlocksDesc(**{**dict(n_layers=6, d=192, n_heads=4, ffn=768, T=29, act=_lib.ACT_RELU,
+                                              n_queries=5, dtype=_lib.F16), **k})
+    size = lib.bsrl_blocks_pack_size(ctypes.byref(d()))
+    # 6 blocks x 72 stages x 12 KB of fragments + 6 x (9 * 192 + 768) fp32 vector entries
+    assert size == 6 * 72 * 12 * 1024 + 6 * (9 * 192 + 768) * 4
+    assert lib.bsrl_blocks_pack_size(ctypes.byref(d(d=128, ffn=512, n_layers=3))) == 3 * 48 * 8 * 1024 + 3 * (9 * 128 + 512) * 4
+    assert lib.bsrl_blocks_pack_size(ctypes.byref(d(d=256, n_heads=8, ffn=1024, T=32, n_layers=4, dtype=_lib.BF16))) > 0
+    for bad in (d(dtype=_lib.F32), d(T=33), d(d=384, n_heads=12), d(n_heads=6), d(ffn=100), d(n_queries=17),
+                d(n_layers=9), d(act=_lib.ACT_NONE), d(n_layers=8, ffn=4096)):       # the last: vectors exceed the LDS budget
+        assert lib.bsrl_blocks_pack_size(ctypes.byref(bad)) == 0
+    rc = lib.bsrl_blocks_forward(ctypes.byref(d(T=33)), 16, 16, 16, None, 16, 4, None)
+    assert rc > 0                                                # unsupported shape: a return code, not an error
+    rc = lib.bsrl_blocks_forward(ctypes.byref(d()), None, 16, 16, None, 16, 4, None)
+    assert rc == -1 and b"null" in lib.bsrl_last_error()
+    assert lib.bsrl_blocks_forward(ctypes.byref(d()), 16, 16, 16, None, 16, 0, None) == 0
+
+
 def test_host_modules_refuse_cpu_tensors():
     import torch
     from beatsaberrl_amd.config_policy import ConfigPolicy
