@@ -85,6 +85,26 @@ __device__ __forceinline__ float gelu_fast(float x) {
     const float e = __builtin_amdgcn_exp2f(xc * q);          // exp(-u)
     return x * __builtin_amdgcn_rcpf(e + 1.0f);
 }
+// The same activation in two pieces, for callers that pin VALU work between MFMAs: the head is the
+// two ops that depend on nothing but x (clamp, square), the tail is the rest of the chain.
+struct Act16Head { float xc, x2; };
+template <int ACT> __device__ __forceinline__ Act16Head act16_head(float x) {
+    Act16Head h = {x, x};
+    if (ACT == BSRL_ACT_GELU) { h.xc = __builtin_amdgcn_fmed3f(x, -9.0f, 9.0f); h.x2 = h.xc * h.xc; }
+    return h;
+}
+template <int ACT> __device__ __forceinline__ float act16_tail(float x, Act16Head h) {
+    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_GELU) {
+        constexpr float L2E = 1.44269504088896340736f;
+        constexpr float C0 = -1.59501576f * L2E, C1 = -7.40113019e-02f * L2E, C2 = 7.03035067e-04f * L2E;
+        float q = fmaf(C2, h.x2, C1);
+        q = fmaf(q, h.x2, C0);
+        const float e = __builtin_amdgcn_exp2f(h.xc * q);
+        return x * __builtin_amdgcn_rcpf(e + 1.0f);
+    }
+    return x;
+}
 // activation for values about to be rounded to fp16 / bf16
 template <int ACT> __device__ __forceinline__ float apply_act16(float x) {
     if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);

@@ -392,12 +392,23 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         for (int c = 0; c < KC; ++c)
 #pragma unroll
                             for (int ntl = 0; ntl < 2; ++ntl) {
-#pragma unroll
-                                for (int rt = 0; rt < RT; ++rt) accB[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, accB[ntl][rt]);
-                                // slice sl = (c, ntl): one hidden unit per upper row tile, element (sl >> 2, sl & 3)
+                                // slice sl = (c, ntl): one hidden unit per upper row tile, element (sl >> 2, sl & 3).
+                                // Issue order MFMA, 2 VALU, MFMA, rest: a 16-cycle MFMA lets two VALU ops issue under it,
+                                // and back-to-back MFMAs would leave the first one's slots empty (in-order issue).
                                 const int sl = c * 2 + ntl;                    // 0..7
+                                Act16Head hd[RH > 0 ? RH : 1];
 #pragma unroll
-                                for (int rt = 0; rt < RH; ++rt) ga[rt][sl] = apply_act16<ACT>(accA[sl >> 2][RH + rt][sl & 3]);
+                                for (int rt = 0; rt < RT; ++rt) {
+                                    accB[ntl][rt] = DT::mfma32(w1[ntl * KC + c], hf[rt][c].v, accB[ntl][rt]);
+                                    __builtin_amdgcn_sched_barrier(0);
+                                    if (rt == 0) {
+#pragma unroll
+                                        for (int r2 = 0; r2 < RH; ++r2) hd[r2] = act16_head<ACT>(accA[sl >> 2][RH + r2][sl & 3]);
+                                        __builtin_amdgcn_sched_barrier(0);
+                                    }
+                                }
+#pragma unroll
+                                for (int rt = 0; rt < RH; ++rt) ga[rt][sl] = act16_tail<ACT>(accA[sl >> 2][RH + rt][sl & 3], hd[rt]);
                                 __builtin_amdgcn_sched_barrier(0);
                             }
 #pragma unroll
@@ -411,10 +422,19 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                         for (int nt = 0; nt < NT; ++nt) {
+                            Act16Head hd[RH > 0 ? RH : 1];
 #pragma unroll
-                            for (int rt = 0; rt < RT; ++rt) x[rt][nt] = DT::mfma32(w2[nt], hidA[rt].v, x[rt][nt]);
+                            for (int rt = 0; rt < RT; ++rt) {
+                                x[rt][nt] = DT::mfma32(w2[nt], hidA[rt].v, x[rt][nt]);
+                                __builtin_amdgcn_sched_barrier(0);
+                                if (rt == 0) {
 #pragma unroll
-                            for (int rt = 0; rt < RH; ++rt) ga[rt][nt] = apply_act16<ACT>(accB[nt >> 2][rt][nt & 3]);
+                                    for (int r2 = 0; r2 < RH; ++r2) hd[r2] = act16_head<ACT>(accB[nt >> 2][r2][nt & 3]);
+                                    __builtin_amdgcn_sched_barrier(0);
+                                }
+                            }
+#pragma unroll
+                            for (int rt = 0; rt < RH; ++rt) ga[rt][nt] = act16_tail<ACT>(accB[nt >> 2][rt][nt & 3], hd[rt]);
                             __builtin_amdgcn_sched_barrier(0);
                         }
 #pragma unroll
