@@ -54,6 +54,7 @@ __host__ __device__ constexpr int vec_floats(int L, int F) { return V_LAYER0 + L
 struct FwdArgs {
     const uint4* frags; const float* vec;
     const void* obs; int64_t obs_ld; int obs_f32;
+    int tok_vec;      // fp32 obs, 16-lane objects, 4-aligned proprio width and rows: the tokenizer reads 16-byte groups
     const int32_t* n_valid;
     float* logits; float* value;
     uint32_t* ws;
@@ -523,6 +524,25 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
+                if (a.tok_vec) {
+                    // a lane's 8 k slots per chunk are two runs of 4 consecutive obs lanes: k0 = 32 c + 4 g + 16 jh.
+                    // Only (c, jh) = (0, 0) falls in the object block (rows 1..15); every other run is proprio (row 0).
+                    const float* orow = static_cast<const float*>(a.obs) + env * a.obs_ld;
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int jh = 0; jh < 2; ++jh) {
+                            const int k0 = 32 * c + 4 * g + 16 * jh;
+                            bool valid; int idx;
+                            if (c == 0 && jh == 0) { valid = r16 >= 1; idx = a.prop_dim + (r16 - 1) * 16 + k0; }
+                            else { valid = r16 == 0 && (k0 - 16) < a.prop_dim; idx = k0 - 16; }
+                            const float4 v = *reinterpret_cast<const float4*>(orow + (valid ? idx : 0));
+                            const uint32_t lo = pack2<DT>(v.x, v.y), hi = pack2<DT>(v.z, v.w);
+                            e[rt][c].w[2 * jh] = valid ? lo : 0u;
+                            e[rt][c].w[2 * jh + 1] = valid ? hi : 0u;
+                        }
+                    continue;
+                }
                 float ev[KC][8];
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
@@ -805,6 +825,7 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.frags = static_cast<const uint4*>(packed);
     a.vec = reinterpret_cast<const float*>(static_cast<const char*>(packed) + frag_bytes(d));
     a.obs = obs; a.obs_ld = obs_ld; a.obs_f32 = obs_dtype == BSRL_F32;
+    a.tok_vec = a.obs_f32 && d->obj_dim == 16 && d->prop_dim % 4 == 0 && obs_ld % 4 == 0 && bsrl_aligned(obs, 16);
     a.n_valid = n_valid; a.logits = logits; a.value = value; a.B = B;
     a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
