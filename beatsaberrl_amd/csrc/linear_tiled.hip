@@ -3,7 +3,11 @@
 // Workgroup tile 256 rows x 128 columns, K walked in steps of 64 through LDS.  All 256
 // threads load the step's x (256 x 64) and W (128 x 64) tiles with 16-byte global loads one
 // step ahead into registers and park them in LDS in MFMA fragment order (fragment = 64
-// lanes x 16 B, so every operand read is one conflict-free ds_read_b128); wave w owns rows
+// lanes x 16 B, one ds_read_b128 per operand).  Inside a fragment the 16-byte slot of lane l
+// is l ^ (2 * (l / 16) + k chunk): the XOR keeps the slots of any 8 consecutive lanes distinct
+// modulo 8 for the reads AND for the loader's writes (8 consecutive loader threads hold the
+// 8 k pieces of one row, which land in lanes r, r + 16, r + 32, r + 48 of two fragments -
+// unswizzled, all on the same 4 banks); wave w owns rows
 // [64w, 64w + 64) x all 128 columns: 4 x 8 accumulator tiles, 64 MFMAs per step against 24
 // fragment reads.  x and y cross HBM exactly once per column block and in full 128-byte
 // rows: the epilogue adds bias, applies the activation, then transposes each wave's
@@ -43,8 +47,8 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) { int c = col0 + lr + 32 * j; wrow[j] = (c < a.M ? c : a.M - 1) * K; }
     // where that piece lives in LDS: fragment (row tile, k chunk), lane (row % 16) + 16 * (piece % 4)
-    const int frag_lane = (lr & 15) + 16 * (lq & 3);
     const int kc_of = lq >> 2;
+    const int frag_lane = ((lr & 15) + 16 * (lq & 3)) ^ (2 * (lq & 3) + kc_of);     // swizzled slot
     uint4 xr[8], wr[4];
     auto gload = [&](int k0) {
         const int k = k0 + 8 * lq;
@@ -78,10 +82,10 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
         for (int c = 0; c < KCH; ++c) {
             s16x8 xf[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) xf[j] = __builtin_bit_cast(s16x8, lds[((wave * 4 + j) * KCH + c) * 64 + lane]);
+            for (int j = 0; j < 4; ++j) xf[j] = __builtin_bit_cast(s16x8, lds[((wave * 4 + j) * KCH + c) * 64 + (lane ^ (2 * g + c))]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const s16x8 wf = __builtin_bit_cast(s16x8, lds[(XF + i * KCH + c) * 64 + lane]);
+                const s16x8 wf = __builtin_bit_cast(s16x8, lds[(XF + i * KCH + c) * 64 + (lane ^ (2 * g + c))]);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = DT::mfma32(wf, xf[j], acc[i][j]);
             }
@@ -104,28 +108,28 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
                                          apply_act16<ACT>(acc[i][j][2] + b.z), apply_act16<ACT>(acc[i][j][3] + b.w));
             *reinterpret_cast<float4*>(ep + r16 * EP_LD + i * 16 + 4 * g) = o;
         }
-        // lane -> (row = lane / 16 + 4 q, 8 columns at 8 * (lane % 16)): 16 lanes cover one 256-byte row segment
+        // lane -> (row = lane / 16 + 4 q, 4 columns at 4 m and 4 at 64 + 4 m, m = lane % 16): consecutive lanes read
+        // consecutive 16-byte slots of the staging row (no bank conflict) and 16 lanes write one 128-byte row segment
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int rl = (lane >> 4) + 4 * q, c8 = 8 * (lane & 15);
+            const int rl = (lane >> 4) + 4 * q, c4 = 4 * (lane & 15);
             const int64_t row = row0 + wave * 64 + j * 16 + rl;
-            const int col = col0 + c8;
-            const float4 lo = *reinterpret_cast<const float4*>(ep + rl * EP_LD + c8);
-            const float4 hi = *reinterpret_cast<const float4*>(ep + rl * EP_LD + c8 + 4);
-            float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            if (row < a.rows && col < a.M) {
-                if (res) {
-                    const uint4 rv = *reinterpret_cast<const uint4*>(res + row * a.ldr + col);
-                    const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) { v[2 * e] += DT::to_f((u16)(rw[e] & 0xffff)); v[2 * e + 1] += DT::to_f((u16)(rw[e] >> 16)); }
+            for (int hh = 0; hh < 2; ++hh) {
+                const int col = col0 + 64 * hh + c4;
+                const float4 f = *reinterpret_cast<const float4*>(ep + rl * EP_LD + 64 * hh + c4);
+                float v[4] = {f.x, f.y, f.z, f.w};
+                if (row < a.rows && col < a.M) {
+                    if (res) {
+                        const uint2 rv = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
+                        v[0] += DT::to_f((u16)(rv.x & 0xffff)); v[1] += DT::to_f((u16)(rv.x >> 16));
+                        v[2] += DT::to_f((u16)(rv.y & 0xffff)); v[3] += DT::to_f((u16)(rv.y >> 16));
+                    }
+                    uint2 ov;
+                    ov.x = (uint32_t)DT::from_f(v[0]) | ((uint32_t)DT::from_f(v[1]) << 16);
+                    ov.y = (uint32_t)DT::from_f(v[2]) | ((uint32_t)DT::from_f(v[3]) << 16);
+                    *reinterpret_cast<uint2*>(y + lin_yoff(a, row) + col) = ov;
                 }
-                uint4 ov;
-                ov.x = (uint32_t)DT::from_f(v[0]) | ((uint32_t)DT::from_f(v[1]) << 16);
-                ov.y = (uint32_t)DT::from_f(v[2]) | ((uint32_t)DT::from_f(v[3]) << 16);
-                ov.z = (uint32_t)DT::from_f(v[4]) | ((uint32_t)DT::from_f(v[5]) << 16);
-                ov.w = (uint32_t)DT::from_f(v[6]) | ((uint32_t)DT::from_f(v[7]) << 16);
-                *reinterpret_cast<uint4*>(y + lin_yoff(a, row) + col) = ov;
             }
         }
     }
