@@ -53,6 +53,12 @@ template <> __device__ __forceinline__ uint32_t bpack2<F16>(float a, float b) {
     f32x2 v = {a, b};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
+template <> __device__ __forceinline__ uint32_t bpack2<BF16>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 union BFrag8 { s16x8 v; uint32_t w[4]; uint2 h[2]; uint4 u; };
 union BFrag4 { s16x4 v; uint32_t w[2]; uint2 h; };
 

@@ -42,12 +42,8 @@ struct F16 {
 };
 struct BF16 {
     static __device__ __forceinline__ float to_f(u16 v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
-    static __device__ __forceinline__ u16 from_f(float f) {   // round to nearest even
-        uint32_t u = __builtin_bit_cast(uint32_t, f);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (u16)(u >> 16);
-    }
+    // round to nearest even; gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32)
+    static __device__ __forceinline__ u16 from_f(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
     static __device__ __forceinline__ f32x4 mfma32(s16x8 a, s16x8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }

@@ -71,6 +71,12 @@ template <> __device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
     f32x2 v = {a, b};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
+template <> __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
 union Frag4 { s16x4 v; uint32_t w[2]; };
 
@@ -159,13 +165,15 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
+        // every lambda below is force-inlined: one left out of line would take the residual registers by reference,
+        // i.e. through scratch memory (seen with the bf16 instantiations, whose pack helper is larger)
         float kmask[RT][4];     // additive key mask for keys 4g..4g+3 of each env: 0 (attendable) or -inf
         f32x4 x[RT][NT];
         Frag8 hf[RT][KC];       // LayerNorm output as GEMM operand fragments
         Frag8 of[RT][KC];       // attention output fragments (chunk == head)
 
         // y = LN(x) * gamma + beta (or the raw x when !affine), packed as operand fragments
-        auto norm_to_frags = [&](const float* gptr, const float* bptr, bool normalise, Frag8 (&dst)[RT][KC]) {
+        auto norm_to_frags = [&](const float* gptr, const float* bptr, bool normalise, Frag8 (&dst)[RT][KC]) __attribute__((always_inline)) {
             float4 gm[NT], bt[NT];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -204,7 +212,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 }
             }
         };
-        auto add_bias = [&](const float* bptr) {
+        auto add_bias = [&](const float* bptr) __attribute__((always_inline)) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 b = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
@@ -214,7 +222,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
         };
 
         // ---- LN1 + QKV + attention of one block (12 stages), head by head: fills `of` ----
-        auto attention = [&](const float* lv) {
+        auto attention = [&](const float* lv) __attribute__((always_inline)) {
             norm_to_frags(lv + LV_LN1G, lv + LV_LN1B, true, hf);
 #pragma unroll
             for (int hd = 0; hd < H; ++hd) {
@@ -284,7 +292,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
         };
 
         // ---- output projection onto the residual (4 stages), then LN2 + FFN (2 * F/32 stages) ----
-        auto proj_and_ffn = [&](const float* lv) {
+        auto proj_and_ffn = [&](const float* lv) __attribute__((always_inline)) {
             add_bias(lv + LV_BOUT);
 #pragma unroll
             for (int st = 0; st < NT / 2; ++st) {
@@ -310,7 +318,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             constexpr int RH = RT / 2;                  // row tiles per activation half (RT == 1: no split)
             f32x4 accA[2][RT];
             Frag8 hidA[RT];                             // activation of the current chunk, as operand fragments
-            auto up_init = [&](int ch, f32x4 (&acc)[2][RT]) {
+            auto up_init = [&](int ch, f32x4 (&acc)[2][RT]) __attribute__((always_inline)) {
 #pragma unroll
                 for (int ntl = 0; ntl < 2; ++ntl) {
                     const float4 b = *reinterpret_cast<const float4*>(lv + LV_B1 + 32 * ch + 16 * ntl + 4 * g);
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 }
             };
             // activation of one (row tile, n-tile) accumulator = 4 hidden units -> 2 packed dwords
-            auto act4 = [&](const f32x4& v, Frag8& dst, int ntl) {
+            auto act4 = [&](const f32x4& v, Frag8& dst, int ntl) __attribute__((always_inline)) {
                 dst.w[ntl * 2] = pack2<DT>(apply_act16<ACT>(v[0]), apply_act16<ACT>(v[1]));
                 dst.w[ntl * 2 + 1] = pack2<DT>(apply_act16<ACT>(v[2]), apply_act16<ACT>(v[3]));
             };
@@ -465,7 +473,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
 
         // ---- 29*K + 1 output projection (8 stages); rf[i] = operand fragments whose rows are envs,
         //      row r16 of tile i being env env_base + i * 16 + r16 (stored when r16 < rows_valid) ----
-        auto heads = [&](auto& rf, int64_t env_base, int rows_valid, const float* fvp) {
+        auto heads = [&](auto& rf, int64_t env_base, int rows_valid, const float* fvp) __attribute__((always_inline)) {
             constexpr int NR = sizeof(rf) / sizeof(rf[0]);
             // The outputs stay in registers until the last stage has been consumed: stores count in the same
             // in-order vmcnt queue as the weight prefetches, so a store issued inside the stage loop would make
@@ -524,45 +532,57 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
-                if (a.tok_vec) {
-                    // a lane's 8 k slots per chunk are two runs of 4 consecutive obs lanes: k0 = 32 c + 4 g + 16 jh.
-                    // Only (c, jh) = (0, 0) falls in the object block (rows 1..15); every other run is proprio (row 0).
+            }
+            if (a.tok_vec) {
+                // a lane's 8 k slots per chunk are two runs of 4 consecutive obs lanes: k0 = 32 c + 4 g + 16 jh.
+                // Only (c, jh) = (0, 0) falls in the object block (rows 1..15); every other run is proprio (row 0).
+                // The lane coordinates go through an opaque copy: the 16 slot offsets and masks derived from them are
+                // tile-invariant, and hoisted out of the tile loop they would sit in (spilled) registers for the whole tile.
+                int tr = r16, tg = g;
+                asm volatile("" : "+v"(tr), "+v"(tg));
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
                     const float* orow = static_cast<const float*>(a.obs) + env * a.obs_ld;
 #pragma unroll
                     for (int c = 0; c < KC; ++c)
 #pragma unroll
                         for (int jh = 0; jh < 2; ++jh) {
-                            const int k0 = 32 * c + 4 * g + 16 * jh;
+                            const int k0 = 32 * c + 4 * tg + 16 * jh;
                             bool valid; int idx;
-                            if (c == 0 && jh == 0) { valid = r16 >= 1; idx = a.prop_dim + (r16 - 1) * 16 + k0; }
-                            else { valid = r16 == 0 && (k0 - 16) < a.prop_dim; idx = k0 - 16; }
+                            if (c == 0 && jh == 0) { valid = tr >= 1; idx = a.prop_dim + (tr - 1) * 16 + k0; }
+                            else { valid = tr == 0 && (k0 - 16) < a.prop_dim; idx = k0 - 16; }
                             const float4 v = *reinterpret_cast<const float4*>(orow + (valid ? idx : 0));
                             const uint32_t lo = pack2<DT>(v.x, v.y), hi = pack2<DT>(v.z, v.w);
                             e[rt][c].w[2 * jh] = valid ? lo : 0u;
                             e[rt][c].w[2 * jh + 1] = valid ? hi : 0u;
                         }
-                    continue;
                 }
-                float ev[KC][8];
+            } else {
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
+                for (int rt = 0; rt < RT; ++rt) {
+                    int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
+                    float ev[KC][8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int k = 32 * c + 4 * g + (j & 3) + (j >> 2) * 16;    // permuted k order
-                        int idx; bool on;
-                        if (k < 16) { on = r16 >= 1 && k < a.obj_dim; idx = a.prop_dim + (r16 - 1) * a.obj_dim + k; }
-                        else { on = r16 == 0 && (k - 16) < a.prop_dim; idx = k - 16; }
-                        float v = 0.f;
-                        if (on) {
-                            const int64_t off = env * a.obs_ld + idx;
-                            v = a.obs_f32 ? static_cast<const float*>(a.obs)[off] : DT::to_f(static_cast<const u16*>(a.obs)[off]);
+                    for (int c = 0; c < KC; ++c)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int k = 32 * c + 4 * g + (j & 3) + (j >> 2) * 16;    // permuted k order
+                            int idx; bool on;
+                            if (k < 16) { on = r16 >= 1 && k < a.obj_dim; idx = a.prop_dim + (r16 - 1) * a.obj_dim + k; }
+                            else { on = r16 == 0 && (k - 16) < a.prop_dim; idx = k - 16; }
+                            float v = 0.f;
+                            if (on) {
+                                const int64_t off = env * a.obs_ld + idx;
+                                v = a.obs_f32 ? static_cast<const float*>(a.obs)[off] : DT::to_f(static_cast<const u16*>(a.obs)[off]);
+                            }
+                            ev[c][j] = v;
                         }
-                        ev[c][j] = v;
-                    }
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
+                    for (int c = 0; c < KC; ++c)
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) e[rt][c].w[w] = pack2<DT>(ev[c][2 * w], ev[c][2 * w + 1]);
+                        for (int w = 0; w < 4; ++w) e[rt][c].w[w] = pack2<DT>(ev[c][2 * w], ev[c][2 * w + 1]);
+                }
             }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
