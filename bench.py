@@ -22,10 +22,10 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 # HBM bytes per forward of the headline workload (config[1], B = 16384, fp16, fused route with the final
 # block pruned: the HEAD + TAIL launch pair), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
 # dispatch) scaled by what the same counters read for a plain 256 MiB device copy (--calib-copy 256):
-# FETCH_SIZE reads 131084.7 for 262144 KiB fetched (factor 2.000), WRITE_SIZE reads 262144.0 (factor 1.000).
-#   fetched: HEAD 13400.4 x 2.000 + TAIL 7792.0 x 2.000 KiB; written: HEAD 12288.0 + TAIL 13559.7 KiB
+# FETCH_SIZE reads 131080 for 262144 KiB fetched (factor 2.000), WRITE_SIZE reads 262140 (factor 1.000).
+#   fetched: HEAD 13373 x 2.000 + TAIL 7784 x 2.000 KiB; written: HEAD 12288 + TAIL 13486 KiB
 # (profiles/cfg_forward_config1_b16384_f16.txt).  Other workloads report null.
-TRAFFIC_BYTES_CFG1_FUSED_PRUNED = int(((13400.4 + 7792.0) * 2.000 + 12288.0 + 13559.7) * 1024)
+TRAFFIC_BYTES_CFG1_FUSED_PRUNED = int(((13373 + 7784) * 2.000 + 12288 + 13486) * 1024)
 HBM_PEAK_GBS = 8000.0
 
 
