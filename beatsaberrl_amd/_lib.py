@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -67,6 +67,8 @@ SIGNATURES = {
     "bsrl_note_frontend": (_i32, [_p, _i64, _i32, _p, _p, _i32, _i32, _f, _p, _p, _p, _p, _p, _i64, _i32, _p]),
     "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _i32,
                                  _p, _p, _p, _p, _p, _p]),
+    "bsrl_vres_mix": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "bsrl_hsphere": (_i32, [_i32, _p, _p, C.c_float, _p, _p, _p, _i64, _i64, _i32, _p]),
 }
 
 _lib = None

@@ -1,0 +1,162 @@
+// Row-wise stages of two architecture options of the policy; HBM-bound elementwise / row-reduction work.
+//
+//  * value-residual mix (reference python/fp16_linear.py:1002-1006, python/policy.py:568-611):
+//        out = a * v + b * v0      fp32 arithmetic, rounded once to the stream dtype; (a, b) live on the device
+//    (learned scalars), exactly v at (a, b) = (1, 0).
+//  * SimBaV2 readout stages (reference python/policy.py:1140-1155, l2n :742-744): scalers, ReLU, row l2
+//    normalisation x / max(|x|, 1e-6) and the LERP in fp32 between the trunk's three GEMMs, each stored value
+//    rounded once.
+//
+// Rows are independent and a row's result never depends on the launch shape: one wave owns a row (fixed
+// butterfly reduction order), one thread owns 8 (16-bit) or 4 (fp32) consecutive elements of the mix.
+#include "bsrl_common.h"
+
+namespace {
+
+template <typename IO> struct El;
+template <> struct El<F16> { typedef u16 T; static __device__ __forceinline__ float f(u16 v) { return F16::to_f(v); }
+                             static __device__ __forceinline__ u16 r(float v) { return F16::from_f(v); } };
+template <> struct El<BF16> { typedef u16 T; static __device__ __forceinline__ float f(u16 v) { return BF16::to_f(v); }
+                              static __device__ __forceinline__ u16 r(float v) { return BF16::from_f(v); } };
+template <> struct El<F32IO> { typedef float T; static __device__ __forceinline__ float f(float v) { return v; }
+                               static __device__ __forceinline__ float r(float v) { return v; } };
+
+struct MixArgs {
+    const void* v; int64_t ldv; const void* v0; int64_t ldv0; const float* a; const float* b;
+    void* out; int64_t ldo; int64_t rows; int d;
+};
+
+// VEC consecutive elements per thread; the host picks VEC > 1 only when every row start is VEC-element aligned
+template <typename IO, int VEC>
+__global__ __launch_bounds__(256) void vres_mix_kernel(MixArgs m) {
+    typedef typename El<IO>::T T;
+    const int per_row = m.d / VEC;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= m.rows * per_row) return;
+    const int64_t row = i / per_row; const int c = (int)(i % per_row) * VEC;
+    const float a = *m.a, b = *m.b;
+    const T* pv = static_cast<const T*>(m.v) + row * m.ldv + c;
+    const T* p0 = static_cast<const T*>(m.v0) + row * m.ldv0 + c;
+    T* po = static_cast<T*>(m.out) + row * m.ldo + c;
+    if (VEC > 1) {
+        typedef T TV __attribute__((ext_vector_type(VEC > 1 ? VEC : 2)));
+        const TV xv = *reinterpret_cast<const TV*>(pv), x0 = *reinterpret_cast<const TV*>(p0);
+        TV o;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const float t = El<IO>::f(xv[j]) * a;                   // v * a, rounded to fp32 ...
+            o[j] = El<IO>::r(fmaf(El<IO>::f(x0[j]), b, t));         // ... then + v0 * b accumulated in fp32
+        }
+        *reinterpret_cast<TV*>(po) = o;
+    } else {
+        *po = El<IO>::r(fmaf(El<IO>::f(*p0), b, El<IO>::f(*pv) * a));
+    }
+}
+
+struct HsArgs {
+    int op; const void* t; const float* s; float c; const float* x32_in; float* x32_out; void* x_out;
+    int64_t rows; int D;
+};
+
+__device__ __forceinline__ float inv_l2(float sumsq) { return 1.0f / fmaxf(sqrtf(sumsq), 1e-6f); }
+
+// one wave per row; the row is re-read from cache for each pass instead of being held in registers
+template <typename IO>
+__global__ __launch_bounds__(256) void hsphere_kernel(HsArgs h) {
+    typedef typename El<IO>::T T;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= h.rows) return;
+    const int D = h.D;
+    const T* t = static_cast<const T*>(h.t) + row * D;
+    T* xo = h.x_out ? static_cast<T*>(h.x_out) + row * D : nullptr;
+    if (h.op == BSRL_HS_SCALE_RELU) {
+        for (int c = lane; c < D; c += 64) xo[c] = El<IO>::r(fmaxf(El<IO>::f(t[c]) * (h.s[c] * h.c), 0.0f));
+        return;
+    }
+    if (h.op == BSRL_HS_SCALE_L2N) {
+        float ss = 0.f;
+        for (int c = lane; c < D; c += 64) { const float v = El<IO>::f(t[c]) * (h.s[c] * h.c); ss += v * v; }
+        const float inv = inv_l2(group_sum<64>(ss));
+        float* x32 = h.x32_out + row * D;
+        for (int c = lane; c < D; c += 64) {
+            const float v = El<IO>::f(t[c]) * (h.s[c] * h.c) * inv;
+            x32[c] = v;
+            if (xo) xo[c] = El<IO>::r(v);
+        }
+        return;
+    }
+    // BSRL_HS_L2N_LERP: y = l2n(t); z = x + alpha (y - x); out = sqrt(D) l2n(z)
+    const float* x32 = h.x32_in + row * D;
+    float ss = 0.f;
+    for (int c = lane; c < D; c += 64) { const float v = El<IO>::f(t[c]); ss += v * v; }
+    const float inv_y = inv_l2(group_sum<64>(ss));
+    float zz = 0.f;
+    for (int c = lane; c < D; c += 64) {
+        const float x = x32[c], y = El<IO>::f(t[c]) * inv_y;
+        const float z = x + (h.s[c] * h.c) * (y - x);
+        zz += z * z;
+    }
+    const float inv_z = inv_l2(group_sum<64>(zz));
+    const float root = sqrtf((float)D);
+    for (int c = lane; c < D; c += 64) {
+        const float x = x32[c], y = El<IO>::f(t[c]) * inv_y;
+        const float z = x + (h.s[c] * h.c) * (y - x);
+        xo[c] = El<IO>::r(z * inv_z * root);
+    }
+}
+
+template <typename IO>
+int mix_launch(const MixArgs& m, int vec, hipStream_t st) {
+    const int64_t n = m.rows * (m.d / vec);
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (vec == 8) hipLaunchKernelGGL((vres_mix_kernel<IO, 8>), grid, block, 0, st, m);
+    else if (vec == 4) hipLaunchKernelGGL((vres_mix_kernel<IO, 4>), grid, block, 0, st, m);
+    else hipLaunchKernelGGL((vres_mix_kernel<IO, 1>), grid, block, 0, st, m);
+    BSRL_CHECK_LAUNCH("bsrl_vres_mix");
+    return BSRL_OK;
+}
+
+}  // namespace
+
+extern "C" int bsrl_vres_mix(const void* v, int64_t ldv, const void* v0, int64_t ldv0, const float* a, const float* b,
+                             void* out, int64_t ldo, int64_t rows, int64_t d, int dtype, bsrl_stream stream) {
+    if (!v || !v0 || !a || !b || !out) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: null pointer");
+    if (rows < 0 || d < 1 || d > (1 << 20) || ldv < d || ldv0 < d || ldo < d)
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: need rows >= 0, 1 <= d <= 2^20 and row pitches >= d");
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: bad dtype %d", dtype);
+    if (rows == 0) return BSRL_OK;
+    if (rows * d > ((int64_t)1 << 40)) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: rows * d too large");
+    const int want = dtype == BSRL_F32 ? 4 : 8;                    // 16-byte accesses
+    const bool vec_ok = d % want == 0 && ldv % want == 0 && ldv0 % want == 0 && ldo % want == 0 &&
+                        bsrl_aligned(v, 16) && bsrl_aligned(v0, 16) && bsrl_aligned(out, 16);
+    const int vec = vec_ok ? want : 1;
+    if ((rows * (d / vec) + 255) / 256 > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: grid too large");
+    const MixArgs m{v, ldv, v0, ldv0, a, b, out, ldo, rows, (int)d};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == BSRL_F32) return mix_launch<F32IO>(m, vec, st);
+    if (dtype == BSRL_F16) return mix_launch<F16>(m, vec, st);
+    return mix_launch<BF16>(m, vec, st);
+}
+
+extern "C" int bsrl_hsphere(int op, const void* t, const float* s, float c, const float* x32_in, float* x32_out,
+                            void* x_out, int64_t rows, int64_t D, int dtype, bsrl_stream stream) {
+    if (op != BSRL_HS_SCALE_L2N && op != BSRL_HS_SCALE_RELU && op != BSRL_HS_L2N_LERP)
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: unknown op %d", op);
+    if (!t || !s) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: null input / scaler");
+    if (op == BSRL_HS_SCALE_L2N && !x32_out) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: SCALE_L2N needs x32_out");
+    if (op == BSRL_HS_SCALE_RELU && !x_out) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: SCALE_RELU needs x_out");
+    if (op == BSRL_HS_L2N_LERP && (!x32_in || !x_out)) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: L2N_LERP needs x32_in and x_out");
+    if (rows < 0 || D < 1 || D > 65536) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: need rows >= 0 and 1 <= D <= 65536");
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: bad dtype %d", dtype);
+    if (rows == 0) return BSRL_OK;
+    if ((rows + 3) / 4 > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_hsphere: too many rows");
+    const HsArgs h{op, t, s, c, x32_in, x32_out, x_out, rows, (int)D};
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == BSRL_F32) hipLaunchKernelGGL(hsphere_kernel<F32IO>, grid, block, 0, st, h);
+    else if (dtype == BSRL_F16) hipLaunchKernelGGL(hsphere_kernel<F16>, grid, block, 0, st, h);
+    else hipLaunchKernelGGL(hsphere_kernel<BF16>, grid, block, 0, st, h);
+    BSRL_CHECK_LAUNCH("bsrl_hsphere");
+    return BSRL_OK;
+}

@@ -309,6 +309,77 @@ def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, acti
     return act_out, logprob, entropy, ent_h, noise
 
 
+# ---- architecture options: value-residual mix, SimBaV2 row stages -------------------------
+def _view2d(t, name):
+    """(rows, d, pitch) of a tensor whose last dim is dense and whose leading dims form one
+    uniform row pitch (a column slice of a packed q|k|v buffer qualifies)."""
+    if t.dim() < 2 or t.stride(-1) != 1:
+        raise TypeError(f"{name}: need a tensor with a unit-stride last dim")
+    lead = [(n, st) for n, st in zip(t.shape[:-1], t.stride()[:-1]) if n != 1]
+    pitch = lead[-1][1] if lead else t.shape[-1]
+    for (_, st_outer), (n_inner, st_inner) in zip(lead[:-1], lead[1:]):
+        if st_outer != st_inner * n_inner:
+            raise TypeError(f"{name}: rows must have one uniform pitch")
+    rows = 1
+    for n in t.shape[:-1]:
+        rows *= n
+    return rows, t.shape[-1], pitch
+
+
+def vres_mix(v, v0, a, b, out=None):
+    """out = a * v + b * v0 in fp32, rounded once to v's dtype (reference fp16_linear.vres_mix,
+    python/fp16_linear.py:1002-1006).  a, b: fp32 (1,) device tensors.  v / v0 / out may be
+    column slices of packed projection buffers; out=None mixes in place into v."""
+    _need_cuda(v, v0, a, b, out)
+    out = v if out is None else out
+    if v0.shape != v.shape or out.shape != v.shape or v0.dtype is not v.dtype or out.dtype is not v.dtype:
+        raise TypeError("vres_mix: v, v0 and out must share shape and dtype")
+    for s in (a, b):
+        if s.dtype is not torch.float32 or s.numel() != 1:
+            raise TypeError("vres_mix: a and b must be fp32 tensors with one element")
+    rows, d, ldv = _view2d(v, "vres_mix v")
+    _, _, ldv0 = _view2d(v0, "vres_mix v0")
+    _, _, ldo = _view2d(out, "vres_mix out")
+    with torch.cuda.device(v.device):
+        rc = _lib.load().bsrl_vres_mix(v.data_ptr(), ldv, v0.data_ptr(), ldv0, a.data_ptr(), b.data_ptr(),
+                                       out.data_ptr(), ldo, rows, d, dt_code(v.dtype), _stream(v))
+    _lib.check(rc, "bsrl_vres_mix")
+    return out
+
+
+HS_SCALE_L2N, HS_SCALE_RELU, HS_L2N_LERP = 0, 1, 2
+
+
+def hsphere(op, t, s, c=1.0, x32=None):
+    """One fp32 row stage of the SimBaV2 trunk on a GEMM output t (rows, D)
+    (reference NotePolicy._trunk_v2, python/policy.py:1140-1155):
+      HS_SCALE_L2N  -> (x32 fp32, x in t's dtype) = l2n(t * (s * c))
+      HS_SCALE_RELU -> relu(t * (s * c)) in t's dtype
+      HS_L2N_LERP   -> sqrt(D) * l2n(x32 + (s * c) * (l2n(t) - x32)) in t's dtype"""
+    _need_cuda(t, s, x32)
+    if t.dim() != 2 or not t.is_contiguous():
+        raise TypeError("hsphere: t must be a contiguous (rows, D) tensor")
+    rows, D = t.shape
+    s = _f32c(s, "hsphere scaler")
+    if s.numel() != D:
+        raise TypeError(f"hsphere: scaler has {s.numel()} lanes, rows have {D}")
+    x32_in = x32_out = None
+    out = torch.empty_like(t)
+    if op == HS_SCALE_L2N:
+        x32_out = torch.empty(rows, D, device=t.device, dtype=torch.float32)
+    elif op == HS_L2N_LERP:
+        if x32 is None or x32.dtype is not torch.float32 or x32.shape != t.shape or not x32.is_contiguous():
+            raise TypeError("hsphere: HS_L2N_LERP needs the contiguous fp32 x32 of the first stage")
+        x32_in = x32
+    elif op != HS_SCALE_RELU:
+        raise ValueError(f"hsphere: unknown op {op}")
+    with torch.cuda.device(t.device):
+        rc = _lib.load().bsrl_hsphere(op, t.data_ptr(), s.data_ptr(), float(c), _ptr(x32_in), _ptr(x32_out),
+                                      out.data_ptr(), rows, D, dt_code(t.dtype), _stream(t))
+    _lib.check(rc, "bsrl_hsphere")
+    return (x32_out, out) if op == HS_SCALE_L2N else out
+
+
 # ---- fused transformer block stack ----------------------------------------------------
 def _blocks_desc(n_layers, d, n_heads, ffn, T, act, n_queries, dtype):
     return _lib.BlocksDesc(n_layers=n_layers, d=d, n_heads=n_heads, ffn=ffn, T=T, act=_ACT[act],

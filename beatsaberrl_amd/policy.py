@@ -19,8 +19,9 @@ same state_dict and checkpoints) and the same `forward_stacked(obs) -> (logits
 Stream dtype: `policy.fp16 = True` runs the 16-bit stream (fp16; set `stream_dtype =
 torch.bfloat16` for bf16) exactly as the reference's switch does (python/policy.py:
 1085-1090); otherwise fp32 kernels.  There is no CPU path and no torch fallback for
-the kernel ops.  Not implemented (raise at construction): value_residual, the simbav2
-trunk."""
+the kernel ops.  Architecture options: emb_ln, final_ln, ragged per-joint heads, the
+value-residual mix (per-op route; its row kernel mixes inside the packed q|k|v buffer)
+and the SimBaV2 trunk (three GEMMs + three fp32 row kernels)."""
 from __future__ import annotations
 
 import contextlib
@@ -122,10 +123,17 @@ class Block(nn.Module):
     """Pre-LN transformer block; parameters as the reference's Block
     (python/policy.py:492-522): ln_attn, q/k/v/out_proj, ln_ffn, ffn.{0,2}."""
 
-    def __init__(self, d: int, n_heads: int = 4, ffn_mult: int = 4):
+    def __init__(self, d: int, n_heads: int = 4, ffn_mult: int = 4, value_residual: bool = False):
         super().__init__()
         if n_heads < 2 or d % n_heads:
             raise ValueError(f"embed {d} must split into >= 2 heads, got n_heads={n_heads}")
+        # value residual (python/policy.py:511-522): v <- a v + b v0 with block 0's values v0;
+        # (a, b) = (1, 0) at init is bitwise the plain block
+        if value_residual:
+            self.vres_a = nn.Parameter(torch.ones(1))
+            self.vres_b = nn.Parameter(torch.zeros(1))
+        else:
+            self.vres_a = self.vres_b = None
         self.ln_attn = FusedLayerNorm(d)
         self.q_proj = nn.Linear(d, d)
         self.k_proj = nn.Linear(d, d)
@@ -135,18 +143,24 @@ class Block(nn.Module):
         self.ffn = _mlp([d, ffn_mult * d, d])
         self.d, self.n_heads, self.dh = d, n_heads, d // n_heads
 
-    def forward(self, x, attn_bias, h=None, n_queries=0, next_ln=None):
+    def forward(self, x, attn_bias, h=None, n_queries=0, next_ln=None, v0=None, want_v=False):
         """x (B, T, d); attn_bias (B, T) additive key bias; h = ln_attn(x) if the
         previous block's fused FFN already produced it.  n_queries > 0 computes only
         the first n_queries rows (keys / values still span all T): exact, masking is
-        key-side only (reference python/policy.py:533-539).  Returns (x_out, h_next)
-        with h_next = next_ln(x_out) when the fused FFN produced it, else None."""
+        key-side only (reference python/policy.py:533-539).  v0: block 0's attention
+        values, mixed into this block's (a v + b v0, python/policy.py:568-611) before the
+        attention.  Returns (x_out, h_next) with h_next = next_ln(x_out) when the fused FFN
+        produced it, else None; with want_v (block 0 of a value-residual stack) a third element,
+        this block's values as a view of its packed projection."""
         d = self.d
         if h is None:
             h = self.ln_attn(x)
         if n_queries:
             wkv, bkv = _fl.packed_halves([self.k_proj, self.v_proj], x.dtype)
             kv = ops.linear(h, wkv, bkv)                                   # (B, T, 2d)
+            v = kv[..., d:]
+            if v0 is not None:
+                ops.vres_mix(v, v0, self.vres_a, self.vres_b)              # in place in the packed buffer
             hq = h[:, :n_queries]
             q = _lin(self.q_proj, hq)                                      # (B, nq, d)
             att = ops.attn_fwd(q, kv[..., :d], kv[..., d:], self.n_heads, key_bias=attn_bias)
@@ -154,14 +168,19 @@ class Block(nn.Module):
         else:
             wqkv, bqkv = _fl.packed_halves([self.q_proj, self.k_proj, self.v_proj], x.dtype)
             qkv = ops.linear(h, wqkv, bqkv)                                # (B, T, 3d)
+            v = qkv[..., 2 * d:]
+            if v0 is not None:
+                ops.vres_mix(v, v0, self.vres_a, self.vres_b)
             att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, key_bias=attn_bias)
         x = _lin(self.out_proj, att, residual=x)                           # x + out(att), one rounding
         h2 = self.ln_ffn(x)
         if _fl.fused_ffn_ok(x, self.ffn, next_ln):
             r = _fl.fused_ffn(x, h2, self.ffn, next_ln)
-            return (r, None) if next_ln is None else r
-        hid = _lin(self.ffn[0], h2, act="relu")
-        return _lin(self.ffn[2], hid, residual=x), None
+            r = (r, None) if next_ln is None else tuple(r)
+        else:
+            hid = _lin(self.ffn[0], h2, act="relu")
+            r = (_lin(self.ffn[2], hid, residual=x), None)
+        return r + (v,) if want_v else r
 
 
 def build_head_gears(n_gears: int) -> tuple:
@@ -181,10 +200,6 @@ class NotePolicy(nn.Module):
         super().__init__()
         if trunk_arch not in TRUNK_ARCHS:
             raise ValueError(f"trunk_arch must be one of {TRUNK_ARCHS}, got {trunk_arch!r}")
-        if trunk_arch != "simba":
-            raise NotImplementedError("the simbav2 trunk is not built on the HIP kernels yet")
-        if value_residual:
-            raise NotImplementedError("value_residual is not built on the HIP kernels yet")
         if game not in ("standard", "flux"):
             raise ValueError(f"game must be 'standard' or 'flux', got {game!r}")
         if not float(z_asinh) > 0:
@@ -214,7 +229,7 @@ class NotePolicy(nn.Module):
                      "trunk_arch": trunk_arch, "trunk_hidden": H, "value_bins": int(value_bins),
                      "value_vmax": float(value_vmax), "value_sigma": float(value_sigma), "game": game,
                      "fp16_accum": fp16_accum, "fused_ffn": fused_ffn, "emb_ln": bool(emb_ln),
-                     "value_residual": False, "final_ln": bool(final_ln)}
+                     "value_residual": bool(value_residual), "final_ln": bool(final_ln)}
         if head_gears != (n_gears,) * N_ACTION_HEADS:
             self.arch["head_gears"] = list(head_gears)
         self.value_bins = int(value_bins)
@@ -229,16 +244,37 @@ class NotePolicy(nn.Module):
         self.body_tokens, self.n_lead = 3, L.N_LEAD
         self.torso_mlp = _mlp([TORSO_FEAT, embed, embed])
         self.leg_mlp = _mlp([LEG_FEAT + 2, embed, embed])
-        self.value_residual = False
+        self.value_residual = bool(value_residual)
         self.emb_ln = FusedLayerNorm(embed) if emb_ln else None
-        self.blocks = nn.ModuleList(Block(embed, n_heads, ffn_mult) for _ in range(n_blocks))
+        self.blocks = nn.ModuleList(Block(embed, n_heads, ffn_mult, value_residual=self.value_residual and i > 0)
+                                    for i in range(n_blocks))
         self.final_ln = FusedLayerNorm(embed) if final_ln else None
         self.trunk_arch = trunk_arch
-        self.trunk_proj = nn.Linear(self.n_lead * embed, trunk_dim)
-        self.trunk_ln1 = FusedLayerNorm(trunk_dim)
-        self.trunk_fc1 = nn.Linear(trunk_dim, H)
-        self.trunk_fc2 = nn.Linear(H, trunk_dim)
-        self.trunk_ln2 = FusedLayerNorm(trunk_dim)
+        if trunk_arch == "simba":
+            self.trunk_proj = nn.Linear(self.n_lead * embed, trunk_dim)
+            self.trunk_ln1 = FusedLayerNorm(trunk_dim)
+            self.trunk_fc1 = nn.Linear(trunk_dim, H)
+            self.trunk_fc2 = nn.Linear(H, trunk_dim)
+            self.trunk_ln2 = FusedLayerNorm(trunk_dim)
+        else:
+            # SimBaV2 readout (python/policy.py:990-1014): three bias-free (zero, frozen bias)
+            # Linears with unit-norm rows and orthogonal init, per-lane scalers s_in / s_1 at
+            # sqrt(2 / width) and the LERP rate alpha at 0.5 (stored as alpha / (0.5 sqrt(D)))
+            D = trunk_dim
+            self.trunk_in = nn.Linear(self.n_lead * embed, D)
+            self.trunk_w1 = nn.Linear(D, H)
+            self.trunk_w2 = nn.Linear(H, D)
+            for lin in (self.trunk_in, self.trunk_w1, self.trunk_w2):
+                nn.init.orthogonal_(lin.weight)
+                nn.init.zeros_(lin.bias)
+                lin.bias.requires_grad_(False)
+            self._v2_c_in = self._v2_c_1 = 1.0
+            self.trunk_s_in = nn.Parameter(torch.full((D,), math.sqrt(2.0 / D)))
+            self.trunk_s_1 = nn.Parameter(torch.full((H,), math.sqrt(2.0 / H)))
+            a_init, a_scale = 0.5, 1.0 / math.sqrt(D)
+            self._v2_c_alpha = a_init / a_scale
+            self.trunk_alpha = nn.Parameter(torch.full((D,), a_scale))
+            self.project_trunk_weights()
         self.heads = nn.ModuleList(nn.Linear(trunk_dim, n) for n in self.head_sizes)
         if min(self.head_sizes) < self.k_max:
             self.register_buffer("_gear_valid", torch.tensor([[a < k for a in range(self.k_max)]
@@ -290,8 +326,8 @@ class NotePolicy(nn.Module):
 
     def fused_blocks_ok(self, dt) -> bool:
         """True when the block stack of this architecture has a fused kernel in dtype dt."""
-        if self.fused_blocks == "off" or dt is torch.float32:
-            return False
+        if self.fused_blocks == "off" or dt is torch.float32 or self.value_residual:
+            return False                    # the value-residual mix has no place in the fused stack
         if self.fused_blocks != "auto":
             raise ValueError(f"fused_blocks must be 'auto' or 'off', got {self.fused_blocks!r}")
         return ops.blocks_pack_size(len(self.blocks), **self._blocks_desc(dt)) > 0
@@ -390,10 +426,14 @@ class NotePolicy(nn.Module):
         else:
             h = None
             nb = len(self.blocks)
+            v0 = None
             for i in range(nb - 1):
-                x, h = self.blocks[i](x, attn_bias, h=h, next_ln=self.blocks[i + 1].ln_attn)
+                if self.value_residual and i == 0:                         # block 0's values feed every later block
+                    x, h, v0 = self.blocks[0](x, attn_bias, h=h, next_ln=self.blocks[1].ln_attn, want_v=True)
+                else:
+                    x, h = self.blocks[i](x, attn_bias, h=h, next_ln=self.blocks[i + 1].ln_attn, v0=v0)
             x_res = x                                                      # the stream entering the final block
-            lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead)
+            lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead, v0=v0)
         if self.final_ln is not None:
             lead = self.final_ln(lead)
         hfeat = self._trunk(lead.reshape(B, self.n_lead * d))
@@ -404,8 +444,33 @@ class NotePolicy(nn.Module):
             out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
         return out.view(B, N_ACTION_HEADS, self.k_max), value
 
+    def trunk_projected(self):
+        """The Linears whose rows `project_trunk_weights` keeps unit-norm (python/policy.py:1157-1162)."""
+        return [self.trunk_in, self.trunk_w1, self.trunk_w2] if self.trunk_arch == "simbav2" else []
+
+    @torch.no_grad()
+    def project_trunk_weights(self) -> bool:
+        """SimBaV2 weight projection, in place on the fp32 masters (python/policy.py:1164-1178): every
+        output row back onto the unit sphere, frozen biases at 0.  The caller bumps the weights
+        version afterwards, as after an optimizer step.  No-op (False) for the SimBa trunk."""
+        lins = self.trunk_projected()
+        for lin in lins:
+            w = lin.weight
+            w.div_(w.norm(dim=1, keepdim=True).clamp_min(1e-12))
+            lin.bias.zero_()
+        return bool(lins)
+
+    def _trunk_v2(self, z):
+        """SimBaV2 readout (python/policy.py:1140-1155): GEMMs on the stream dtype, the fp32 row
+        work between them (scalers, ReLU, l2 normalisation, LERP) in one kernel per stage."""
+        x32, x = ops.hsphere(ops.HS_SCALE_L2N, _lin(self.trunk_in, z), self.trunk_s_in, self._v2_c_in)
+        u = ops.hsphere(ops.HS_SCALE_RELU, _lin(self.trunk_w1, x), self.trunk_s_1, self._v2_c_1)
+        return ops.hsphere(ops.HS_L2N_LERP, _lin(self.trunk_w2, u), self.trunk_alpha, self._v2_c_alpha, x32=x32)
+
     def _trunk(self, x):
         """SimBa readout: proj -> LN1 -> fc1 -> ReLU -> fc2 -> (+proj) -> LN2 (policy.py:1107-1138)."""
+        if self.trunk_arch == "simbav2":
+            return self._trunk_v2(x)
         t = _lin(self.trunk_proj, x)
         u = self.trunk_ln1(t)
         r = _lin(self.trunk_fc1, u, act="relu")

@@ -253,6 +253,35 @@ int bsrl_blocks_forward(const bsrl_blocks_desc* desc, const void* packed,
                         const void* x_in, const void* key_bias,
                         void* x_res, void* x_out, int64_t B, bsrl_stream stream);
 
+/* ---- Value-residual mix -------------------------------------------------------
+ * out = a * v + b * v0: what every block after the first does to its attention
+ * values under the reference's value_residual option (fp16_linear.vres_mix,
+ * python/fp16_linear.py:1002-1006; call site python/policy.py:568-611).  fp32
+ * arithmetic ((v * a) rounded to fp32, then + v0 * b fused), one rounding to
+ * `dtype`; exactly v at (a, b) = (1, 0).  a, b: device pointers to the learned
+ * fp32 scalars (no host read).  v, v0, out: (rows, d) with row pitches ldv,
+ * ldv0, ldo in elements (views into packed q|k|v buffers); out may alias v. */
+int bsrl_vres_mix(const void* v, int64_t ldv, const void* v0, int64_t ldv0,
+                  const float* a, const float* b, void* out, int64_t ldo,
+                  int64_t rows, int64_t d, int dtype, bsrl_stream stream);
+
+/* ---- SimBaV2 readout stages ----------------------------------------------------
+ * The fp32 row work between the three GEMMs of the reference's hyperspherical
+ * trunk (NotePolicy._trunk_v2, python/policy.py:1140-1155; l2n = F.normalize
+ * with eps 1e-6, :742-744), with l2n(x) = x / max(|x|_2, 1e-6), t (rows, D) in
+ * `dtype` (a GEMM output), s (D) fp32 scaler and c its constant factor:
+ *   BSRL_HS_SCALE_L2N : x = l2n(t * (s * c))      -> x32_out (rows, D) fp32 and,
+ *                       if x_out is not NULL, the same rounded to `dtype`
+ *   BSRL_HS_SCALE_RELU: x_out = relu(t * (s * c))  rounded to `dtype`
+ *   BSRL_HS_L2N_LERP  : y = l2n(t); z = l2n(x32_in + (s * c) * (y - x32_in));
+ *                       x_out = sqrt(D) * z rounded to `dtype` */
+#define BSRL_HS_SCALE_L2N 0
+#define BSRL_HS_SCALE_RELU 1
+#define BSRL_HS_L2N_LERP 2
+int bsrl_hsphere(int op, const void* t, const float* s, float c,
+                 const float* x32_in, float* x32_out, void* x_out,
+                 int64_t rows, int64_t D, int dtype, bsrl_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

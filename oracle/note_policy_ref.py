@@ -11,6 +11,8 @@ following the reference's fp32 record path:
   * key bias                   reference python/policy.py:428, 1257-1260
   * blocks, final-block pruning reference python/policy.py:524-715 (`else` arms), 1267-1305
   * SimBa readout trunk        reference python/policy.py:1107-1138
+  * SimBaV2 readout trunk      reference python/policy.py:1140-1155 (scalers :1003-1014)
+  * value residual (a v + b v0) reference python/policy.py:568-611, 1264-1275; fp16_linear.py:1002-1006
   * packed heads + ragged fill reference python/policy.py:1311-1344, 430-434
   * adapool critic             reference python/policy.py:1346-1403
 
@@ -18,8 +20,9 @@ Pinned (tests/test_oracle_notepolicy.py) against tests/golden/notepolicy_*.npz, 
 written by the reference module itself (tests/golden/make_notepolicy_golden.py), and
 against the hand-computed note-geometry cases the reference's own tests hold
 (python/tests/test_policy.py:141-183, test_i07_blade_geo.py:149-200 - restated there).
-Not covered here: the value_residual option and the simbav2 trunk ("parity unpinned":
-neither this oracle nor the product implements them).
+The value-residual mix and the SimBaV2 trunk are pinned by the notepolicy_vres_v2 vector and
+by the reference's own properties (python/tests/test_arch_ab_options.py:131-139, 250-256:
+(a, b) = (1, 0) is bitwise the plain policy; the SimBaV2 feature has RMS 1 per row).
 
 `forward(..., emulate="f16")` restates the rounding points of the 16-bit stream (obs,
 weights and every GEMM operand rounded, fp32 accumulate, fp32 LayerNorm / softmax /
@@ -167,10 +170,17 @@ def _blocks(net, arch, x, bias, round_residual=True):
     rr = r if round_residual else (lambda t: t)
     H, L = arch["n_heads"], arch["n_blocks"]
 
+    vres = bool(arch.get("value_residual", False))
+    v0 = [None]
+
     def block(i, x, n_q):
         p = f"blocks.{i}."
         h = r(net.ln(p + "ln_attn", x))
         k, v = r(net.lin(p + "k_proj", h)), r(net.lin(p + "v_proj", h))
+        if vres and i == 0:
+            v0[0] = v                       # block 0 hands its values to every later block
+        elif vres:
+            v = r(v * net.sd[p + "vres_a"] + v0[0] * net.sd[p + "vres_b"])
         x_full = x
         if n_q:
             x, h = x[:, :n_q], h[:, :n_q]
@@ -212,6 +222,26 @@ def frontend(obs, note_geo_on=False, flux=False, z_asinh=8.0, emulate=None):
     return torch.cat([sab, eye], -1), obs[:, TORSO], torch.cat([legs, eye], -1), notes, r(bias)
 
 
+def _l2n(x):
+    return x / x.norm(dim=-1, keepdim=True).clamp_min(1e-6)
+
+
+def _trunk_v2(net, arch, z):
+    """SimBaV2 readout (reference python/policy.py:1140-1155): x = l2n(s_in * W_in z);
+    y = l2n(W2 relu(s_1 * W1 x)); x = l2n(x + alpha (y - x)); h = sqrt(D) x.  GEMM outputs are
+    rounded to the stream dtype; scalers, ReLU, normalisations and the LERP stay fp32 and are
+    rounded once before each GEMM and at the output.  Scaler factors (:1003-1014): s_in and s_1
+    enter as they are, alpha times 0.5 * sqrt(D)."""
+    r, sd = net.r, net.sd
+    D = arch["trunk_dim"]
+    x = _l2n(r(net.lin("trunk_in", z)) * sd["trunk_s_in"])
+    u = F.relu(r(net.lin("trunk_w1", r(x))) * sd["trunk_s_1"])
+    y = _l2n(r(net.lin("trunk_w2", r(u))))
+    alpha = sd["trunk_alpha"] * (0.5 * math.sqrt(D))
+    x = _l2n(x + alpha * (y - x))
+    return r(x * math.sqrt(D))
+
+
 @torch.no_grad()
 def forward(sd, arch, obs, emulate=None, return_parts=False):
     """obs (B, 630) -> logits (B, 29, k_max) fp32, value (B,) fp32."""
@@ -241,11 +271,14 @@ def forward(sd, arch, obs, emulate=None, return_parts=False):
     lead, x_res = _blocks(net, arch, x, bias)
     if arch.get("final_ln", False):
         lead = r(net.ln("final_ln", lead))
-    # SimBa readout trunk
-    t = r(net.lin("trunk_proj", lead.reshape(B, N_LEAD * d)))
-    u = r(net.ln("trunk_ln1", t))
-    dlt = net.lin("trunk_fc2", r(F.relu(net.lin("trunk_fc1", u))))
-    h = r(net.ln("trunk_ln2", r(t + dlt)))
+    if arch.get("trunk_arch", "simba") == "simbav2":
+        h = _trunk_v2(net, arch, lead.reshape(B, N_LEAD * d))
+    else:
+        # SimBa readout trunk
+        t = r(net.lin("trunk_proj", lead.reshape(B, N_LEAD * d)))
+        u = r(net.ln("trunk_ln1", t))
+        dlt = net.lin("trunk_fc2", r(F.relu(net.lin("trunk_fc1", u))))
+        h = r(net.ln("trunk_ln2", r(t + dlt)))
     # packed heads
     sizes = arch.get("head_gears") or [arch["n_gears"]] * N_HEADS_OUT
     w = torch.cat([sd[f"heads.{j}.weight"] for j in range(N_HEADS_OUT)])

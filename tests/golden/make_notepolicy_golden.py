@@ -3,7 +3,7 @@ reference's NotePolicy on CPU fp32.
 
 Run ONCE in the build container, where the reference checkout is mounted read-only:
 
-    python tests/golden/make_notepolicy_golden.py [/root/reference/python]
+    python tests/golden/make_notepolicy_golden.py [/root/reference/python [case ...]]
 
 The composition of the full forward (token order, one-hot placement, the 40-lane note
 input order, trunk wiring, the critic's use of token 2 and of the pre-final-block stream)
@@ -21,6 +21,7 @@ import numpy as np
 import torch
 
 REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference/python"
+ONLY = set(sys.argv[2:])          # optional: write just these cases
 sys.path.insert(0, REF)
 import policy as ref_policy  # noqa: E402
 
@@ -36,6 +37,10 @@ CASES = {
     "notepolicy_flux": (dict(embed=64, trunk_dim=64, n_blocks=1, n_heads=2, n_gears=3, ffn_mult=4, note_geo=True,
                              game="flux", z_asinh=4.0, value_bins=51, value_vmax=4.0,
                              head_gears=(3,) * 29), 5, 2),
+    # the value-residual mix (blocks 1.. read block 0's values) and the SimBaV2 readout trunk
+    "notepolicy_vres_v2": (dict(embed=64, trunk_dim=96, n_blocks=3, n_heads=2, n_gears=5, ffn_mult=2, note_geo=True,
+                                value_residual=True, trunk_arch="simbav2", trunk_hidden=128,
+                                head_gears=(5,) * 29), 6, 3),
 }
 
 
@@ -55,6 +60,8 @@ def make_obs(n, seed):
 
 def main():
     for name, (kw, B, seed) in CASES.items():
+        if ONLY and name not in ONLY:
+            continue
         torch.manual_seed(100 + seed)
         m = ref_policy.NotePolicy(**kw).eval()
         with torch.no_grad():

@@ -47,11 +47,44 @@ def test_refusals():
         load_policy({"arch": {**arch, "game": "flux"}, "state_dict": sd})
     with pytest.raises(SystemExit):
         load_policy({"arch": {k: v for k, v in arch.items() if k != "z_asinh"}, "state_dict": sd})
-    with pytest.raises(NotImplementedError):
-        NotePolicy(value_residual=True)
-    with pytest.raises(NotImplementedError):
-        NotePolicy(trunk_arch="simbav2")
+    with pytest.raises(ValueError):
+        NotePolicy(trunk_arch="simbav3")
     with pytest.raises(ValueError):
         NotePolicy(n_gears=4)
     with pytest.raises(RuntimeError, match="GPU only"):
         NotePolicy().forward_stacked(torch.zeros(1, 630))
+
+
+def test_option_modules_exist_only_when_on_and_register_in_the_reference_order():
+    """python/tests/test_arch_ab_options.py:131-135, 190-207."""
+    kw = dict(embed=64, trunk_dim=96, n_blocks=3, n_heads=2, n_gears=5)
+    p = NotePolicy(**kw)
+    assert p.emb_ln is None and p.final_ln is None and all(b.vres_a is None for b in p.blocks)
+    q = NotePolicy(emb_ln=True, value_residual=True, final_ln=True, trunk_arch="simbav2", **kw)
+    assert q.blocks[0].vres_a is None                       # block 0 provides v0
+    for blk in q.blocks[1:]:
+        assert blk.vres_a.item() == 1.0 and blk.vres_b.item() == 0.0
+    order = [n for n, _ in q.named_parameters()]
+    assert {"emb_ln.weight", "final_ln.weight", "blocks.1.vres_b", "trunk_alpha", "trunk_in.weight"} <= set(order)
+    assert not any(n.startswith(("trunk_proj", "trunk_ln", "trunk_fc")) for n in order)
+    assert order.index("emb_ln.bias") < order.index("blocks.0.ln_attn.weight")
+    assert order.index("blocks.2.vres_b") < order.index("final_ln.weight") < order.index("trunk_in.weight")
+    assert q.arch["value_residual"] is True and q.arch["trunk_arch"] == "simbav2"
+
+
+def test_simbav2_init_and_projection():
+    """python/tests/test_arch_ab_options.py:220-256: unit-norm rows, zero frozen biases, alpha at 0.5."""
+    p = NotePolicy(embed=64, trunk_dim=96, n_blocks=2, n_heads=2, n_gears=5, trunk_arch="simbav2", trunk_hidden=128)
+    assert [m.weight.shape for m in p.trunk_projected()] == [(96, 320), (128, 96), (96, 128)]
+    for m in p.trunk_projected():
+        assert torch.allclose(m.weight.norm(dim=1), torch.ones(m.weight.shape[0]), atol=1e-6)
+        assert torch.count_nonzero(m.bias) == 0 and not m.bias.requires_grad
+    assert torch.allclose(p.trunk_alpha * p._v2_c_alpha, torch.full((96,), 0.5))
+    assert torch.allclose(p.trunk_s_in, torch.full((96,), (2.0 / 96) ** 0.5))
+    with torch.no_grad():
+        p.trunk_w1.weight.mul_(3.0)
+        p.trunk_w1.bias.add_(1.0)
+    assert p.project_trunk_weights()
+    assert torch.allclose(p.trunk_w1.weight.norm(dim=1), torch.ones(128), atol=1e-6)
+    assert torch.count_nonzero(p.trunk_w1.bias) == 0
+    assert not NotePolicy(embed=64, trunk_dim=96, n_blocks=2, n_heads=2).project_trunk_weights()

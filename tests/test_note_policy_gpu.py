@@ -48,7 +48,10 @@ def test_fp32_matches_reference_golden_vectors(path):
     assert len(lst) == 29 and torch.equal(lst[3].cpu(), lg[:, 3])
 
 
-@pytest.mark.parametrize("path", GOLD[:2], ids=[os.path.basename(p)[:-4] for p in GOLD[:2]])
+_GOLD16 = GOLD[:2] + GOLD[3:]
+
+
+@pytest.mark.parametrize("path", _GOLD16, ids=[os.path.basename(p)[:-4] for p in _GOLD16])
 def test_fp16_stream_on_golden_vectors(path):
     arch, sd, obs, logits, value = nr.load_fixture(path)
     m = load_policy({"arch": arch, "state_dict": sd}, game=arch["game"]).to(DEV)
@@ -70,6 +73,8 @@ def _big(seed, **kw):
     return m, sd
 
 
+_VRES_V2 = dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,
+                value_residual=True, trunk_arch="simbav2", trunk_hidden=512)
 _RAGGED = dict(embed=128, trunk_dim=256, n_blocks=2, n_heads=4, n_gears=7, ffn_mult=2, emb_ln=True, final_ln=True,
                note_geo=True, head_gears=tuple(7 if j in (8, 15) else 5 for j in range(29)))
 
@@ -85,6 +90,11 @@ _RAGGED = dict(embed=128, trunk_dim=256, n_blocks=2, n_heads=4, n_gears=7, ffn_m
     (_RAGGED, "bf16", "on", "off"),
     (_RAGGED, "bf16", "off", "auto"),
     (dict(embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True), "f32", "off", "auto"),
+    # value-residual mix + SimBaV2 trunk: always the per-op route
+    (_VRES_V2, "f16", "on", "off"),
+    (_VRES_V2, "f16", "off", "off"),
+    (_VRES_V2, "bf16", "off", "off"),
+    (_VRES_V2, "f32", "off", "off"),
 ])
 def test_production_shapes_against_the_oracle(kw, dtype, ffn, blocks):
     m, sd = _big(5, **kw)
@@ -119,6 +129,30 @@ def test_production_shapes_against_the_oracle(kw, dtype, ffn, blocks):
         top = ref_lg.topk(2, -1).values
         decided = (top[..., 0] - top[..., 1]) > 1e-2
         assert bool(((lg.argmax(-1) == ref_lg.argmax(-1)) | ~decided).all())
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_value_residual_at_init_is_bitwise_the_plain_policy(dtype):
+    """(a, b) = (1, 0): the mix returns v exactly (python/tests/test_arch_ab_options.py:131-139)."""
+    kw = dict(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True)
+    torch.manual_seed(3)
+    base = NotePolicy(**kw)
+    p = NotePolicy(value_residual=True, **kw)
+    missing = p.load_state_dict(base.state_dict(), strict=False)
+    assert sorted(missing.missing_keys) == ["blocks.1.vres_a", "blocks.1.vres_b", "blocks.2.vres_a", "blocks.2.vres_b"]
+    base, p = base.to(DEV), p.to(DEV)
+    base.fp16 = p.fp16 = dtype == "f16"
+    base.fused_blocks = "off"
+    assert not p.fused_blocks_ok(torch.float16)
+    od = _make_obs(33, 4).to(DEV)
+    lb, vb = base.forward_stacked(od)
+    lp, vp = p.forward_stacked(od)
+    assert torch.equal(lb, lp) and torch.equal(vb, vp)
+    with torch.no_grad():
+        for blk in p.blocks[1:]:
+            blk.vres_b.fill_(0.5)
+    lq, _ = p.forward_stacked(od)
+    assert not torch.equal(lq, lp)                              # and with b != 0 block 0's values do get through
 
 
 @pytest.mark.parametrize("blocks", ["auto", "off"])

@@ -329,3 +329,64 @@ def test_cfg_embed(dtype, T, d):
     assert tok.shape == (B, T, d)
     tol = 1e-5 if dtype is torch.float32 else 1.2 * EPS16[dtype] * (ref.abs().max().item() + 1)
     assert (tok.float().cpu() - ref).abs().max().item() <= tol
+
+
+# ---------------------------------------------------------------- value-residual mix
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("B,T,d,packed", [(3, 29, 192, True), (17, 29, 128, True), (5, 7, 20, False), (1, 1, 3, False)])
+def test_vres_mix(dtype, B, T, d, packed):
+    """torch.addcmul(v * a, v0, b).to(dtype) (python/fp16_linear.py:1002-1006); exact at (a, b) = (1, 0)."""
+    if packed:      # v and v0 as column slices of packed q|k|v buffers, mixed in place
+        qkv = _rand(B, T, 3 * d, dtype=dtype, seed=11)
+        qkv0 = _rand(B, T, 3 * d, dtype=dtype, seed=12)
+        v, v0 = qkv[..., 2 * d:], qkv0[..., 2 * d:]
+    else:
+        v, v0 = _rand(B, T, d, dtype=dtype, seed=11), _rand(B, T, d, dtype=dtype, seed=12)
+    a = torch.tensor([0.83], device=DEV)
+    b = torch.tensor([-0.41], device=DEV)
+    ref = (v.double() * a.double() + v0.double() * b.double())
+    keep = v.clone()
+    one, zero = torch.ones(1, device=DEV), torch.zeros(1, device=DEV)
+    same = ops.vres_mix(v, v0, one, zero, out=torch.empty_like(keep))
+    assert torch.equal(same, keep)
+    out = ops.vres_mix(v, v0, a, b)                      # in place
+    assert out.data_ptr() == v.data_ptr()
+    if packed:                                           # the q | k columns of the buffer are untouched
+        assert torch.equal(qkv[..., :2 * d], _rand(B, T, 3 * d, dtype=dtype, seed=11)[..., :2 * d])
+    if dtype is torch.float32:
+        assert torch.allclose(out.double(), ref, rtol=1e-6, atol=1e-6)
+    else:
+        assert (out.double() - ref).abs().max().item() <= EPS16[dtype] * (ref.abs().max().item() + 1e-3)
+        assert (out.double() - ref.to(dtype).double()).abs().max().item() <= 2 * EPS16[dtype] * ref.abs().max().item()
+
+
+# ---------------------------------------------------------------- SimBaV2 row stages
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,D", [(1, 96), (7, 384), (1001, 256), (5, 50)])
+def test_hsphere_stages(dtype, rows, D):
+    """The three fp32 row stages against F.normalize (library routine) in fp64
+    (python/policy.py:1140-1155); the output rows have RMS 1 (python/tests/test_arch_ab_options.py:250-254)."""
+    t = _rand(rows, D, dtype=dtype, seed=21, scale=30.0)
+    s = _rand(D, seed=22) * 0.05 + 0.14
+    x32, x = ops.hsphere(ops.HS_SCALE_L2N, t, s, 1.5)
+    ref_x = F.normalize(t.double() * (s.double() * 1.5), dim=-1, eps=1e-6)
+    assert x32.dtype is torch.float32 and x.dtype is dtype
+    assert torch.allclose(x32.double(), ref_x, rtol=1e-5, atol=1e-6)
+    assert torch.equal(x, x32.to(dtype))
+    u = ops.hsphere(ops.HS_SCALE_RELU, t, s, 0.5)
+    ref_u = F.relu(t.double() * (s.double() * 0.5))
+    tol = 1e-6 if dtype is torch.float32 else EPS16[dtype]
+    assert (u.double() - ref_u).abs().max().item() <= tol * (ref_u.abs().max().item() + 1)
+    alpha = _rand(D, seed=23) * 0.3 + 0.5
+    y_in = _rand(rows, D, dtype=dtype, seed=24, scale=3.0)
+    h = ops.hsphere(ops.HS_L2N_LERP, y_in, alpha, 0.9, x32=x32)
+    y = F.normalize(y_in.double(), dim=-1, eps=1e-6)
+    z = F.normalize(x32.double() + alpha.double() * 0.9 * (y - x32.double()), dim=-1, eps=1e-6)
+    ref_h = z * math.sqrt(D)
+    assert (h.double() - ref_h).abs().max().item() <= (1e-5 if dtype is torch.float32 else 2 * EPS16[dtype]) * ref_h.abs().max().item()
+    rms = h.double().square().mean(-1)
+    assert torch.allclose(rms, torch.ones_like(rms), atol=1e-5 if dtype is torch.float32 else 4 * EPS16[dtype])
+    # a zero row normalises to zero (eps clamp), not NaN
+    z0 = torch.zeros(2, D, dtype=dtype, device=DEV)
+    x32z, _ = ops.hsphere(ops.HS_SCALE_L2N, z0, s, 1.0)
+    assert torch.equal(x32z, torch.zeros_like(x32z))

@@ -15,7 +15,7 @@ GOLD = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "notep
 
 
 def test_fixtures_exist():
-    assert len(GOLD) == 3
+    assert len(GOLD) == 4
 
 
 @pytest.mark.parametrize("path", GOLD, ids=[os.path.basename(p)[:-4] for p in GOLD])
@@ -136,3 +136,22 @@ def test_emulated_fp16_stream_is_in_the_reference_tolerance_class():
     lg, v = nr.forward(sd, arch, obs, emulate="f16")
     live = logits > -1e8
     assert (lg[live] - logits[live]).abs().max().item() < 2e-2 * logits[live].abs().max().item()
+
+
+def test_value_residual_and_simbav2_properties_of_the_oracle():
+    """What the reference's own tests hold for the two options (python/tests/test_arch_ab_options.py:
+    131-139, 250-256): the mix at (a, b) = (1, 0) is bitwise the plain policy; a SimBaV2 feature row
+    is sqrt(D) times a unit vector."""
+    path = [p for p in GOLD if p.endswith("notepolicy_vres_v2.npz")][0]
+    arch, sd, obs, _, _ = nr.load_fixture(path)
+    sd1 = {k: (torch.ones(1) if k.endswith("vres_a") else torch.zeros(1) if k.endswith("vres_b") else v)
+           for k, v in sd.items()}
+    plain = {k: v for k, v in sd1.items() if "vres" not in k}
+    lg1, v1 = nr.forward(sd1, arch, obs)
+    lg0, v0 = nr.forward(plain, {**arch, "value_residual": False}, obs)
+    assert torch.equal(lg1, lg0) and torch.equal(v1, v0)
+    lg, _ = nr.forward(sd, arch, obs)
+    assert not torch.equal(lg, lg0)                         # the fixture's (a, b) do move the output
+    _, _, parts = nr.forward(sd, arch, obs, return_parts=True)
+    rms = parts["h"].square().mean(-1)
+    assert torch.allclose(rms, torch.ones_like(rms), atol=1e-5)
