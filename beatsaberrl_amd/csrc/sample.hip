@@ -9,7 +9,11 @@
 // result is a pure function of the inputs) or from a counter-based Philox4x32-10 stream keyed by
 // (seed, offset) inside the kernel; a different stream than the caller's generator is the
 // same accepted class of difference the reference documents for its own sampler change
-// (python/policy.py:1476-1483).
+// (python/policy.py:1476-1483).  The offset may live on the device (`offset_dev`, added to the
+// host offset): a launch captured in a graph then draws fresh noise on every replay, provided
+// something on the stream advances the counter between launches - bsrl_counter_add is that
+// one-thread kernel (the role torch's graph-registered generator offset plays for the
+// reference's captured rollout, python/rollout_graph.py:43-78).
 //
 // One thread per (env, head); a workgroup owns EPB envs and reduces the 29 per-head terms of
 // each env in head order (a fixed order: results do not depend on the launch shape).
@@ -23,7 +27,7 @@ constexpr int KMAX = 8;
 struct SampleArgs {
     const float* logits; int64_t B; int n_heads, K;
     const int32_t* head_sizes; const float* exp_noise;
-    uint64_t seed, offset;
+    uint64_t seed, offset; const uint64_t* offset_dev;
     const void* action_in; int action_in_u8;
     int64_t* action_out; float* logprob; float* entropy; float* ent_h; float* noise_out;
 };
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(256) void sample_heads_kernel(SampleArgs a) {
                 // counter = (row, 2 * offset + block): 8 draws per row from two 128-bit blocks
 #pragma unroll
                 for (int blk = 0; blk < 2; ++blk) {
-                    const uint64_t hi = a.offset * 2u + (uint64_t)blk;
+                    const uint64_t hi = (a.offset + (a.offset_dev ? *a.offset_dev : 0)) * 2u + (uint64_t)blk;
                     uint32_t c[4] = {(uint32_t)row, (uint32_t)((uint64_t)row >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
                     philox4x32_10(c, (uint32_t)a.seed, (uint32_t)(a.seed >> 32));
 #pragma unroll
@@ -115,11 +119,20 @@ __global__ __launch_bounds__(256) void sample_heads_kernel(SampleArgs a) {
     }
 }
 
+__global__ void counter_add_kernel(uint64_t* ctr, uint64_t inc) { *ctr += inc; }
+
 }  // namespace
+
+extern "C" int bsrl_counter_add(uint64_t* counter, uint64_t inc, bsrl_stream stream) {
+    if (!counter) BSRL_FAIL(BSRL_EINVAL, "bsrl_counter_add: null counter");
+    hipLaunchKernelGGL(counter_add_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), counter, inc);
+    BSRL_CHECK_LAUNCH("bsrl_counter_add");
+    return BSRL_OK;
+}
 
 extern "C" int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads, int64_t K,
                                  const int32_t* head_sizes, const float* exp_noise,
-                                 uint64_t seed, uint64_t offset,
+                                 uint64_t seed, uint64_t offset, const uint64_t* offset_dev,
                                  const void* action_in, int action_in_u8,
                                  int64_t* action_out, float* logprob, float* entropy, float* ent_h,
                                  float* noise_out, bsrl_stream stream) {
@@ -128,7 +141,7 @@ extern "C" int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads
         BSRL_FAIL(BSRL_EINVAL, "bsrl_sample_heads: need B >= 0, 1 <= n_heads <= 32, 1 <= K <= %d", KMAX);
     if (!action_in && !action_out) BSRL_FAIL(BSRL_EINVAL, "bsrl_sample_heads: sampling needs action_out");
     if (B == 0) return BSRL_OK;
-    SampleArgs a{logits, B, (int)n_heads, (int)K, head_sizes, exp_noise, seed, offset, action_in, action_in_u8,
+    SampleArgs a{logits, B, (int)n_heads, (int)K, head_sizes, exp_noise, seed, offset, offset_dev, action_in, action_in_u8,
                  action_out, logprob, entropy, ent_h, noise_out};
     const dim3 grid((unsigned)((B + EPB - 1) / EPB)), block(256);
     hipLaunchKernelGGL(sample_heads_kernel, grid, block, 0, static_cast<hipStream_t>(stream), a);

@@ -274,10 +274,12 @@ def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z
 
 
 def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, action=None,
-                 need_entropy=True, want_ent_h=False, want_noise=False):
+                 need_entropy=True, want_ent_h=False, want_noise=False, counter=None):
     """Action epilogue on fp32 logits (B, n_heads, K).  action=None samples (Gumbel-max with the
     caller's Exp(1) draws `exp_noise`, or the kernel's Philox stream keyed by (seed, offset));
-    otherwise evaluates the given (B, n_heads) int64 / uint8 actions.
+    otherwise evaluates the given (B, n_heads) int64 / uint8 actions.  counter: a one-element
+    int64 device tensor whose value is added to `offset` on the device and advanced by one after
+    a sampling launch (a captured launch then draws fresh noise on every replay).
     Returns (action int64, logprob, entropy | None, ent_h | None, noise | None)."""
     _need_cuda(logits, head_sizes, exp_noise, action)
     if logits.dtype is not torch.float32 or logits.dim() != 3 or not logits.is_contiguous():
@@ -294,6 +296,8 @@ def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, acti
         if action.shape != (B, NH) or action.dtype not in (torch.int64, torch.uint8) or not action.is_contiguous():
             raise TypeError("sample_heads: action must be a contiguous (B, n_heads) int64 or uint8 tensor")
         u8 = int(action.dtype is torch.uint8)
+    if counter is not None and (counter.dtype is not torch.int64 or counter.numel() != 1 or not counter.is_cuda):
+        raise TypeError("sample_heads: counter must be a one-element int64 device tensor")
     dev = logits.device
     act_out = torch.empty(B, NH, device=dev, dtype=torch.int64)
     logprob = torch.empty(B, device=dev, dtype=torch.float32)
@@ -302,9 +306,12 @@ def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, acti
     noise = torch.empty_like(logits) if (want_noise and action is None) else None
     with torch.cuda.device(dev):
         rc = _lib.load().bsrl_sample_heads(logits.data_ptr(), B, NH, K, _ptr(head_sizes), _ptr(exp_noise),
-                                           int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1), _ptr(action), u8,
-                                           act_out.data_ptr(), logprob.data_ptr(), _ptr(entropy), _ptr(ent_h),
-                                           _ptr(noise), _stream(logits))
+                                           int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1), _ptr(counter),
+                                           _ptr(action), u8, act_out.data_ptr(), logprob.data_ptr(), _ptr(entropy),
+                                           _ptr(ent_h), _ptr(noise), _stream(logits))
+        _lib.check(rc, "bsrl_sample_heads")
+        if counter is not None and action is None and exp_noise is None:
+            rc = _lib.load().bsrl_counter_add(counter.data_ptr(), 1, _stream(logits))
     _lib.check(rc, "bsrl_sample_heads")
     return act_out, logprob, entropy, ent_h, noise
 

@@ -302,7 +302,9 @@ class NotePolicy(nn.Module):
         # shape has one (ops.blocks_pack_size > 0); "off": always the per-op launch train
         self.fused_blocks = "auto"
         self._blocks_image = None               # [weights version, dtype, uint8 image]
-        self._sample_calls = 0
+        # sampling-call counter of the in-kernel Philox stream; on the device so that a captured
+        # get_action_and_value draws fresh noise on every replay
+        self.register_buffer("_sample_ctr", torch.zeros(1, dtype=torch.int64), persistent=False)
         self.fp16 = False                       # True: 16-bit stream (python/policy.py:1085-1090)
         self.stream_dtype = torch.float16       # the 16-bit type used when fp16 is on
         self.fp16_accum = fp16_accum
@@ -353,16 +355,17 @@ class NotePolicy(nn.Module):
         return c[2]
 
     def refresh_fp16_caches(self):
-        """Force every 16-bit replica up to date for the current weights version
-        (python/policy.py:1448-1461): call after optimizer steps under a captured graph."""
-        if not self.fp16:
-            return
-        dt = self.stream_dtype
+        """Force every weight copy the kernels read up to date for the current weights version
+        (python/policy.py:1448-1461): call after optimizer steps under a captured graph.  On the
+        16-bit stream these are the replicas and the fused block image; on the fp32 stream only
+        the concatenated q|k|v / k|v / head matrices (single Linears read the masters)."""
+        dt = self.stream_dtype if self.fp16 else torch.float32
         if self.fused_blocks_ok(dt):
             self.blocks_image(dt)
-        for m in self.modules():
-            if isinstance(m, nn.Linear):
-                _fl._replica(m.weight, dt)
+        if dt is not torch.float32:
+            for m in self.modules():
+                if isinstance(m, nn.Linear):
+                    _fl._replica(m.weight, dt)
         for blk in self.blocks:
             _fl.packed_halves([blk.q_proj, blk.k_proj, blk.v_proj], dt)
             _fl.packed_halves([blk.k_proj, blk.v_proj], dt)
@@ -503,9 +506,9 @@ class NotePolicy(nn.Module):
         """log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) in one kernel on
         the forward's fp32 logits (reference python/policy.py:1467-1516).  `self.sampler`:
         "kernel" draws inside the kernel (Philox keyed by torch's seed and a per-module call
-        counter); "torch" feeds the kernel Exp(1) draws from torch's default generator, the
-        stream the reference rides (use it under graph capture: a captured launch would replay
-        the same in-kernel counter)."""
+        counter that lives on the device and is advanced on the stream, so a captured call draws
+        fresh noise on every replay); "torch" feeds the kernel Exp(1) draws from torch's default
+        generator, the stream the reference rides."""
         logits, value = self.forward_stacked(obs)
         logits = logits.contiguous()
         if action is not None and action.dtype not in (torch.int64, torch.uint8):
@@ -517,11 +520,9 @@ class NotePolicy(nn.Module):
             raise ValueError(f"sampler must be 'kernel' or 'torch', got {self.sampler!r}")
         sizes = self._head_sizes32 if self._gear_valid is not None else None
         act, logprob, entropy, ent_h, _ = ops.sample_heads(
-            logits, head_sizes=sizes, exp_noise=noise, seed=torch.initial_seed(), offset=self._sample_calls,
+            logits, head_sizes=sizes, exp_noise=noise, seed=torch.initial_seed(), counter=self._sample_ctr,
             action=None if action is None else action.contiguous(), need_entropy=need_entropy,
             want_ent_h=need_entropy)
-        if action is None:
-            self._sample_calls += 1
         if need_entropy:
             self._ent_h = ent_h
         return act, logprob, entropy, value

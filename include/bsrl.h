@@ -211,17 +211,23 @@ int bsrl_note_frontend(const void* obs, int64_t obs_ld, int obs_dtype,
  * exp_noise, or, when it is NULL, from Philox4x32-10 with key = seed and
  * counter = (row, 2 * offset + block) inside the kernel (row = env * n_heads +
  * head; draw k of a row is word k & 3 of block k >> 2, mapped to
- * E = -log(((word >> 8) + 1) * 2^-24)); noise_out, if not NULL, receives the E
- * used.  Evaluation (action_in != NULL, int64 or uint8 when action_in_u8):
+ * E = -log(((word >> 8) + 1) * 2^-24)); offset_dev, if not NULL, points to a
+ * device uint64 added to `offset` when the kernel runs, so a launch captured in
+ * a graph draws fresh noise on each replay once bsrl_counter_add follows it on
+ * the stream (the part torch's graph-registered generator offset plays in the
+ * reference's captured rollout, python/rollout_graph.py:43-78).  noise_out, if
+ * not NULL, receives the E used.  Evaluation (action_in != NULL, int64 or uint8 when action_in_u8):
  * no sampling; action_out may be NULL.
  * Outputs: action_out (B, n_heads) int64; logprob (B); entropy (B) or NULL;
  * ent_h (B, n_heads) or NULL. */
 int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads, int64_t K,
                       const int32_t* head_sizes, const float* exp_noise,
-                      uint64_t seed, uint64_t offset,
+                      uint64_t seed, uint64_t offset, const uint64_t* offset_dev,
                       const void* action_in, int action_in_u8,
                       int64_t* action_out, float* logprob, float* entropy, float* ent_h,
                       float* noise_out, bsrl_stream stream);
+/* *counter += inc, one thread, on `stream` (ordered after the launches before it). */
+int bsrl_counter_add(uint64_t* counter, uint64_t inc, bsrl_stream stream);
 
 /* ---- Transformer block stack in one persistent kernel ------------------------
  * Replaces the block loop of NotePolicy._forward_stacked (python/policy.py:

@@ -61,10 +61,19 @@ def test_new_entry_points_reject_bad_arguments_without_a_device(lib):
     ok = list(args); ok[13] = 0
     assert lib.bsrl_note_frontend(*ok) == 0                     # B == 0: nothing to do
     # action epilogue: K and head-count limits, sampling without an output
-    assert lib.bsrl_sample_heads(16, 4, 29, 9, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == -1
-    assert lib.bsrl_sample_heads(16, 4, 33, 7, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == -1
-    assert lib.bsrl_sample_heads(16, 4, 29, 7, None, None, 0, 0, None, 0, None, 16, None, None, None, None) == -1
-    assert lib.bsrl_sample_heads(16, 0, 29, 7, None, None, 0, 0, None, 0, 16, 16, None, None, None, None) == 0
+    assert lib.bsrl_sample_heads(16, 4, 29, 9, None, None, 0, 0, None, None, 0, 16, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 4, 33, 7, None, None, 0, 0, None, None, 0, 16, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 4, 29, 7, None, None, 0, 0, None, None, 0, None, 16, None, None, None, None) == -1
+    assert lib.bsrl_sample_heads(16, 0, 29, 7, None, None, 0, 0, None, None, 0, 16, 16, None, None, None, None) == 0
+    assert lib.bsrl_counter_add(None, 1, None) == -1
+    # value-residual mix and SimBaV2 row stages: null pointers, pitches below the row width, unknown op
+    assert lib.bsrl_vres_mix(16, 8, 16, 8, None, 16, 16, 8, 4, 8, _lib.F16, None) == -1
+    assert lib.bsrl_vres_mix(16, 4, 16, 8, 16, 16, 16, 8, 4, 8, _lib.F16, None) == -1 and b"pitches" in lib.bsrl_last_error()
+    assert lib.bsrl_vres_mix(16, 8, 16, 8, 16, 16, 16, 8, 0, 8, _lib.F16, None) == 0
+    assert lib.bsrl_hsphere(7, 16, 16, 1.0, None, 16, 16, 4, 8, _lib.F32, None) == -1 and b"unknown op" in lib.bsrl_last_error()
+    assert lib.bsrl_hsphere(0, 16, 16, 1.0, None, None, 16, 4, 8, _lib.F32, None) == -1
+    assert lib.bsrl_hsphere(2, 16, 16, 1.0, None, None, 16, 4, 8, _lib.F32, None) == -1
+    assert lib.bsrl_hsphere(1, 16, 16, 1.0, None, None, 16, 0, 8, _lib.F32, None) == 0
     # grouped linear: the group must divide the rows, fit its stride and exclude a split output
     g = lambda rows, grp, gs, y2=None, split=0: lib.bsrl_linear_grouped(
         16, 8, 16, None, None, 0, 16, 8, y2, 8 if y2 else 0, split, rows, 8, 8, 0, _lib.F16, _lib.F16, grp, gs, None)

@@ -141,6 +141,14 @@ def test_sampling_kernel_stream_matches_the_documented_philox_mapping():
     act3, _, _, _, _ = ops.sample_heads(lg.to(DEV), head_sizes=hs, seed=0x1234567890ABCDEF, offset=4)
     act4, _, _, _, _ = ops.sample_heads(lg.to(DEV), head_sizes=hs, seed=0x1234567890ABCDEE, offset=3)
     assert not torch.equal(act, act3) and not torch.equal(act, act4)
+    # a device-side counter adds to the offset and is advanced by one per sampling launch
+    ctr = torch.tensor([2], dtype=torch.int64, device=DEV)
+    act5, lp5, _, _, _ = ops.sample_heads(lg.to(DEV), head_sizes=hs, seed=0x1234567890ABCDEF, offset=1, counter=ctr)
+    assert torch.equal(act5, act) and torch.equal(lp5, lp) and ctr.item() == 3
+    act6, _, _, _, _ = ops.sample_heads(lg.to(DEV), head_sizes=hs, seed=0x1234567890ABCDEF, offset=1, counter=ctr)
+    assert torch.equal(act6, act3) and ctr.item() == 4
+    ops.sample_heads(lg.to(DEV), head_sizes=hs, action=act, counter=ctr)      # evaluation draws nothing
+    assert ctr.item() == 4
 
 
 def test_sampling_kernel_stream_follows_the_softmax_distribution():
