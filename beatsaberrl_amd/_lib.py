@@ -68,6 +68,10 @@ SIGNATURES = {
     "bsrl_counter_add": (_i32, [_p, C.c_uint64, _p]),
     "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _p, _i32,
                                  _p, _p, _p, _p, _p, _p]),
+    "bsrl_ln_bwd_workspace_size": (_i64, [_i64]),
+    "bsrl_ln_bwd": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),
+    "bsrl_wgrad_workspace_size": (_i64, [_i64, _i64]),
+    "bsrl_wgrad": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_vres_mix": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_hsphere": (_i32, [_i32, _p, _p, C.c_float, _p, _p, _p, _i64, _i64, _i32, _p]),
 }

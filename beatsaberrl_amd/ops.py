@@ -95,6 +95,74 @@ def ln_fwd_add(a, b, weight, bias, eps=1e-5, b_bias=None, want_stats=False):
     return (x, y, mean, rstd) if want_stats else (x, y)
 
 
+def ln_bwd(x, dy, weight, mean, rstd, gx=None, want_dbb=False):
+    """LayerNorm backward (reference layer_norm_cuda.ln_bwd, layer_norm.cu:645-729):
+    returns [dx, dw, db] (+ [dbb] with want_dbb: column sums of the stored dx).  gx, if given,
+    is added into dx before its one rounding (the residual-path gradient of ln_fwd_add)."""
+    _need_cuda(x, dy, weight, mean, rstd, gx)
+    if not (x.is_contiguous() and dy.is_contiguous()) or dy.shape != x.shape or dy.dtype is not x.dtype:
+        raise TypeError("ln_bwd: x and dy must be contiguous with one shape and dtype")
+    if gx is not None and (not gx.is_contiguous() or gx.shape != x.shape or gx.dtype is not x.dtype):
+        raise TypeError("ln_bwd: gx must be contiguous with x's shape and dtype")
+    d = x.shape[-1]
+    rows = x.numel() // d if d else 0
+    weight, mean, rstd = _f32c(weight, "ln weight"), _f32c(mean, "ln mean"), _f32c(rstd, "ln rstd")
+    if weight.numel() != d or mean.numel() != rows or rstd.numel() != rows:
+        raise TypeError("ln_bwd: weight must be (d), mean / rstd (rows)")
+    dev = x.device
+    dx = torch.empty_like(x)
+    dw = torch.empty(d, device=dev, dtype=torch.float32)
+    db = torch.empty(d, device=dev, dtype=torch.float32)
+    dbb = torch.empty(d, device=dev, dtype=torch.float32) if want_dbb else None
+    lib = _lib.load()
+    ws = _workspace(dev, _stream(x), lib.bsrl_ln_bwd_workspace_size(d))
+    with torch.cuda.device(dev):
+        rc = lib.bsrl_ln_bwd(x.data_ptr(), dy.data_ptr(), weight.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                             _ptr(gx), dx.data_ptr(), dw.data_ptr(), db.data_ptr(), _ptr(dbb), ws.data_ptr(),
+                             rows, d, dt_code(x.dtype), _stream(x))
+    if not _lib.check(rc, "bsrl_ln_bwd"):
+        raise Unsupported(f"ln_bwd: no kernel for d={d} {x.dtype}")
+    return [dx, dw, db] + ([dbb] if want_dbb else [])
+
+
+_WS = {}
+
+
+def _workspace(dev, stream, nbytes):
+    """One scratch buffer per (device, stream), grown on demand: calls on one stream are ordered,
+    so they may share it (the C entry points never allocate)."""
+    key = (dev, stream)
+    ws = _WS.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = _WS[key] = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    return ws
+
+
+def wgrad(dy, x, want_db=True):
+    """(dW (M, K) fp32, db (M) fp32 | None) of a Linear from dy (rows, M) and its input x (rows, K),
+    16-bit operands with fp32 accumulation (reference fp16_gemm.wgrad / wgrad_bgrad,
+    fp16_gemm.cu:189-277, 404-476)."""
+    _need_cuda(dy, x)
+    if dy.dim() != 2 or x.dim() != 2 or dy.shape[0] != x.shape[0] or dy.dtype is not x.dtype:
+        raise TypeError("wgrad: dy (rows, M) and x (rows, K) must share rows and dtype")
+    if dy.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("wgrad: 16-bit operands only (the fp32 stream uses the vendor GEMM)")
+    if dy.stride(1) != 1 or x.stride(1) != 1:
+        raise TypeError("wgrad: unit-stride rows needed")
+    rows, M = dy.shape
+    K = x.shape[1]
+    dev = dy.device
+    dw = torch.empty(M, K, device=dev, dtype=torch.float32)
+    db = torch.empty(M, device=dev, dtype=torch.float32) if want_db else None
+    lib = _lib.load()
+    ws = _workspace(dev, _stream(dy), lib.bsrl_wgrad_workspace_size(M, K))
+    with torch.cuda.device(dev):
+        rc = lib.bsrl_wgrad(dy.data_ptr(), dy.stride(0) if rows > 1 else M, x.data_ptr(), x.stride(0) if rows > 1 else K,
+                            dw.data_ptr(), _ptr(db), ws.data_ptr(), rows, M, K, dt_code(dy.dtype), _stream(dy))
+    _lib.check(rc, "bsrl_wgrad")
+    return dw, db
+
+
 def _rows2d(t):
     """View t (..., K) as rows with one row stride; returns (tensor, rows, ld)."""
     K = t.shape[-1]

@@ -259,6 +259,42 @@ int bsrl_blocks_forward(const bsrl_blocks_desc* desc, const void* packed,
                         const void* x_in, const void* key_bias,
                         void* x_res, void* x_out, int64_t B, bsrl_stream stream);
 
+/* ---- LayerNorm backward --------------------------------------------------------
+ * Replaces layer_norm_cuda.ln_bwd(x, dy, w, mean, rstd, gx=None, want_dbb=False)
+ * (python/beat_arena_env/csrc/layer_norm.cu:645-729), the backward of both
+ * _LnFn and _LnAddFn (python/fused_ln.py:56-112).  x, dy, gx (NULL = none),
+ * dx: (rows, d) contiguous in `dtype`; weight (d), mean / rstd (rows) fp32 (the
+ * forward's statistics).  With g = dy * w, xhat = (x - mean) * rstd:
+ *   dx = (g - mean_d(g) - xhat * mean_d(g * xhat)) * rstd + gx   (one rounding)
+ *   dw = sum_rows dy * xhat, db = sum_rows dy                      (fp32, (d))
+ *   dbb (NULL = skip) = sum_rows of the stored dx: the folded-bias gradient of
+ *   ln_fwd_add's b_bias (python/fused_ln.py:96-106)
+ * Column sums are reproducible run to run (fixed-order partials, no atomics).
+ * workspace: caller-owned scratch of bsrl_ln_bwd_workspace_size(d) bytes, 16-byte
+ * aligned, overwritten by each call.  Same shape limits as the forward up to
+ * d = 1024 (fp32) / 2048 (16-bit); returns BSRL_UNSUPPORTED beyond. */
+int64_t bsrl_ln_bwd_workspace_size(int64_t d);
+int bsrl_ln_bwd(const void* x, const void* dy, const float* weight,
+                const float* mean, const float* rstd, const void* gx,
+                void* dx, float* dw, float* db, float* dbb, void* workspace,
+                int64_t rows, int64_t d, int dtype, bsrl_stream stream);
+
+/* ---- Linear weight / bias gradient -----------------------------------------------
+ * Replaces fp16_gemm.wgrad(dy, x) -> dW and wgrad_bgrad(dy, x) -> [dW, db]
+ * (python/beat_arena_env/csrc/fp16_gemm.cu:189-277, 404-476; callers
+ * python/fp16_linear.py:442-458):
+ *   dW[m, k] = sum_r dy[r, m] * x[r, k]   (fp32, (M, K) contiguous)
+ *   db[m]    = sum_r dy[r, m]              (fp32 (M), NULL = skip)
+ * dy (rows, M) row pitch lddy, x (rows, K) row pitch ldx, both F16 or BF16 (the
+ * fp32 stream uses the vendor GEMM, as the reference does); fp32 accumulation
+ * on MFMA, reproducible run to run (row splits folded in a fixed order).
+ * workspace: caller-owned scratch of bsrl_wgrad_workspace_size(M, K) bytes,
+ * overwritten by each call. */
+int64_t bsrl_wgrad_workspace_size(int64_t M, int64_t K);
+int bsrl_wgrad(const void* dy, int64_t lddy, const void* x, int64_t ldx,
+               float* dw, float* db, void* workspace,
+               int64_t rows, int64_t M, int64_t K, int dtype, bsrl_stream stream);
+
 /* ---- Value-residual mix -------------------------------------------------------
  * out = a * v + b * v0: what every block after the first does to its attention
  * values under the reference's value_residual option (fp16_linear.vres_mix,

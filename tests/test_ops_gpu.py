@@ -390,3 +390,80 @@ def test_hsphere_stages(dtype, rows, D):
     z0 = torch.zeros(2, D, dtype=dtype, device=DEV)
     x32z, _ = ops.hsphere(ops.HS_SCALE_L2N, z0, s, 1.0)
     assert torch.equal(x32z, torch.zeros_like(x32z))
+
+
+# ---------------------------------------------------------------- LayerNorm backward
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,d", [(1, 128), (7, 64), (1000, 128), (257, 192), (4099, 192), (64, 256), (33, 384),
+                                    (5, 512), (3, 1024), (9, 40), (70000, 128)])
+@pytest.mark.parametrize("with_gx", [False, True])
+def test_ln_bwd(dtype, rows, d, with_gx):
+    """Against torch autograd through F.layer_norm in fp64 on the same operands (the reference's idiom,
+    python/tests/test_fused_ln.py:91-135): dx to the type's rounding, dw / db / dbb to fp32 summation error."""
+    x = _rand(rows, d, dtype=dtype, seed=rows + d, scale=2.0) + 0.5
+    dy = _rand(rows, d, dtype=dtype, seed=rows + d + 1)
+    gx = _rand(rows, d, dtype=dtype, seed=rows + d + 2) if with_gx else None
+    w = _rand(d, seed=1) * 0.3 + 1.0
+    b = _rand(d, seed=2) * 0.3
+    _, mean, rstd = ops.ln_fwd(x, w, b, 1e-5, want_stats=True)
+    dx, dw, db, dbb = ops.ln_bwd(x, dy, w, mean, rstd, gx=gx, want_dbb=True)
+    assert dx.dtype is dtype and dw.dtype is torch.float32 and dw.shape == (d,)
+    xd = x.double().requires_grad_(True)
+    wd = w.double().requires_grad_(True)
+    bd = b.double().requires_grad_(True)
+    F.layer_norm(xd, (d,), wd, bd, 1e-5).backward(dy.double())
+    ref_dx = xd.grad + (gx.double() if with_gx else 0.0)
+    tol = 2e-5 if dtype is torch.float32 else 1.5 * EPS16[dtype]
+    assert (dx.double() - ref_dx).abs().max().item() <= tol * (ref_dx.abs().max().item() + 1.0)
+    # column sums: fp32 accumulation over `rows` terms of O(1) magnitude
+    tol_c = 3e-6 * max(rows, 64) ** 0.5 * 4
+    scale_w = (dy.double().abs() * ((x.double() - mean.double()[:, None]) * rstd.double()[:, None]).abs()).sum(0).max().item()
+    assert (dw.double() - wd.grad).abs().max().item() <= tol_c * max(scale_w, 1.0) / max(rows, 64) ** 0.5
+    assert (db.double() - bd.grad).abs().max().item() <= tol_c * max(dy.double().abs().sum(0).max().item(), 1.0) / max(rows, 64) ** 0.5
+    assert (dbb.double() - dx.double().sum(0)).abs().max().item() <= tol_c * max(dx.double().abs().sum(0).max().item(), 1.0) / max(rows, 64) ** 0.5
+    # reproducible: no atomics anywhere in the column sums
+    dx2, dw2, db2 = ops.ln_bwd(x, dy, w, mean, rstd, gx=gx)
+    assert torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.equal(db, db2)
+
+
+def test_ln_bwd_no_rows_and_unsupported_width():
+    w = torch.ones(128, device=DEV)
+    e = torch.empty(0, 128, device=DEV)
+    s = torch.empty(0, device=DEV)
+    dx, dw, db = ops.ln_bwd(e, e, w, s, s)
+    assert dx.shape == (0, 128) and torch.equal(dw, torch.zeros_like(dw)) and torch.equal(db, torch.zeros_like(db))
+    x = torch.zeros(2, 4096, device=DEV, dtype=torch.float16)
+    with pytest.raises(ops.Unsupported):
+        ops.ln_bwd(x, x, torch.ones(4096, device=DEV), torch.zeros(2, device=DEV), torch.ones(2, device=DEV))
+
+
+# ---------------------------------------------------------------- Linear weight / bias gradient
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,M,K", [(1, 8, 8), (31, 128, 128), (32, 192, 192), (1000, 576, 192), (5000, 768, 192),
+                                      (4097, 192, 768), (70001, 192, 192), (300, 145, 384), (77, 101, 40), (9, 7, 5),
+                                      (20000, 384, 256)])
+def test_wgrad(dtype, rows, M, K):
+    """dy^T x and column sums of dy against fp64 on the same rounded operands (fp32-accumulate class:
+    python/tests/test_fp16_accum.py:84-89 uses 2e-3 relative; this is fp32 accumulation of exact products)."""
+    dy = _rand(rows, M, dtype=dtype, seed=rows + M)
+    x = _rand(rows, K, dtype=dtype, seed=rows + K + 1)
+    dw, db = ops.wgrad(dy, x)
+    ref_w = dy.double().t() @ x.double()
+    ref_b = dy.double().sum(0)
+    tol = 2e-6 * max(rows, 16) ** 0.5 + 1e-6
+    assert (dw.double() - ref_w).abs().max().item() <= tol * max((dy.double().abs().t() @ x.double().abs()).max().item(), 1.0)
+    assert (db.double() - ref_b).abs().max().item() <= tol * max(dy.double().abs().sum(0).max().item(), 1.0)
+    dw2, none = ops.wgrad(dy, x, want_db=False)
+    assert none is None and torch.equal(dw, dw2)                  # reproducible, and db is optional
+
+
+def test_wgrad_strided_operands_and_empty_batch():
+    """Operands as column slices of packed buffers (the q|k|v gradient, the k|v input), and rows = 0."""
+    g = _rand(513, 3 * 192, dtype=torch.float16, seed=5)
+    h = _rand(513, 2 * 128, dtype=torch.float16, seed=6)
+    dw, db = ops.wgrad(g[:, 192:384], h[:, 128:])
+    assert torch.allclose(dw.double(), g[:, 192:384].double().t() @ h[:, 128:].double(), rtol=1e-5, atol=1e-4)
+    assert torch.allclose(db.double(), g[:, 192:384].double().sum(0), rtol=1e-5, atol=1e-4)
+    e = torch.empty(0, 64, device=DEV, dtype=torch.float16)
+    dw, db = ops.wgrad(e, e)
+    assert torch.equal(dw, torch.zeros(64, 64, device=DEV)) and torch.equal(db, torch.zeros(64, device=DEV))
