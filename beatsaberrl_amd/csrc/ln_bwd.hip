@@ -44,23 +44,41 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(const void* __restrict__ x,
             if (DBB) abb[c][j] = 0.f;
         }
     }
+    // the next pass's x / dy are in flight (raw registers) while this pass computes
+    typename io::raw nx[NCH], ng[NCH];
+    float nmu = 0.f, nr = 0.f;
+    auto fetch = [&](int64_t rb) {
+        const int64_t row = (rb * 4 + wave) * RPW + rsub;
+        nmu = row < rows ? mean[row] : 0.f;
+        nr = row < rows ? rstd[row] : 0.f;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int e0 = (c * LPR + sub) * VEC;
+            if (row < rows && e0 < d) { nx[c] = io::load_raw(x, row * (int64_t)d + e0); ng[c] = io::load_raw(dy, row * (int64_t)d + e0); }
+        }
+    };
+    if ((int64_t)blockIdx.x * SLOTS < rows) fetch(blockIdx.x);
     for (int64_t rb = blockIdx.x; rb * SLOTS < rows; rb += gridDim.x) {
         const int64_t row = (rb * 4 + wave) * RPW + rsub;
         const bool rv = row < rows;
         const int64_t base = row * (int64_t)d;
-        const float mu = rv ? mean[row] : 0.f, r = rv ? rstd[row] : 0.f;
+        const float mu = nmu, r = nr;
         float xh[NCH][VEC], g[NCH][VEC];
         float s1 = 0.f, s2 = 0.f;
+        typename io::raw cx[NCH], cg[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) { cx[c] = nx[c]; cg[c] = ng[c]; }
+        if ((rb + gridDim.x) * SLOTS < rows) fetch(rb + gridDim.x);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int e0 = (c * LPR + sub) * VEC;
             float xv[VEC], gv[VEC];
 #pragma unroll
             for (int j = 0; j < VEC; ++j) { xv[j] = 0.f; gv[j] = 0.f; }
-            if (rv && e0 < d) { io::load(x, base + e0, xv); io::load(dy, base + e0, gv); }
+            if (rv && e0 < d) { io::cvt(cx[c], xv); io::cvt(cg[c], gv); }
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
-                xh[c][j] = (xv[j] - mu) * r;                 // 0 for rows / columns past the end (r = 0, x = mu = 0)
+                xh[c][j] = (xv[j] - mu) * r;                 // 0 for rows past the end (r = 0, x = mu = 0)
                 g[c][j] = gv[j] * wv[c][j];
                 s1 += g[c][j];
                 s2 += g[c][j] * xh[c][j];
@@ -129,9 +147,25 @@ __global__ __launch_bounds__(256) void ln_bwd_reduce_kernel(const float* __restr
     }
 }
 
+// workgroups that are resident at once on the current device: the persistent grid is one such round, so that no
+// workgroup waits for a slot while others are already in their tail
+template <typename K> int resident_grid(K kernel) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || cus < 1 || per_cu < 1)
+        return LNB_MAX_GRID;
+    const int64_t g = (int64_t)cus * per_cu;
+    return g < LNB_MAX_GRID ? (int)g : LNB_MAX_GRID;
+}
+
 template <typename IO, int LPR, int NCH>
 void launch(const void* x, const void* dy, const float* w, const float* mean, const float* rstd, const void* gx,
-            void* dx, float* part, bool dbb, int64_t rows, int d, int grid, hipStream_t st) {
+            void* dx, float* part, bool dbb, int64_t rows, int d, int* grid_io, hipStream_t st) {
+    // one cap for both forms, so that dw / db do not depend on whether dbb was asked for
+    static const int cap = [] { const int c0 = resident_grid(ln_bwd_kernel<IO, LPR, NCH, false>), c1 = resident_grid(ln_bwd_kernel<IO, LPR, NCH, true>);
+                                return c0 < c1 ? c0 : c1; }();
+    const int grid = *grid_io < cap ? *grid_io : cap;
+    *grid_io = grid;
     if (dbb) hipLaunchKernelGGL((ln_bwd_kernel<IO, LPR, NCH, true>), dim3(grid), dim3(256), 0, st, x, dy, w, mean, rstd, gx, dx, part, rows, d);
     else hipLaunchKernelGGL((ln_bwd_kernel<IO, LPR, NCH, false>), dim3(grid), dim3(256), 0, st, x, dy, w, mean, rstd, gx, dx, part, rows, d);
 }
@@ -159,9 +193,8 @@ int dispatch(const void* x, const void* dy, const float* w, const float* mean, c
     const int rpb = pick<IO>(d, &lpr, &nch);
     if (!rpb) return BSRL_UNSUPPORTED;
     const int64_t want = (rows + rpb - 1) / rpb;
-    const int grid = (int)(want < LNB_MAX_GRID ? want : LNB_MAX_GRID);
-    *grid_out = grid;
-#define LNB_GO(LPR, NCH) if (lpr == LPR && nch == NCH) { launch<IO, LPR, NCH>(x, dy, w, mean, rstd, gx, dx, part, dbb, rows, (int)d, grid, st); return BSRL_OK; }
+    *grid_out = (int)(want < LNB_MAX_GRID ? want : LNB_MAX_GRID);
+#define LNB_GO(LPR, NCH) if (lpr == LPR && nch == NCH) { launch<IO, LPR, NCH>(x, dy, w, mean, rstd, gx, dx, part, dbb, rows, (int)d, grid_out, st); return BSRL_OK; }
     LNB_GO(16, 1) LNB_GO(16, 2) LNB_GO(32, 1) LNB_GO(16, 3) LNB_GO(32, 2) LNB_GO(32, 3) LNB_GO(32, 4) LNB_GO(64, 4)
 #undef LNB_GO
     return BSRL_UNSUPPORTED;

@@ -9,10 +9,12 @@ template <typename IO> struct LnIO;
 template <> struct LnIO<F32IO> {
     static constexpr int VEC = 4;
     typedef float elem;
-    static __device__ __forceinline__ void load(const void* p, int64_t off, float* v) {
-        float4 t = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + off);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    typedef float4 raw;
+    static __device__ __forceinline__ raw load_raw(const void* p, int64_t off) {
+        return *reinterpret_cast<const float4*>(static_cast<const float*>(p) + off);
     }
+    static __device__ __forceinline__ void cvt(raw t, float* v) { v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+    static __device__ __forceinline__ void load(const void* p, int64_t off, float* v) { cvt(load_raw(p, off), v); }
     static __device__ __forceinline__ void store(void* p, int64_t off, const float* v) {
         *reinterpret_cast<float4*>(static_cast<float*>(p) + off) = make_float4(v[0], v[1], v[2], v[3]);
     }
@@ -20,12 +22,16 @@ template <> struct LnIO<F32IO> {
 };
 template <typename DT> struct LnIO16 {
     static constexpr int VEC = 8;
-    static __device__ __forceinline__ void load(const void* p, int64_t off, float* v) {
-        uint4 t = *reinterpret_cast<const uint4*>(static_cast<const u16*>(p) + off);
+    typedef uint4 raw;
+    static __device__ __forceinline__ raw load_raw(const void* p, int64_t off) {
+        return *reinterpret_cast<const uint4*>(static_cast<const u16*>(p) + off);
+    }
+    static __device__ __forceinline__ void cvt(raw t, float* v) {
         uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) { v[2 * i] = DT::to_f((u16)(w[i] & 0xffff)); v[2 * i + 1] = DT::to_f((u16)(w[i] >> 16)); }
     }
+    static __device__ __forceinline__ void load(const void* p, int64_t off, float* v) { cvt(load_raw(p, off), v); }
     static __device__ __forceinline__ void store(void* p, int64_t off, const float* v) {
         uint32_t w[4];
 #pragma unroll
