@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(LinArgs a) {
                 if (c >= a.M) break;
                 float o = a.out_f32 ? apply_act<ACT>(acc[i][j][e] + bv[e]) : apply_act16<ACT>(acc[i][j][e] + bv[e]);
                 if (res) o += DT::to_f(res[row * a.ldr + c]);
+                if (a.gate && !(DT::to_f(static_cast<const u16*>(a.gate)[row * a.ldgate + c]) > 0.f)) o = 0.f;
                 const bool second = a.y2 && c >= a.split;
                 void* dst = second ? a.y2 : a.y;
                 const int64_t off = second ? row * a.ldy2 + (c - a.split) : lin_yoff(a, row) + c;
@@ -147,6 +148,13 @@ __global__ __launch_bounds__(256) void linear_mfma_vec_kernel(LinArgs a) {
                 uint2 rv = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
                 o[0] += DT::to_f((u16)(rv.x & 0xffff)); o[1] += DT::to_f((u16)(rv.x >> 16));
                 o[2] += DT::to_f((u16)(rv.y & 0xffff)); o[3] += DT::to_f((u16)(rv.y >> 16));
+            }
+            if (a.gate) {
+                const uint2 gv = *reinterpret_cast<const uint2*>(static_cast<const u16*>(a.gate) + row * a.ldgate + col);
+                if (!(DT::to_f((u16)(gv.x & 0xffff)) > 0.f)) o[0] = 0.f;
+                if (!(DT::to_f((u16)(gv.x >> 16)) > 0.f)) o[1] = 0.f;
+                if (!(DT::to_f((u16)(gv.y & 0xffff)) > 0.f)) o[2] = 0.f;
+                if (!(DT::to_f((u16)(gv.y >> 16)) > 0.f)) o[3] = 0.f;
             }
             if (a.out_f32) {
                 *reinterpret_cast<float4*>(static_cast<float*>(a.y) + lin_yoff(a, row) + col) = make_float4(o[0], o[1], o[2], o[3]);
@@ -202,6 +210,7 @@ __global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs a) {
             if (c >= a.M) continue;
             float o = apply_act<ACT>(acc[i][j] + (a.bias ? a.bias[c] : 0.f));
             if (res) o += res[row * a.ldr + c];
+            if (a.gate && !(static_cast<const float*>(a.gate)[row * a.ldgate + c] > 0.f)) o = 0.f;
             if (a.y2 && c >= a.split) static_cast<float*>(a.y2)[row * a.ldy2 + (c - a.split)] = o;
             else static_cast<float*>(a.y)[lin_yoff(a, row) + c] = o;
         }
@@ -219,6 +228,30 @@ void launch16(const LinArgs& a, int act, bool fast, bool vec, hipStream_t st) {
     else if (act == BSRL_ACT_GELU) GO(BSRL_ACT_GELU);
     else GO(BSRL_ACT_NONE);
 #undef GO
+}
+
+int lin_dispatch(const LinArgs& a, int act, int dtype, int out_dtype, hipStream_t st, const char* what) {
+    if ((a.rows + 127) / 128 > 65535 * 16) return BSRL_UNSUPPORTED;
+    if (dtype == BSRL_F32) {
+        dim3 grid((unsigned)((a.M + 63) / 64), (unsigned)((a.rows + 63) / 64));
+        if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_RELU>), grid, dim3(256), 0, st, a);
+        else if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_GELU>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_NONE>), grid, dim3(256), 0, st, a);
+    } else {
+        const bool fast = a.K % 8 == 0 && a.ldx % 8 == 0 && bsrl_aligned(a.x, 16) && bsrl_aligned(a.w, 16);
+        const int osz = out_dtype == BSRL_F32 ? 4 : 2;
+        const bool vec = fast && !a.y2 && a.M % 4 == 0 && a.ldy % 4 == 0 && a.y_gstride % 4 == 0 && bsrl_aligned(a.y, 4 * osz) &&
+                         (!a.bias || bsrl_aligned(a.bias, 16)) &&
+                         (!a.res || (a.ldr % 4 == 0 && bsrl_aligned(a.res, 8))) &&
+                         (!a.gate || (a.ldgate % 4 == 0 && bsrl_aligned(a.gate, 8)));
+        if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
+            // large, aligned, 16-bit-out problems: the LDS-tiled kernel
+        } else if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
+        else launch16<BF16>(a, act, fast, vec, st);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) BSRL_FAIL(BSRL_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return BSRL_OK;
 }
 
 }  // namespace
@@ -248,26 +281,20 @@ extern "C" int bsrl_linear_grouped(const void* x, int64_t ldx, const void* w, co
                                                   y_group_stride < y_group_rows * ldy)))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_grouped: groups need rows %% group == 0, group stride >= group * ldy, no split");
     if (rows == 0) return BSRL_OK;
-    if ((rows + 127) / 128 > 65535 * 16) return BSRL_UNSUPPORTED;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     LinArgs a{x, ldx, w, bias, residual, ldr, y, ldy, y2, ldy2, split, rows, (int)K, (int)M, out_dtype == BSRL_F32,
-              (int)y_group_rows, y_group_stride};
-    if (dtype == BSRL_F32) {
-        dim3 grid((unsigned)((M + 63) / 64), (unsigned)((rows + 63) / 64));
-        if (act == BSRL_ACT_RELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_RELU>), grid, dim3(256), 0, st, a);
-        else if (act == BSRL_ACT_GELU) hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_GELU>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((linear_f32_kernel<BSRL_ACT_NONE>), grid, dim3(256), 0, st, a);
-    } else {
-        const bool fast = K % 8 == 0 && ldx % 8 == 0 && bsrl_aligned(x, 16) && bsrl_aligned(w, 16);
-        const int osz = out_dtype == BSRL_F32 ? 4 : 2;
-        const bool vec = fast && !y2 && M % 4 == 0 && ldy % 4 == 0 && y_group_stride % 4 == 0 && bsrl_aligned(y, 4 * osz) &&
-                         (!bias || bsrl_aligned(bias, 16)) &&
-                         (!residual || (ldr % 4 == 0 && bsrl_aligned(residual, 8)));
-        if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
-            // large, aligned, 16-bit-out problems: the LDS-tiled kernel
-        } else if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
-        else launch16<BF16>(a, act, fast, vec, st);
-    }
-    BSRL_CHECK_LAUNCH("bsrl_linear");
-    return BSRL_OK;
+              (int)y_group_rows, y_group_stride, nullptr, 0};
+    return lin_dispatch(a, act, dtype, out_dtype, static_cast<hipStream_t>(stream), "bsrl_linear");
+}
+
+extern "C" int bsrl_linear_gated(const void* x, int64_t ldx, const void* w, const void* gate, int64_t ldgate,
+                                 void* y, int64_t ldy, int64_t rows, int64_t K, int64_t M, int dtype,
+                                 bsrl_stream stream) {
+    if (!x || !w || !y || !gate) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_gated: null pointer");
+    if (rows < 0 || K <= 0 || M <= 0 || K > (1 << 20) || M > (1 << 20))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_gated: bad shape rows=%lld K=%lld M=%lld", (long long)rows, (long long)K, (long long)M);
+    if (ldx < K || ldy < M || ldgate < M) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_gated: row stride smaller than row");
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_linear_gated: bad dtype");
+    if (rows == 0) return BSRL_OK;
+    LinArgs a{x, ldx, w, nullptr, nullptr, 0, y, ldy, nullptr, 0, 0, rows, (int)K, (int)M, 0, 0, 0, gate, ldgate};
+    return lin_dispatch(a, BSRL_ACT_NONE, dtype, dtype, static_cast<hipStream_t>(stream), "bsrl_linear_gated");
 }

@@ -14,6 +14,9 @@ struct LinArgs {
     // grouped output rows (0 = off): output row r lives at (r / y_group) * y_gstride + (r % y_group) * ldy,
     // i.e. y is a (rows / y_group, y_group, M) view of a larger tensor (a token slice of a (B, T, d) stream)
     int y_group; int64_t y_gstride;
+    // ReLU gate (NULL = off): the result is kept where gate[row * ldgate + col] > 0 and zeroed elsewhere - the
+    // backward of a ReLU whose forward output is `gate`, applied in the epilogue of the data-gradient GEMM
+    const void* gate; int64_t ldgate;
 };
 
 // element offset of output row `row` in y (rows < 2^31 is checked on the host)

@@ -125,6 +125,13 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
                         v[0] += DT::to_f((u16)(rv.x & 0xffff)); v[1] += DT::to_f((u16)(rv.x >> 16));
                         v[2] += DT::to_f((u16)(rv.y & 0xffff)); v[3] += DT::to_f((u16)(rv.y >> 16));
                     }
+                    if (a.gate) {
+                        const uint2 gv = *reinterpret_cast<const uint2*>(static_cast<const u16*>(a.gate) + row * a.ldgate + col);
+                        if (!(DT::to_f((u16)(gv.x & 0xffff)) > 0.f)) v[0] = 0.f;
+                        if (!(DT::to_f((u16)(gv.x >> 16)) > 0.f)) v[1] = 0.f;
+                        if (!(DT::to_f((u16)(gv.y & 0xffff)) > 0.f)) v[2] = 0.f;
+                        if (!(DT::to_f((u16)(gv.y >> 16)) > 0.f)) v[3] = 0.f;
+                    }
                     uint2 ov;
                     ov.x = (uint32_t)DT::from_f(v[0]) | ((uint32_t)DT::from_f(v[1]) << 16);
                     ov.y = (uint32_t)DT::from_f(v[2]) | ((uint32_t)DT::from_f(v[3]) << 16);
@@ -150,6 +157,7 @@ bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st) {
     // worth it only when there are enough rows to fill the chip with 256-row tiles
     if (a.out_f32 || a.y2 || a.rows < 4096 || a.M % 8 != 0 || a.K % 8 != 0) return false;
     if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16) || (a.res && (a.ldr % 8 != 0 || !bsrl_aligned(a.res, 16)))) return false;
+    if (a.gate && (a.ldgate % 4 != 0 || !bsrl_aligned(a.gate, 8))) return false;
     if ((a.rows + BM - 1) / BM > 65535) return false;
     if (dtype == BSRL_F16) launch<F16>(a, act, st);
     else launch<BF16>(a, act, st);

@@ -234,6 +234,29 @@ def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None,
     return y if split is None else (y, y2)
 
 
+def linear_gated(x, w, gate):
+    """(x @ w.T) * [gate > 0]: the data gradient of a Linear masked by the ReLU before it, in one
+    GEMM (reference fp16_gemm.dgrad_drelu, fp16_gemm.cu:479-518).  x (..., K), w (M, K) contiguous
+    (the forward weight transposed), gate (..., M) = the ReLU's forward output; one dtype."""
+    _need_cuda(x, w, gate)
+    if x.dtype is not w.dtype or gate.dtype is not x.dtype:
+        raise TypeError("linear_gated: x, w and gate must share one dtype")
+    if not w.is_contiguous() or w.dim() != 2 or x.shape[-1] != w.shape[1]:
+        raise RuntimeError("linear_gated: w must be a contiguous (M, K) matrix matching x's K")
+    M, K = w.shape
+    if gate.shape != (*x.shape[:-1], M):
+        raise RuntimeError("linear_gated: gate must be (..., M)")
+    x2, rows, ldx = _rows2d(x)
+    g2, _, ldg = _rows2d(gate)
+    y = torch.empty(*x.shape[:-1], M, device=x.device, dtype=x.dtype)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_linear_gated(x2.data_ptr(), ldx, w.data_ptr(), g2.data_ptr(), ldg, y.data_ptr(), M,
+                                           rows, K, M, dt_code(x.dtype), _stream(x))
+    if not _lib.check(rc, "bsrl_linear_gated"):
+        raise Unsupported(f"linear_gated rows={rows} K={K} M={M} dtype={x.dtype}")
+    return y
+
+
 def attn_fwd(q, k, v, n_heads, key_bias=None, n_valid=None):
     """softmax(q k^T / sqrt(dh) + key_bias) v per head.  q (B, TQ, d), k/v
     (B, T, d): any batch/row strides (views of a packed projection are fine),

@@ -279,6 +279,19 @@ int bsrl_ln_bwd(const void* x, const void* dy, const float* weight,
                 void* dx, float* dw, float* db, float* dbb, void* workspace,
                 int64_t rows, int64_t d, int dtype, bsrl_stream stream);
 
+/* ---- Data gradient through a ReLU -------------------------------------------------
+ * Replaces fp16_gemm.dgrad_drelu(g, w, mask) (python/beat_arena_env/csrc/
+ * fp16_gemm.cu:479-518; caller python/fp16_linear.py:719-727, 1241-1245):
+ *   y[r, m] = (sum_k x[r, k] * w[m, k]) * [gate[r, m] > 0]
+ * i.e. the data gradient of the Linear AFTER a ReLU (x = its output gradient,
+ * w = its weight transposed, (M, K) contiguous) masked by that ReLU in the GEMM
+ * epilogue; gate = the ReLU's forward output (the saved hidden), which stands in
+ * for the reference's bitmask.  x (rows, K) pitch ldx, gate / y (rows, M) pitches
+ * ldgate / ldy, all in `dtype`; same kernels and shape coverage as bsrl_linear. */
+int bsrl_linear_gated(const void* x, int64_t ldx, const void* w, const void* gate, int64_t ldgate,
+                      void* y, int64_t ldy, int64_t rows, int64_t K, int64_t M, int dtype,
+                      bsrl_stream stream);
+
 /* ---- Linear weight / bias gradient -----------------------------------------------
  * Replaces fp16_gemm.wgrad(dy, x) -> dW and wgrad_bgrad(dy, x) -> [dW, db]
  * (python/beat_arena_env/csrc/fp16_gemm.cu:189-277, 404-476; callers

@@ -467,3 +467,20 @@ def test_wgrad_strided_operands_and_empty_batch():
     e = torch.empty(0, 64, device=DEV, dtype=torch.float16)
     dw, db = ops.wgrad(e, e)
     assert torch.equal(dw, torch.zeros(64, 64, device=DEV)) and torch.equal(db, torch.zeros(64, device=DEV))
+
+
+# ---------------------------------------------------------------- data gradient through a ReLU
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("rows,K,M", [(1, 8, 8), (77, 192, 768), (5000, 192, 768), (4096, 128, 512), (333, 40, 101), (129, 256, 96)])
+def test_linear_gated(dtype, rows, K, M):
+    """(g @ W) * [hidden > 0] == autograd through relu(h @ W1^T) @ W2^T at the hidden (python/fp16_linear.py:719-727)."""
+    g = _rand(rows, K, dtype=dtype, seed=rows + K)
+    wt = _rand(M, K, dtype=dtype, seed=rows + M + 1, scale=K ** -0.5)          # forward weight (K, M) transposed
+    hid = torch.relu(_rand(rows, M, dtype=dtype, seed=rows + 2))
+    hid[0, 0] = 0.0                                                             # an exact zero is gated off (relu'(0) = 0)
+    out = ops.linear_gated(g, wt, hid)
+    ref = (g.double() @ wt.double().t()) * (hid > 0).double()
+    assert torch.equal(out == 0, ref == 0) or ((out != 0) != (ref != 0)).sum().item() <= 2       # exact cancellations aside
+    tol = 1e-5 if dtype is torch.float32 else 1.5 * EPS16[dtype]
+    assert (out.double() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
+    assert torch.equal(out[hid <= 0], torch.zeros_like(out[hid <= 0]))
