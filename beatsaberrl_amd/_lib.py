@@ -70,6 +70,8 @@ SIGNATURES = {
                                  _p, _p, _p, _p, _p, _p]),
     "bsrl_ln_bwd_workspace_size": (_i64, [_i64]),
     "bsrl_ln_bwd": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),
+    "bsrl_attn_bwd": (_i32, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _i64,
+                             _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_linear_gated": (_i32, [_p, _i64, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_wgrad_workspace_size": (_i64, [_i64, _i64]),
     "bsrl_wgrad": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),

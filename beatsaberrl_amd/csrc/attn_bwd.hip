@@ -1,0 +1,324 @@
+// Backward of the short-sequence masked multi-head attention (T <= 48 keys) for gfx950.
+//
+// Replaces fp16_gemm.attn29_bwd(q, k, v, bias, dout, dq, dk, dv) (reference
+// python/beat_arena_env/csrc/small_attn.cu:345-463, 539-571; callers python/fp16_linear.py:930-1000):
+// the probabilities are recomputed from q, k and the key mask exactly as the forward computes them
+// (fp32 scores, fp32 softmax), then
+//     dP = dO V^T,  dS = P * (dP - rowsum(P * dP)),  dQ = scale dS K,  dK = scale dS^T Q,  dV = P^T dO
+// and the three gradients are written through strides, so they may be column slices of one packed
+// q|k|v gradient buffer (what the reference's callers pass).
+//
+// 16-bit path: one wave64 per (env, head), 2 waves per workgroup.  q, k, v, dO of the pair are
+// staged once in LDS as they lie in memory (rows = tokens); every product is a chain of
+// v_mfma_f32_16x16x16 with the operand orientation each one needs:
+//   S^T = K Q^T and dP^T = V dO^T contract over features: both operands are plain 8-byte row reads;
+//   a lane ends with 4 consecutive KEYS of one query, so the softmax and the rowsum are in-lane
+//   steps plus two butterflies (lane ^ 16, lane ^ 32), and dS^T packs straight into the B operand of
+//   dQ^T = K^T dS^T, whose A operand (K^T) is an LDS transpose load (ds_read_b64_tr_b16);
+//   dV^T = dO^T P and dK^T = Q^T dS contract over QUERIES: P and dS of the current 16-query tile go
+//   through a 16-row LDS tile and both operands come back through transpose loads.
+// Every output lane holds 4 consecutive features of one token: 8-byte stores.  dK^T / dV^T stay in
+// accumulators across the query tiles.  HBM traffic: q, k, v, dO read once, dq, dk, dv written once.
+//
+// fp32 path (parity configuration): one wave per (env, head) on LDS-staged fp32 tiles, plain FMA loops.
+#include "bsrl_common.h"
+
+namespace {
+
+struct AttnBwdArgs {
+    const void *q, *k, *v, *dout;
+    int64_t q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs;
+    const void* key_bias; const int32_t* n_valid;
+    void *dq, *dk, *dv;
+    int64_t dq_bs, dq_rs, dk_bs, dk_rs, dv_bs, dv_rs;
+    int64_t B; int T, TQ, H;
+    float scale;
+    int wave_elems;            // 16-bit path: LDS elements per wave
+};
+
+constexpr int kMaxKT = 3;      // key tiles of 16 (T <= 48)
+typedef short s16x4v __attribute__((ext_vector_type(4)));
+
+// 16x16x16 operand whose contraction index runs over the ROWS of a row-major LDS tile: lane (i = lane % 16,
+// g = lane / 16) ends with rows k0 + 4 g + {0..3} of column c0 + i.  Lanes 4 r + s of a 16-lane group present
+// the 4 elements at column c0 + 4 s of row k0 + 4 g + r; the hardware hands lane i element i of rows 0..3.
+__device__ __forceinline__ s16x4 tr16(const u16* tile, int pitch, int k0, int c0, int lane) {
+    const int i = lane & 15, g = lane >> 4;
+    const u16* p = tile + (k0 + 4 * g + (i >> 2)) * pitch + c0 + 4 * (i & 3);
+    typedef __attribute__((address_space(3))) s16x4v* lptr;
+    const s16x4v t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p));
+    return (s16x4){t[0], t[1], t[2], t[3]};
+}
+// operand whose contraction index runs ALONG a row: lane (i, g) reads columns c0 + 4 g .. + 3 of row r0 + i
+__device__ __forceinline__ s16x4 row16(const u16* tile, int pitch, int r0, int c0, int lane) {
+    return *reinterpret_cast<const s16x4*>(tile + (r0 + (lane & 15)) * pitch + c0 + 4 * (lane >> 4));
+}
+
+template <typename DT, int DH>
+__global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
+    constexpr int DHP = DH == 32 ? 48 : 56;     // LDS row pitch of the token tiles (elements)
+    constexpr int FT = DH / 16;
+    extern __shared__ __attribute__((aligned(16))) u16 smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int64_t pair = (int64_t)blockIdx.x * 2 + wave;
+    if (pair >= a.B * a.H) return;                                   // waves are independent: no workgroup barrier below
+    const int64_t b = pair / a.H;
+    const int h = (int)(pair % a.H);
+    const int T = a.T, TQ = a.TQ;
+    const int nkt = (T + 15) >> 4, nqt = (TQ + 15) >> 4;
+    const int TP = nkt * 16, TQP = nqt * 16, PP = TP + 8;
+    u16* Qs = smem + (int64_t)wave * a.wave_elems;
+    u16* dOs = Qs + TQP * DHP;
+    u16* Ks = dOs + TQP * DHP;
+    u16* Vs = Ks + TP * DHP;
+    u16* Ps = Vs + TP * DHP;
+    u16* dSs = Ps + 16 * PP;
+
+    // stage the pair's q, dO (TQ rows) and k, v (T rows), zero rows up to the tile edge
+    auto stage = [&](u16* dst, const void* src, int64_t bs, int64_t rs, int nrows, int prows) {
+        const u16* sp = static_cast<const u16*>(src) + b * bs + h * DH;
+        for (int c = lane; c < prows * (DH / 8); c += WAVE) {
+            const int row = c / (DH / 8), part = c % (DH / 8);
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (row < nrows) val = *reinterpret_cast<const uint4*>(sp + (int64_t)row * rs + part * 8);
+            *reinterpret_cast<uint4*>(dst + row * DHP + part * 8) = val;
+        }
+    };
+    stage(Qs, a.q, a.q_bs, a.q_rs, TQ, TQP);
+    stage(dOs, a.dout, a.do_bs, a.do_rs, TQ, TQP);
+    stage(Ks, a.k, a.k_bs, a.k_rs, T, TP);
+    stage(Vs, a.v, a.v_bs, a.v_rs, T, TP);
+
+    // additive bias / validity of keys 16 kt + 4 g + e, as the forward applies them
+    float kb[kMaxKT][4];
+    const int nv = a.n_valid ? a.n_valid[b] : T;
+#pragma unroll
+    for (int kt = 0; kt < kMaxKT; ++kt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int key = kt * 16 + g * 4 + e;
+            float bias = 0.f;
+            if (key >= T || key > nv) bias = -INFINITY;
+            else if (a.key_bias) {
+                const float kbv = DT::to_f(static_cast<const u16*>(a.key_bias)[b * T + key]);
+                bias = kbv < -0.5f * BSRL_MASK_BIAS ? -INFINITY : kbv;
+            }
+            kb[kt][e] = bias;
+        }
+
+    f32x4 dkt[FT][kMaxKT], dvt[FT][kMaxKT];      // dK^T, dV^T: lane holds features 16 ft + 4 g + e of key 16 kt + r16
+#pragma unroll
+    for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt) { dkt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; dvt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+
+    u16* dqp = static_cast<u16*>(a.dq) + b * a.dq_bs + h * DH;
+    for (int qt = 0; qt < nqt; ++qt) {
+        // S^T and dP^T tiles: lane holds keys 16 kt + 4 g + e of query 16 qt + r16
+        float s[kMaxKT][4], dp[kMaxKT][4];
+        float m = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt) {
+            f32x4 sa = {0.f, 0.f, 0.f, 0.f}, da = {0.f, 0.f, 0.f, 0.f};
+            if (kt < nkt) {
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    sa = DT::mfma16(row16(Ks, DHP, kt * 16, ft * 16, lane), row16(Qs, DHP, qt * 16, ft * 16, lane), sa);
+                    da = DT::mfma16(row16(Vs, DHP, kt * 16, ft * 16, lane), row16(dOs, DHP, qt * 16, ft * 16, lane), da);
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                s[kt][e] = sa[e] * a.scale + kb[kt][e];
+                dp[kt][e] = da[e];
+                m = fmaxf(m, s[kt][e]);
+            }
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, WAVE));
+        m = fmaxf(m, __shfl_xor(m, 32, WAVE));
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { s[kt][e] = __expf(s[kt][e] - m); sum += s[kt][e]; }
+        sum += __shfl_xor(sum, 16, WAVE);
+        sum += __shfl_xor(sum, 32, WAVE);
+        const float inv = 1.0f / sum;
+        float dsum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { s[kt][e] *= inv; dsum += s[kt][e] * dp[kt][e]; }      // s = P from here on
+        dsum += __shfl_xor(dsum, 16, WAVE);
+        dsum += __shfl_xor(dsum, 32, WAVE);
+        s16x4 dsf[kMaxKT];
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt) {
+            uint32_t pw[2], dw[2];
+#pragma unroll
+            for (int e = 0; e < 4; e += 2) {
+                const float d0 = s[kt][e] * (dp[kt][e] - dsum), d1 = s[kt][e + 1] * (dp[kt][e + 1] - dsum);
+                pw[e >> 1] = (uint32_t)DT::from_f(s[kt][e]) | ((uint32_t)DT::from_f(s[kt][e + 1]) << 16);
+                dw[e >> 1] = (uint32_t)DT::from_f(d0) | ((uint32_t)DT::from_f(d1) << 16);
+            }
+            dsf[kt] = __builtin_bit_cast(s16x4, make_uint2(dw[0], dw[1]));
+            if (kt < nkt) {                     // row = the lane's query, 4 consecutive keys: one 8-byte LDS write each
+                *reinterpret_cast<uint2*>(Ps + r16 * PP + kt * 16 + 4 * g) = make_uint2(pw[0], pw[1]);
+                *reinterpret_cast<uint2*>(dSs + r16 * PP + kt * 16 + 4 * g) = make_uint2(dw[0], dw[1]);
+            }
+        }
+        // dQ^T = K^T dS^T: A = K^T (transpose load, contraction over keys), B = dS^T from registers
+        const int qrow = qt * 16 + r16;
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) {
+            f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kt = 0; kt < kMaxKT; ++kt)
+                if (kt < nkt) o = DT::mfma16(tr16(Ks, DHP, kt * 16, ft * 16, lane), dsf[kt], o);
+            if (qrow < TQ) {
+                uint2 ov;
+                ov.x = (uint32_t)DT::from_f(o[0] * a.scale) | ((uint32_t)DT::from_f(o[1] * a.scale) << 16);
+                ov.y = (uint32_t)DT::from_f(o[2] * a.scale) | ((uint32_t)DT::from_f(o[3] * a.scale) << 16);
+                *reinterpret_cast<uint2*>(dqp + (int64_t)qrow * a.dq_rs + ft * 16 + 4 * g) = ov;
+            }
+        }
+        // dV^T += dO^T P, dK^T += Q^T dS: contraction over this tile's 16 queries, both operands transposed
+#pragma unroll
+        for (int kt = 0; kt < kMaxKT; ++kt) {
+            if (kt < nkt) {
+                const s16x4 pb = tr16(Ps, PP, 0, kt * 16, lane), db = tr16(dSs, PP, 0, kt * 16, lane);
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    dvt[ft][kt] = DT::mfma16(tr16(dOs, DHP, qt * 16, ft * 16, lane), pb, dvt[ft][kt]);
+                    dkt[ft][kt] = DT::mfma16(tr16(Qs, DHP, qt * 16, ft * 16, lane), db, dkt[ft][kt]);
+                }
+            }
+        }
+    }
+    u16* dkp = static_cast<u16*>(a.dk) + b * a.dk_bs + h * DH;
+    u16* dvp = static_cast<u16*>(a.dv) + b * a.dv_bs + h * DH;
+#pragma unroll
+    for (int kt = 0; kt < kMaxKT; ++kt) {
+        const int key = kt * 16 + r16;
+        if (kt < nkt && key < T) {
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                uint2 kv, vv;
+                kv.x = (uint32_t)DT::from_f(dkt[ft][kt][0] * a.scale) | ((uint32_t)DT::from_f(dkt[ft][kt][1] * a.scale) << 16);
+                kv.y = (uint32_t)DT::from_f(dkt[ft][kt][2] * a.scale) | ((uint32_t)DT::from_f(dkt[ft][kt][3] * a.scale) << 16);
+                vv.x = (uint32_t)DT::from_f(dvt[ft][kt][0]) | ((uint32_t)DT::from_f(dvt[ft][kt][1]) << 16);
+                vv.y = (uint32_t)DT::from_f(dvt[ft][kt][2]) | ((uint32_t)DT::from_f(dvt[ft][kt][3]) << 16);
+                *reinterpret_cast<uint2*>(dkp + (int64_t)key * a.dk_rs + ft * 16 + 4 * g) = kv;
+                *reinterpret_cast<uint2*>(dvp + (int64_t)key * a.dv_rs + ft * 16 + 4 * g) = vv;
+            }
+        }
+    }
+}
+
+// fp32: one wave per (env, head); tiles in LDS, thread-per-element loops.  dh <= 48, T <= 48.
+__global__ __launch_bounds__(64) void attn_bwd_f32_kernel(AttnBwdArgs a, int dh) {
+    __shared__ float Qs[48 * 49], Ks[48 * 49], Vs[48 * 49], Os[48 * 49], Pm[48 * 49], Dm[48 * 49];
+    const int lane = threadIdx.x;
+    const int64_t pair = blockIdx.x;
+    const int64_t b = pair / a.H;
+    const int h = (int)(pair % a.H);
+    const int T = a.T, TQ = a.TQ;
+    const float* qp = static_cast<const float*>(a.q) + b * a.q_bs + h * dh;
+    const float* kp = static_cast<const float*>(a.k) + b * a.k_bs + h * dh;
+    const float* vp = static_cast<const float*>(a.v) + b * a.v_bs + h * dh;
+    const float* op = static_cast<const float*>(a.dout) + b * a.do_bs + h * dh;
+    for (int i = lane; i < TQ * dh; i += 64) { const int r = i / dh, c = i % dh; Qs[r * 49 + c] = qp[(int64_t)r * a.q_rs + c]; Os[r * 49 + c] = op[(int64_t)r * a.do_rs + c]; }
+    for (int i = lane; i < T * dh; i += 64) { const int r = i / dh, c = i % dh; Ks[r * 49 + c] = kp[(int64_t)r * a.k_rs + c]; Vs[r * 49 + c] = vp[(int64_t)r * a.v_rs + c]; }
+    __syncthreads();
+    const float* kbp = a.key_bias ? static_cast<const float*>(a.key_bias) + b * T : nullptr;
+    const int nv = a.n_valid ? a.n_valid[b] : T;
+    // scores and dP, one (query, key) per thread step
+    for (int i = lane; i < TQ * T; i += 64) {
+        const int qi = i / T, key = i % T;
+        float s = 0.f, d = 0.f;
+        for (int c = 0; c < dh; ++c) { s = fmaf(Qs[qi * 49 + c], Ks[key * 49 + c], s); d = fmaf(Os[qi * 49 + c], Vs[key * 49 + c], d); }
+        float bias = 0.f;
+        if (key > nv) bias = -INFINITY;
+        else if (kbp) bias = kbp[key] < -0.5f * BSRL_MASK_BIAS ? -INFINITY : kbp[key];
+        Pm[qi * 49 + key] = s * a.scale + bias;
+        Dm[qi * 49 + key] = d;
+    }
+    __syncthreads();
+    // softmax and dS per query row
+    for (int qi = lane; qi < TQ; qi += 64) {
+        float m = -INFINITY;
+        for (int key = 0; key < T; ++key) m = fmaxf(m, Pm[qi * 49 + key]);
+        float sum = 0.f;
+        for (int key = 0; key < T; ++key) { const float e = expf(Pm[qi * 49 + key] - m); Pm[qi * 49 + key] = e; sum += e; }
+        const float inv = 1.0f / sum;
+        float dsum = 0.f;
+        for (int key = 0; key < T; ++key) { const float p = Pm[qi * 49 + key] * inv; Pm[qi * 49 + key] = p; dsum = fmaf(p, Dm[qi * 49 + key], dsum); }
+        for (int key = 0; key < T; ++key) Dm[qi * 49 + key] = Pm[qi * 49 + key] * (Dm[qi * 49 + key] - dsum);
+    }
+    __syncthreads();
+    float* dqp = static_cast<float*>(a.dq) + b * a.dq_bs + h * dh;
+    float* dkp = static_cast<float*>(a.dk) + b * a.dk_bs + h * dh;
+    float* dvp = static_cast<float*>(a.dv) + b * a.dv_bs + h * dh;
+    for (int i = lane; i < TQ * dh; i += 64) {
+        const int qi = i / dh, c = i % dh;
+        float o = 0.f;
+        for (int key = 0; key < T; ++key) o = fmaf(Dm[qi * 49 + key], Ks[key * 49 + c], o);
+        dqp[(int64_t)qi * a.dq_rs + c] = o * a.scale;
+    }
+    for (int i = lane; i < T * dh; i += 64) {
+        const int key = i / dh, c = i % dh;
+        float ok = 0.f, ov = 0.f;
+        for (int qi = 0; qi < TQ; ++qi) { ok = fmaf(Dm[qi * 49 + key], Qs[qi * 49 + c], ok); ov = fmaf(Pm[qi * 49 + key], Os[qi * 49 + c], ov); }
+        dkp[(int64_t)key * a.dk_rs + c] = ok * a.scale;
+        dvp[(int64_t)key * a.dv_rs + c] = ov;
+    }
+}
+
+}  // namespace
+
+extern "C" int bsrl_attn_bwd(const void* q, int64_t q_bs, int64_t q_rs, const void* k, int64_t k_bs, int64_t k_rs,
+                             const void* v, int64_t v_bs, int64_t v_rs, const void* key_bias, const int32_t* n_valid,
+                             const void* dout, int64_t do_bs, int64_t do_rs,
+                             void* dq, int64_t dq_bs, int64_t dq_rs, void* dk, int64_t dk_bs, int64_t dk_rs,
+                             void* dv, int64_t dv_bs, int64_t dv_rs,
+                             int64_t B, int64_t T, int64_t TQ, int64_t H, int64_t dh, int dtype, bsrl_stream stream) {
+    if (!q || !k || !v || !dout || !dq || !dk || !dv) BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: null pointer");
+    if (B < 0 || T <= 0 || TQ <= 0 || TQ > T || H <= 0 || dh <= 0)
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: bad shape B=%lld T=%lld TQ=%lld H=%lld dh=%lld", (long long)B,
+                  (long long)T, (long long)TQ, (long long)H, (long long)dh);
+    if (key_bias && n_valid) BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: pass key_bias or n_valid, not both");
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: bad dtype %d", dtype);
+    if (T > BSRL_MAX_T) return BSRL_UNSUPPORTED;
+    if (B == 0) return BSRL_OK;
+    if (B * H > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: too many (env, head) pairs");
+    const double scale = 1.0 / sqrt((double)dh);
+    AttnBwdArgs a{q, k, v, dout, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs, key_bias, n_valid, dq, dk, dv,
+                  dq_bs, dq_rs, dk_bs, dk_rs, dv_bs, dv_rs, B, (int)T, (int)TQ, (int)H, (float)scale, 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == BSRL_F32) {
+        if (dh > 48) return BSRL_UNSUPPORTED;
+        hipLaunchKernelGGL(attn_bwd_f32_kernel, dim3((unsigned)(B * H)), dim3(64), 0, st, a, (int)dh);
+    } else {
+        if (dh != 32 && dh != 48) return BSRL_UNSUPPORTED;
+        // 16-byte row reads and 8-byte gradient stores through the strides
+        const int64_t in_s[] = {q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs};
+        for (int64_t s : in_s) if (s % 8 != 0) return BSRL_UNSUPPORTED;
+        const int64_t out_s[] = {dq_bs, dq_rs, dk_bs, dk_rs, dv_bs, dv_rs};
+        for (int64_t s : out_s) if (s % 4 != 0) return BSRL_UNSUPPORTED;
+        if (!bsrl_aligned(q, 16) || !bsrl_aligned(k, 16) || !bsrl_aligned(v, 16) || !bsrl_aligned(dout, 16) ||
+            !bsrl_aligned(dq, 8) || !bsrl_aligned(dk, 8) || !bsrl_aligned(dv, 8)) return BSRL_UNSUPPORTED;
+        const int dhp = dh == 32 ? 48 : 56;
+        const int tp = (int)((T + 15) / 16) * 16, tqp = (int)((TQ + 15) / 16) * 16;
+        a.wave_elems = (2 * tqp + 2 * tp) * dhp + 2 * 16 * (tp + 8);
+        a.wave_elems = (a.wave_elems + 7) & ~7;                          // keep each wave's region 16-byte aligned
+        const size_t lds = (size_t)2 * a.wave_elems * sizeof(u16);        // <= 50 KB
+        const dim3 grid((unsigned)((B * H + 1) / 2)), block(128);
+#define AB_GO(DT, DH) hipLaunchKernelGGL((attn_bwd_mfma_kernel<DT, DH>), grid, block, lds, st, a)
+        if (dtype == BSRL_F16) { if (dh == 32) AB_GO(F16, 32); else AB_GO(F16, 48); }
+        else { if (dh == 32) AB_GO(BF16, 32); else AB_GO(BF16, 48); }
+#undef AB_GO
+    }
+    BSRL_CHECK_LAUNCH("bsrl_attn_bwd");
+    return BSRL_OK;
+}

@@ -286,6 +286,37 @@ def attn_fwd(q, k, v, n_heads, key_bias=None, n_valid=None):
     return out
 
 
+def attn_bwd(q, k, v, dout, n_heads, key_bias=None, n_valid=None, out=None):
+    """(dq, dk, dv) of attn_fwd for the output gradient dout (B, TQ, d) (reference fp16_gemm.attn29_bwd,
+    small_attn.cu:539-571).  q / k / v / dout: any batch / row strides, unit last stride.  out: optional
+    (dq, dk, dv) views to write into (e.g. the column slices of one packed q|k|v gradient buffer)."""
+    _need_cuda(q, k, v, dout, key_bias, n_valid)
+    B, TQ, d = q.shape
+    T = k.shape[1]
+    if k.shape != (B, T, d) or v.shape != (B, T, d) or dout.shape != (B, TQ, d) or d % n_heads:
+        raise RuntimeError("attn_bwd: shape mismatch")
+    if out is None:
+        out = (torch.empty(B, TQ, d, device=q.device, dtype=q.dtype), torch.empty(B, T, d, device=q.device, dtype=q.dtype),
+               torch.empty(B, T, d, device=q.device, dtype=q.dtype))
+    dq, dk, dv = out
+    if dq.shape != q.shape or dk.shape != k.shape or dv.shape != v.shape:
+        raise RuntimeError("attn_bwd: gradient views must have the shapes of q, k, v")
+    for t in (q, k, v, dout, dq, dk, dv):
+        if t.stride(2) != 1 or t.dtype is not q.dtype:
+            raise RuntimeError("attn_bwd: every tensor needs unit last stride and one dtype")
+    if key_bias is not None and (key_bias.shape != (B, T) or key_bias.dtype is not q.dtype or not key_bias.is_contiguous()):
+        raise RuntimeError("attn_bwd: key_bias must be contiguous (B, T) in q's dtype")
+    if n_valid is not None and (n_valid.shape != (B,) or n_valid.dtype is not torch.int32 or not n_valid.is_contiguous()):
+        raise RuntimeError("attn_bwd: n_valid must be contiguous int32 (B,)")
+    st = lambda t: (t.data_ptr(), t.stride(0), t.stride(1))
+    with torch.cuda.device(q.device):
+        rc = _lib.load().bsrl_attn_bwd(*st(q), *st(k), *st(v), _ptr(key_bias), _ptr(n_valid), *st(dout), *st(dq), *st(dk),
+                                       *st(dv), B, T, TQ, n_heads, d // n_heads, dt_code(q.dtype), _stream(q))
+    if not _lib.check(rc, "bsrl_attn_bwd"):
+        raise Unsupported(f"attn_bwd T={T} TQ={TQ} H={n_heads} dh={d // n_heads} dtype={q.dtype}")
+    return dq, dk, dv
+
+
 def ffn_fused_supported(d, F, dtype) -> bool:
     return bool(_lib.load().bsrl_ffn_fused_supported(d, F, dt_code(dtype)))
 

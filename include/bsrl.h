@@ -105,6 +105,27 @@ int bsrl_attn_fwd(const void* q, int64_t q_bs, int64_t q_rs,
                   int64_t B, int64_t T, int64_t TQ, int64_t H, int64_t dh,
                   int dtype, bsrl_stream stream);
 
+/* Backward of bsrl_attn_fwd; replaces fp16_gemm.attn29_bwd(q, k, v, bias, dout,
+ * dq, dk, dv) (small_attn.cu:345-463, 539-571), which likewise writes the three
+ * gradients into caller views (column slices of one packed q|k|v gradient).
+ * The probabilities are recomputed from q, k and the mask as the forward does:
+ *   dP = dO V^T, dS = P * (dP - rowsum(P * dP)), dQ = dS K / sqrt(dh),
+ *   dK = dS^T Q / sqrt(dh), dV = P^T dO        (fp32 scores / softmax / sums)
+ * q, k, v, key_bias, n_valid, B, T, TQ, H, dh: as bsrl_attn_fwd.  dout (B, TQ, H*dh),
+ * dq (B, TQ, H*dh), dk, dv (B, T, H*dh): element (b, t, c) at p[b*bs + t*rs + c],
+ * each with its own strides; masked keys get dk = dv = 0.  16-bit: dh in {32, 48},
+ * 16-byte aligned input rows, 8-byte aligned gradient rows; F32: dh <= 48. */
+int bsrl_attn_bwd(const void* q, int64_t q_bs, int64_t q_rs,
+                  const void* k, int64_t k_bs, int64_t k_rs,
+                  const void* v, int64_t v_bs, int64_t v_rs,
+                  const void* key_bias, const int32_t* n_valid,
+                  const void* dout, int64_t do_bs, int64_t do_rs,
+                  void* dq, int64_t dq_bs, int64_t dq_rs,
+                  void* dk, int64_t dk_bs, int64_t dk_rs,
+                  void* dv, int64_t dv_bs, int64_t dv_rs,
+                  int64_t B, int64_t T, int64_t TQ, int64_t H, int64_t dh,
+                  int dtype, bsrl_stream stream);
+
 /* ---- Fused FFN ------------------------------------------------------------
  * Replaces fp16_gemm.ffn_fused (fused_ffn.cu:551-619):
  *   xo = x + act(h2 w0^T + b0) w2^T + b2 ;  ho = LN_next(xo) if ln_w != NULL

@@ -484,3 +484,40 @@ def test_linear_gated(dtype, rows, K, M):
     tol = 1e-5 if dtype is torch.float32 else 1.5 * EPS16[dtype]
     assert (out.double() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
     assert torch.equal(out[hid <= 0], torch.zeros_like(out[hid <= 0]))
+
+
+# ---------------------------------------------------------------- Attention backward
+@pytest.mark.parametrize("dtype", DTS)
+@pytest.mark.parametrize("T,TQ,H,dh", [(16, 16, 4, 32), (29, 29, 4, 48), (29, 5, 4, 48), (29, 1, 4, 48),
+                                       (32, 32, 8, 32), (48, 48, 12, 32), (48, 1, 12, 32), (6, 6, 2, 32), (17, 3, 4, 32)])
+@pytest.mark.parametrize("mask", ["none", "n_valid", "bias"])
+def test_attention_backward(dtype, T, TQ, H, dh, mask):
+    """dq, dk, dv against torch autograd through the fp64 closed form on the same rounded operands
+    (python/tests/test_attn29.py:157-214 compares the same three gradients against the SDPA path)."""
+    B, d = 7, H * dh
+    qkv = _rand(B, T, 3 * d, dtype=dtype, seed=T + TQ)
+    q, k, v = qkv[:, :TQ, :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+    dout = _rand(B, TQ, d, dtype=dtype, seed=T + TQ + 9)
+    g = torch.Generator().manual_seed(5)
+    nv = torch.randint(0, T, (B,), generator=g, dtype=torch.int32)
+    nv[0] = 0
+    nv[1] = T - 1
+    valid = (torch.arange(T)[None, :] <= nv[:, None]).float()
+    bias = ((valid - 1.0) * 16384.0).to(dtype).to(DEV)
+    kw = {} if mask == "none" else {"n_valid": nv.to(DEV)} if mask == "n_valid" else {"key_bias": bias}
+    # gradients land in the column slices of one packed buffer, as the reference's callers have them
+    packed = torch.full((B, T, 3 * d), 7.0, device=DEV, dtype=dtype)
+    dq, dk, dv = ops.attn_bwd(q, k, v, dout, H, out=(packed[:, :TQ, :d], packed[..., d:2 * d], packed[..., 2 * d:]), **kw)
+    qd, kd, vd = (t.double().detach().clone().requires_grad_(True) for t in (q, k, v))
+    _attn_ref(qd, kd, vd, H, None if mask == "none" else bias).backward(dout.double())
+    for name, got, want in (("dq", dq, qd.grad), ("dk", dk, kd.grad), ("dv", dv, vd.grad)):
+        tol = 3e-5 if dtype is torch.float32 else 4 * EPS16[dtype]
+        err = (got.double() - want).abs().max().item()
+        assert err <= tol * (want.abs().max().item() + 1.0), (name, err)
+    if TQ < T:
+        assert torch.equal(packed[:, TQ:, :d], torch.full_like(packed[:, TQ:, :d], 7.0))      # nothing written past the queries
+    if mask != "none":                                        # masked keys: exactly zero gradient
+        dead = ~(valid.bool().to(DEV))
+        assert torch.equal(dk[dead], torch.zeros_like(dk[dead])) and torch.equal(dv[dead], torch.zeros_like(dv[dead]))
+    dq2, dk2, dv2 = ops.attn_bwd(q, k, v, dout, H, **kw)      # fresh contiguous outputs, same bits
+    assert torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
