@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -73,6 +73,7 @@ SIGNATURES = {
     "bsrl_attn_bwd": (_i32, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _i64,
                              _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_linear_gated": (_i32, [_p, _i64, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "bsrl_relu_bwd": (_i32, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_wgrad_workspace_size": (_i64, [_i64, _i64]),
     "bsrl_wgrad": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_vres_mix": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),

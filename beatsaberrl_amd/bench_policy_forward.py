@@ -80,6 +80,7 @@ def build_policy(args, device):
     return policy
 
 
+@torch.no_grad()
 def main(argv=None):
     p = argparse.ArgumentParser(description=__doc__.splitlines()[0])
     p.add_argument("--ckpt", default="runs/perf_ref.pt")

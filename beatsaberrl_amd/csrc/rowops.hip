@@ -1,5 +1,8 @@
-// Row-wise stages of two architecture options of the policy; HBM-bound elementwise / row-reduction work.
+// Row-wise stages of two architecture options of the policy, and the ReLU gradient mask; HBM-bound
+// elementwise / row-reduction work.
 //
+//  * ReLU backward (reference fp16_gemm.relu_bwd, python/beat_arena_env/csrc/fp16_gemm.cu:113-187): gm = g * [y > 0]
+//    from the saved post-ReLU y, for a ReLU whose consumer is not a GEMM this library can gate.
 //  * value-residual mix (reference python/fp16_linear.py:1002-1006, python/policy.py:568-611):
 //        out = a * v + b * v0      fp32 arithmetic, rounded once to the stream dtype; (a, b) live on the device
 //    (learned scalars), exactly v at (a, b) = (1, 0).
@@ -50,6 +53,29 @@ __global__ __launch_bounds__(256) void vres_mix_kernel(MixArgs m) {
         *reinterpret_cast<TV*>(po) = o;
     } else {
         *po = El<IO>::r(fmaf(El<IO>::f(*p0), b, El<IO>::f(*pv) * a));
+    }
+}
+
+// gradient through a ReLU: out = g where the ReLU's forward output y is positive, 0 elsewhere
+template <typename IO, int VEC>
+__global__ __launch_bounds__(256) void relu_bwd_kernel(MixArgs m) {
+    typedef typename El<IO>::T T;
+    const int per_row = m.d / VEC;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= m.rows * per_row) return;
+    const int64_t row = i / per_row; const int c = (int)(i % per_row) * VEC;
+    const T* pg = static_cast<const T*>(m.v) + row * m.ldv + c;
+    const T* py = static_cast<const T*>(m.v0) + row * m.ldv0 + c;
+    T* po = static_cast<T*>(m.out) + row * m.ldo + c;
+    if (VEC > 1) {
+        typedef T TV __attribute__((ext_vector_type(VEC > 1 ? VEC : 2)));
+        const TV gv = *reinterpret_cast<const TV*>(pg), yv = *reinterpret_cast<const TV*>(py);
+        TV o;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = El<IO>::f(yv[j]) > 0.f ? gv[j] : (T)0;
+        *reinterpret_cast<TV*>(po) = o;
+    } else {
+        *po = El<IO>::f(*py) > 0.f ? *pg : (T)0;
     }
 }
 
@@ -107,36 +133,53 @@ __global__ __launch_bounds__(256) void hsphere_kernel(HsArgs h) {
 }
 
 template <typename IO>
-int mix_launch(const MixArgs& m, int vec, hipStream_t st) {
+int mix_launch(const MixArgs& m, int vec, bool relu, hipStream_t st) {
     const int64_t n = m.rows * (m.d / vec);
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-    if (vec == 8) hipLaunchKernelGGL((vres_mix_kernel<IO, 8>), grid, block, 0, st, m);
-    else if (vec == 4) hipLaunchKernelGGL((vres_mix_kernel<IO, 4>), grid, block, 0, st, m);
-    else hipLaunchKernelGGL((vres_mix_kernel<IO, 1>), grid, block, 0, st, m);
-    BSRL_CHECK_LAUNCH("bsrl_vres_mix");
+    if (relu) {
+        if (vec == 8) hipLaunchKernelGGL((relu_bwd_kernel<IO, 8>), grid, block, 0, st, m);
+        else if (vec == 4) hipLaunchKernelGGL((relu_bwd_kernel<IO, 4>), grid, block, 0, st, m);
+        else hipLaunchKernelGGL((relu_bwd_kernel<IO, 1>), grid, block, 0, st, m);
+    } else {
+        if (vec == 8) hipLaunchKernelGGL((vres_mix_kernel<IO, 8>), grid, block, 0, st, m);
+        else if (vec == 4) hipLaunchKernelGGL((vres_mix_kernel<IO, 4>), grid, block, 0, st, m);
+        else hipLaunchKernelGGL((vres_mix_kernel<IO, 1>), grid, block, 0, st, m);
+    }
+    BSRL_CHECK_LAUNCH(relu ? "bsrl_relu_bwd" : "bsrl_vres_mix");
     return BSRL_OK;
+}
+
+// shared argument checks and dispatch of the two elementwise (rows, d) kernels above
+int mix_entry(const char* what, bool relu, const void* v, int64_t ldv, const void* v0, int64_t ldv0, const float* a,
+              const float* b, void* out, int64_t ldo, int64_t rows, int64_t d, int dtype, bsrl_stream stream) {
+    if (!v || !v0 || !out || (!relu && (!a || !b))) BSRL_FAIL(BSRL_EINVAL, "%s: null pointer", what);
+    if (rows < 0 || d < 1 || d > (1 << 20) || ldv < d || ldv0 < d || ldo < d)
+        BSRL_FAIL(BSRL_EINVAL, "%s: need rows >= 0, 1 <= d <= 2^20 and row pitches >= d", what);
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "%s: bad dtype %d", what, dtype);
+    if (rows == 0) return BSRL_OK;
+    if (rows * d > ((int64_t)1 << 40)) BSRL_FAIL(BSRL_EINVAL, "%s: rows * d too large", what);
+    const int want = dtype == BSRL_F32 ? 4 : 8;                    // 16-byte accesses
+    const bool vec_ok = d % want == 0 && ldv % want == 0 && ldv0 % want == 0 && ldo % want == 0 &&
+                        bsrl_aligned(v, 16) && bsrl_aligned(v0, 16) && bsrl_aligned(out, 16);
+    const int vec = vec_ok ? want : 1;
+    if ((rows * (d / vec) + 255) / 256 > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "%s: grid too large", what);
+    const MixArgs m{v, ldv, v0, ldv0, a, b, out, ldo, rows, (int)d};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == BSRL_F32) return mix_launch<F32IO>(m, vec, relu, st);
+    if (dtype == BSRL_F16) return mix_launch<F16>(m, vec, relu, st);
+    return mix_launch<BF16>(m, vec, relu, st);
 }
 
 }  // namespace
 
 extern "C" int bsrl_vres_mix(const void* v, int64_t ldv, const void* v0, int64_t ldv0, const float* a, const float* b,
                              void* out, int64_t ldo, int64_t rows, int64_t d, int dtype, bsrl_stream stream) {
-    if (!v || !v0 || !a || !b || !out) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: null pointer");
-    if (rows < 0 || d < 1 || d > (1 << 20) || ldv < d || ldv0 < d || ldo < d)
-        BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: need rows >= 0, 1 <= d <= 2^20 and row pitches >= d");
-    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: bad dtype %d", dtype);
-    if (rows == 0) return BSRL_OK;
-    if (rows * d > ((int64_t)1 << 40)) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: rows * d too large");
-    const int want = dtype == BSRL_F32 ? 4 : 8;                    // 16-byte accesses
-    const bool vec_ok = d % want == 0 && ldv % want == 0 && ldv0 % want == 0 && ldo % want == 0 &&
-                        bsrl_aligned(v, 16) && bsrl_aligned(v0, 16) && bsrl_aligned(out, 16);
-    const int vec = vec_ok ? want : 1;
-    if ((rows * (d / vec) + 255) / 256 > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_vres_mix: grid too large");
-    const MixArgs m{v, ldv, v0, ldv0, a, b, out, ldo, rows, (int)d};
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == BSRL_F32) return mix_launch<F32IO>(m, vec, st);
-    if (dtype == BSRL_F16) return mix_launch<F16>(m, vec, st);
-    return mix_launch<BF16>(m, vec, st);
+    return mix_entry("bsrl_vres_mix", false, v, ldv, v0, ldv0, a, b, out, ldo, rows, d, dtype, stream);
+}
+
+extern "C" int bsrl_relu_bwd(const void* g, int64_t ldg, const void* y, int64_t ldy, void* out, int64_t ldo,
+                             int64_t rows, int64_t d, int dtype, bsrl_stream stream) {
+    return mix_entry("bsrl_relu_bwd", true, g, ldg, y, ldy, nullptr, nullptr, out, ldo, rows, d, dtype, stream);
 }
 
 extern "C" int bsrl_hsphere(int op, const void* t, const float* s, float c, const float* x32_in, float* x32_out,

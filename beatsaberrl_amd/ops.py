@@ -476,6 +476,21 @@ def vres_mix(v, v0, a, b, out=None):
     return out
 
 
+def relu_bwd(g, y):
+    """g * [y > 0] (reference fp16_gemm.relu_bwd): the gradient through a ReLU from its saved output."""
+    _need_cuda(g, y)
+    if g.shape != y.shape or g.dtype is not y.dtype:
+        raise TypeError("relu_bwd: g and y must share shape and dtype")
+    rows, d, ldg = _view2d(g, "relu_bwd g")
+    _, _, ldy = _view2d(y, "relu_bwd y")
+    out = torch.empty(g.shape, device=g.device, dtype=g.dtype)
+    with torch.cuda.device(g.device):
+        rc = _lib.load().bsrl_relu_bwd(g.data_ptr(), ldg, y.data_ptr(), ldy, out.data_ptr(), d, rows, d,
+                                       dt_code(g.dtype), _stream(g))
+    _lib.check(rc, "bsrl_relu_bwd")
+    return out
+
+
 HS_SCALE_L2N, HS_SCALE_RELU, HS_L2N_LERP = 0, 1, 2
 
 

@@ -16,6 +16,12 @@ same state_dict and checkpoints) and the same `forward_stacked(obs) -> (logits
   * in torch on the GPU (pure data movement): token concatenation, the ragged-head
     scatter and the 101-bin value expectation.
 
+Grad mode selects the path, as in the reference: under torch.no_grad() (rollout, evaluation) the
+forward-only routes above run; with grad mode on (the update), `forward_stacked` /
+`get_action_and_value(obs, action)` run op for op the per-op route as autograd Functions over the
+backward kernels (autograd_ops.py: LayerNorm, Linear data / weight / bias gradients, attention),
+so parameters receive fp32 gradients and the update forward is bitwise the per-op rollout forward.
+
 Stream dtype: `policy.fp16 = True` runs the 16-bit stream (fp16; set `stream_dtype =
 torch.bfloat16` for bf16) exactly as the reference's switch does (python/policy.py:
 1085-1090); otherwise fp32 kernels.  There is no CPU path and no torch fallback for
@@ -34,6 +40,7 @@ import torch.nn.functional as F
 from . import fp16_linear as _fl
 from . import obs_layout as L
 from . import ops
+from .autograd_ops import AttnPackedFn, AttnQKVFn, ChainFn, LinearFn
 from .fused_ln import FusedLayerNorm
 
 OBS_DIM = L.OBS_DIM
@@ -78,6 +85,25 @@ def _seq(seq: nn.Sequential, x, out=None):
         x = _lin(m, x, act="relu" if relu else None, out=out if last else None)
         i += 2 if relu else 1
     return x
+
+
+def _lin_t(m: nn.Linear, x, act=None, residual=None, out_f32=False):
+    """_lin under autograd: forward on the same kernel, backward on the gradient kernels."""
+    return LinearFn.apply(x, m.weight, m.bias, act, residual, out_f32)
+
+
+def _seq_t(seq: nn.Sequential, x, residual=None, out_f32=False):
+    """_seq under autograd: the whole Linear (ReLU Linear)* chain as one Function."""
+    lins = [m for m in seq if isinstance(m, nn.Linear)]
+    if len(lins) != (len(seq) + 1) // 2 or not all(isinstance(m, nn.ReLU) for m in list(seq)[1::2]):
+        raise RuntimeError("training path: Sequential must be Linear (ReLU Linear)*")
+    return ChainFn.apply(x, residual, out_f32, *[t for m in lins for t in (m.weight, m.bias)])
+
+
+def _packed_t(ms, x):
+    """Several same-input Linears as one GEMM under autograd: the concatenation is a torch op, so each
+    master receives its row block of the packed gradient (reference python/fp16_linear.py:459-470)."""
+    return LinearFn.apply(x, torch.cat([m.weight for m in ms]), torch.cat([m.bias for m in ms]), None, None, False)
 
 
 def note_geo(notes, sabers, z_asinh, flux, z_off):
@@ -181,6 +207,33 @@ class Block(nn.Module):
             hid = _lin(self.ffn[0], h2, act="relu")
             r = (_lin(self.ffn[2], hid, residual=x), None)
         return r + (v,) if want_v else r
+
+
+def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False):
+    """Block.forward under autograd (update path): the same kernels in the same order as the per-op
+    rollout route without the fused FFN, each paired with its backward; returns x_out (, v)."""
+    d = self.d
+    h = self.ln_attn(x)
+    if n_queries:
+        kv = _packed_t([self.k_proj, self.v_proj], h)
+        v = kv[..., d:]
+        if v0 is not None:
+            kv = torch.cat([kv[..., :d], torch.addcmul(v * self.vres_a, v0, self.vres_b).to(v.dtype)], -1)
+        q = _lin_t(self.q_proj, h[:, :n_queries])
+        att = AttnQKVFn.apply(q, kv, attn_bias, self.n_heads)
+        x = x[:, :n_queries].contiguous()
+    else:
+        qkv = _packed_t([self.q_proj, self.k_proj, self.v_proj], h)
+        v = qkv[..., 2 * d:]
+        if v0 is not None:
+            qkv = torch.cat([qkv[..., :2 * d], torch.addcmul(v * self.vres_a, v0, self.vres_b).to(v.dtype)], -1)
+        att = AttnPackedFn.apply(qkv, attn_bias, self.n_heads)
+    x = _lin_t(self.out_proj, att, residual=x)
+    x = _seq_t(self.ffn, self.ln_ffn(x), residual=x)
+    return (x, v) if want_v else x
+
+
+Block.forward_train = _block_train
 
 
 def build_head_gears(n_gears: int) -> tuple:
@@ -385,13 +438,16 @@ class NotePolicy(nn.Module):
         note_mask = obs[:, OFF_NOTE_MASK:OFF_NOTE_MASK + N_NOTE_SLOTS]
         return sabers, body, notes, note_mask
 
-    @torch.no_grad()
     def forward_stacked(self, obs):
-        """obs (B, 630) on the GPU -> logits (B, 29, k_max) fp32, value (B,) fp32."""
+        """obs (B, 630) on the GPU -> logits (B, 29, k_max) fp32, value (B,) fp32.  Under
+        torch.no_grad() (rollout, evaluation) the forward-only routes run, fused kernels included; with
+        grad mode on (the update) every op runs as an autograd Function over the backward kernels."""
         if not obs.is_cuda:
             raise RuntimeError("NotePolicy.forward_stacked runs on the GPU only (no CPU path)")
         if obs.dim() != 2 or obs.shape[1] != OBS_DIM:
             raise RuntimeError(f"obs must be (B, {OBS_DIM}), got {tuple(obs.shape)}")
+        if torch.is_grad_enabled():
+            return self._forward_train(obs)
         with contextlib.ExitStack() as modes:
             if self.fp16 and self.fp16_accum != "off":
                 modes.enter_context(_fl.fp16_accum(self.fp16_accum))
@@ -447,6 +503,66 @@ class NotePolicy(nn.Module):
             out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
         return out.view(B, N_ACTION_HEADS, self.k_max), value
 
+    def _forward_train(self, obs):
+        """The update-path forward: op for op the per-op rollout route (no fused FFN, no fused block
+        stack), so its outputs are that route's bits, with autograd Functions instead of bare kernels."""
+        dt = self.stream_dtype if self.fp16 else torch.float32
+        B, d = obs.shape[0], self.embed
+        obs = obs.detach()
+        if obs.dtype is not torch.float32 and obs.dtype is not dt:
+            obs = obs.float()
+        if obs.stride(1) != 1:
+            obs = obs.contiguous()
+        sab_in, torso_in, leg_in, note_in, attn_bias = ops.note_frontend(
+            obs, self._saber_idx32, self._body_idx32, dt, note_geo=self.note_geo, flux=self.game == "flux",
+            z_asinh=self.z_asinh)
+        x = torch.cat([_seq_t(self.saber_mlp, sab_in), _seq_t(self.torso_mlp, torso_in).unsqueeze(1),
+                       _seq_t(self.leg_mlp, leg_in), _seq_t(self.note_mlp, note_in)], 1)
+        if self.emb_ln is not None:
+            x = self.emb_ln(x)
+        v0 = None
+        for i, blk in enumerate(self.blocks[:-1]):
+            if self.value_residual and i == 0:
+                x, v0 = blk.forward_train(x, attn_bias, want_v=True)
+            else:
+                x = blk.forward_train(x, attn_bias, v0=v0)
+        x_res = x
+        lead = self.blocks[-1].forward_train(x, attn_bias, n_queries=self.n_lead, v0=v0)
+        if self.final_ln is not None:
+            lead = self.final_ln(lead)
+        z = lead.reshape(B, self.n_lead * d)
+        if self.trunk_arch == "simbav2":
+            hfeat = self._trunk_v2_train(z)
+        else:
+            t = _lin_t(self.trunk_proj, z)
+            hfeat = self.trunk_ln2(ChainFn.apply(self.trunk_ln1(t), t, False, self.trunk_fc1.weight, self.trunk_fc1.bias,
+                                                 self.trunk_fc2.weight, self.trunk_fc2.bias))
+        out = LinearFn.apply(hfeat, torch.cat([m.weight for m in self.heads]), torch.cat([m.bias for m in self.heads]),
+                             None, None, True)
+        # critic (adapool_v1)
+        hv = self.critic_ln(x_res)
+        q = _lin_t(self.critic_q, hv[:, 2:3])
+        kv = _packed_t([self.critic_k, self.critic_v], hv)
+        a = _lin_t(self.critic_out, AttnQKVFn.apply(q, kv, attn_bias, self.n_heads).view(B, d))
+        vlogits = _seq_t(self.critic_mlp, torch.cat([a, hfeat], dim=-1), out_f32=True)
+        self._value_logits = vlogits
+        value = torch.softmax(vlogits, dim=-1) @ self.value_centers
+        if self._gear_idx is not None:
+            out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
+        return out.view(B, N_ACTION_HEADS, self.k_max), value
+
+    def _trunk_v2_train(self, z):
+        """SimBaV2 readout under autograd: the three GEMMs on the gradient-aware Linear, the fp32 row work
+        (scalers, ReLU, normalisations, LERP) in torch ops on B rows, as the reference writes it
+        (python/policy.py:1146-1155)."""
+        dt = z.dtype
+        l2n = lambda t: F.normalize(t, dim=-1, eps=1e-6)
+        x = l2n(_lin_t(self.trunk_in, z).float() * (self.trunk_s_in * self._v2_c_in))
+        u = F.relu(_lin_t(self.trunk_w1, x.to(dt)).float() * (self.trunk_s_1 * self._v2_c_1))
+        y = l2n(_lin_t(self.trunk_w2, u.to(dt)).float())
+        x = l2n(x + (self.trunk_alpha * self._v2_c_alpha) * (y - x))
+        return (x * math.sqrt(x.shape[-1])).to(dt)
+
     def trunk_projected(self):
         """The Linears whose rows `project_trunk_weights` keeps unit-norm (python/policy.py:1157-1162)."""
         return [self.trunk_in, self.trunk_w1, self.trunk_w2] if self.trunk_arch == "simbav2" else []
@@ -501,14 +617,28 @@ class NotePolicy(nn.Module):
         logits, value = self.forward_stacked(obs)
         return list(logits.unbind(1)), value
 
-    @torch.no_grad()
     def get_action_and_value(self, obs, action=None, need_entropy=True):
-        """log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) in one kernel on
+        """With grad mode on and an action given (the update): log-prob and entropy of that action from
+        the training forward, in torch ops on the fp32 logits so that they carry gradients.  Otherwise:
+        log_softmax + Gumbel-max sampling + log-prob (+ per-head entropy) in one kernel on
         the forward's fp32 logits (reference python/policy.py:1467-1516).  `self.sampler`:
         "kernel" draws inside the kernel (Philox keyed by torch's seed and a per-module call
         counter that lives on the device and is advanced on the stream, so a captured call draws
         fresh noise on every replay); "torch" feeds the kernel Exp(1) draws from torch's default
         generator, the stream the reference rides."""
+        if torch.is_grad_enabled() and action is not None:
+            logits, value = self.forward_stacked(obs)
+            logsm = torch.log_softmax(logits, dim=-1)
+            logprob = logsm.gather(-1, action.long().unsqueeze(-1)).squeeze(-1).sum(-1)
+            entropy = None
+            if need_entropy:
+                self._ent_h = -(logsm.exp() * logsm).sum(-1)
+                entropy = self._ent_h.sum(-1)
+            return action, logprob, entropy, value
+        with torch.no_grad():
+            return self._act_rollout(obs, action, need_entropy)
+
+    def _act_rollout(self, obs, action, need_entropy):
         logits, value = self.forward_stacked(obs)
         logits = logits.contiguous()
         if action is not None and action.dtype not in (torch.int64, torch.uint8):

@@ -313,6 +313,13 @@ int bsrl_linear_gated(const void* x, int64_t ldx, const void* w, const void* gat
                       void* y, int64_t ldy, int64_t rows, int64_t K, int64_t M, int dtype,
                       bsrl_stream stream);
 
+/* gm = g * [y > 0]: the gradient through a ReLU from its saved forward output
+ * (fp16_gemm.relu_bwd, python/beat_arena_env/csrc/fp16_gemm.cu:113-187; the bias
+ * gradient the reference folds into that pass comes from bsrl_wgrad here).
+ * g, y, out: (rows, d) in `dtype` with row pitches in elements; out may alias g. */
+int bsrl_relu_bwd(const void* g, int64_t ldg, const void* y, int64_t ldy, void* out, int64_t ldo,
+                  int64_t rows, int64_t d, int dtype, bsrl_stream stream);
+
 /* ---- Linear weight / bias gradient -----------------------------------------------
  * Replaces fp16_gemm.wgrad(dy, x) -> dW and wgrad_bgrad(dy, x) -> [dW, db]
  * (python/beat_arena_env/csrc/fp16_gemm.cu:189-277, 404-476; callers

@@ -303,7 +303,7 @@ def forward(sd, arch, obs, emulate=None, return_parts=False):
     centers = torch.linspace(-float(arch["value_vmax"]), float(arch["value_vmax"]), int(arch["value_bins"]))
     value = torch.softmax(vlog, -1) @ centers
     if return_parts:
-        return logits, value, {"tokens": x, "x_res": x_res, "lead": lead, "h": h, "value_logits": vlog}
+        return logits, value, {"tokens": x, "x_res": x_res, "lead": lead, "h": h, "value_logits": vlog, "critic_a": a}
     return logits, value
 
 

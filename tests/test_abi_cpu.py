@@ -74,6 +74,24 @@ def test_new_entry_points_reject_bad_arguments_without_a_device(lib):
     assert lib.bsrl_hsphere(0, 16, 16, 1.0, None, None, 16, 4, 8, _lib.F32, None) == -1
     assert lib.bsrl_hsphere(2, 16, 16, 1.0, None, None, 16, 4, 8, _lib.F32, None) == -1
     assert lib.bsrl_hsphere(1, 16, 16, 1.0, None, None, 16, 0, 8, _lib.F32, None) == 0
+    # backward entry points: null pointers, bad shapes and dtypes are refused before any launch
+    assert lib.bsrl_ln_bwd_workspace_size(192) == 2048 * 3 * 192 * 4 and lib.bsrl_ln_bwd_workspace_size(0) == 0
+    assert lib.bsrl_ln_bwd(16, 16, 16, 16, 16, None, 16, 16, 16, None, None, 4, 128, _lib.F16, None) == -1
+    assert lib.bsrl_ln_bwd(16, 16, 16, 16, 16, None, 16, 16, 16, None, 16, 4, 0, _lib.F16, None) == -1
+    assert lib.bsrl_ln_bwd(16, 16, 16, 16, 16, None, 16, 16, 16, None, 16, 4, 100, _lib.F16, None) == 1      # d % 8 != 0: unsupported
+    assert lib.bsrl_wgrad_workspace_size(768, 192) == 128 * (768 * 192 + 768) * 4
+    assert lib.bsrl_wgrad(16, 8, 16, 8, 16, None, 16, 4, 8, 8, _lib.F32, None) == -1 and b"F16 or BF16" in lib.bsrl_last_error()
+    assert lib.bsrl_wgrad(16, 4, 16, 8, 16, None, 16, 4, 8, 8, _lib.F16, None) == -1
+    assert lib.bsrl_wgrad(16, 8, 16, 8, 16, None, None, 4, 8, 8, _lib.F16, None) == -1
+    assert lib.bsrl_linear_gated(16, 8, 16, None, 8, 16, 8, 4, 8, 8, _lib.F16, None) == -1
+    assert lib.bsrl_linear_gated(16, 8, 16, 16, 4, 16, 8, 4, 8, 8, _lib.F16, None) == -1
+    assert lib.bsrl_linear_gated(16, 8, 16, 16, 8, 16, 8, 0, 8, 8, _lib.F16, None) == 0
+    assert lib.bsrl_relu_bwd(16, 8, None, 8, 16, 8, 4, 8, _lib.F16, None) == -1
+    assert lib.bsrl_relu_bwd(16, 8, 16, 8, 16, 8, 0, 8, _lib.F16, None) == 0
+    ab = lambda T, TQ, dh, dt, q=16: lib.bsrl_attn_bwd(q, 96, 96, 16, 96, 96, 16, 96, 96, None, None, 16, 96, 96,
+                                                      16, 96, 96, 16, 96, 96, 16, 96, 96, 4, T, TQ, 1, dh, dt, None)
+    assert ab(29, 30, 32, _lib.F16) == -1 and ab(29, 29, 32, _lib.F16, q=None) == -1
+    assert ab(49, 5, 32, _lib.F16) == 1 and ab(29, 5, 40, _lib.F16) == 1 and ab(29, 5, 64, _lib.F32) == 1      # unsupported shapes
     # grouped linear: the group must divide the rows, fit its stride and exclude a split output
     g = lambda rows, grp, gs, y2=None, split=0: lib.bsrl_linear_grouped(
         16, 8, 16, None, None, 0, 16, 8, y2, 8 if y2 else 0, split, rows, 8, 8, 0, _lib.F16, _lib.F16, grp, gs, None)

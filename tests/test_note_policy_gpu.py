@@ -18,6 +18,13 @@ from beatsaberrl_amd.policy import NotePolicy, load_policy  # noqa: E402
 from oracle import note_policy_ref as nr  # noqa: E402
 
 DEV = "cuda"
+
+
+@pytest.fixture(autouse=True)
+def _rollout_mode():
+    """These tests exercise the forward-only (rollout) routes: grad mode off, as the rollout runs."""
+    with torch.no_grad():
+        yield
 GOLD = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "notepolicy_*.npz")))
 
 

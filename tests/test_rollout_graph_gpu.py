@@ -16,6 +16,13 @@ from oracle import note_policy_ref as nr  # noqa: E402
 DEV = "cuda"
 
 
+@pytest.fixture(autouse=True)
+def _rollout_mode():
+    """These tests exercise the forward-only (rollout) routes: grad mode off, as the rollout runs."""
+    with torch.no_grad():
+        yield
+
+
 def _obs(n, seed):
     g = torch.Generator().manual_seed(seed)
     obs = torch.randn(n, nr.OBS_DIM, generator=g) * 0.7
