@@ -244,7 +244,9 @@ int lin_dispatch(const LinArgs& a, int act, int dtype, int out_dtype, hipStream_
                          (!a.bias || bsrl_aligned(a.bias, 16)) &&
                          (!a.res || (a.ldr % 4 == 0 && bsrl_aligned(a.res, 8))) &&
                          (!a.gate || (a.ldgate % 4 == 0 && bsrl_aligned(a.gate, 8)));
-        if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
+        if (vec && bsrl_linear_stream(a, act, dtype, st)) {
+            // many rows, modest K: the weight-resident streaming kernel
+        } else if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
             // large, aligned, 16-bit-out problems: the LDS-tiled kernel
         } else if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);
         else launch16<BF16>(a, act, fast, vec, st);

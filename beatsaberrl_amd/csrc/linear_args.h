@@ -29,3 +29,7 @@ __device__ __forceinline__ int64_t lin_yoff(const LinArgs& a, int64_t row) {
 // LDS-tiled 16-bit kernel for large row counts (linear_tiled.hip); returns false when the
 // shape is outside what it covers (the caller then takes the direct-from-global kernel).
 bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st);
+
+// Weight-resident streaming 16-bit kernel for many rows and K a multiple of 32 up to 1536 (linear_stream.hip);
+// false when the shape is outside what it covers.
+bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st);

@@ -1,0 +1,218 @@
+// Weight-resident streaming linear for many rows and a modest K: y = act(x W^T + b) (+ residual) (* ReLU gate).
+//
+// The policy's token-level Linears have millions of rows and K = 128 .. 1536, i.e. they are HBM streams
+// (x in, y out) with a small weight.  This kernel keeps a block of the weight - MT 16-feature tiles x all
+// of K - resident in LDS in MFMA fragment order for the whole life of a persistent workgroup, and every
+// wave streams its own 32-row tiles of x STRAIGHT from global memory into MFMA B fragments (lane = row,
+// 16 bytes = 8 consecutive k): no LDS staging of activations, no workgroup barrier after the prologue,
+// so the 8 waves of a workgroup drift freely and hide each other's memory latency.  A ring of PD
+// k-chunks of x per wave is always in flight, running ahead across tile boundaries.
+// Per 32-k chunk a wave reads MT fragments (1 KB each) from LDS for 2 MT MFMAs (two 16-row tiles share
+// each fragment): the LDS read path allows ~50 % of MFMA peak, which is above what the HBM stream needs
+// at these K.  Bias, activation, residual and gate are applied in registers (a lane holds 4 consecutive
+// features of one row); the rounded results of 16 rows then cross a per-wave LDS tile so that they leave as
+// 16-byte stores covering whole row segments - written as 32-byte pieces straight from the MFMA layout the
+// same kernel ran at 3.1 TB/s instead of the 5 TB/s a plain copy reaches on this part (measured: the stores
+// alone cost as much as the whole read stream).
+// Column blocks of the same rows are mapped to the same XCD (block id % 8) and walk the rows in the same
+// order, so x is fetched from HBM once and re-read from that XCD's L2 by the other column blocks.
+//
+// Same arithmetic contract as the other linear kernels (fp32 accumulate in a fixed k order, a row's
+// result independent of the batch); the entry point picks by shape.
+#include "linear_args.h"
+
+namespace {
+
+constexpr int ST_THREADS = 512;                  // 8 waves share one resident weight block
+constexpr int ST_ROWS = 32;                      // rows per wave tile (2 MFMA row tiles)
+
+template <typename DT, int KC, int MT, int PD>
+__global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, int act, int nb, int walkers) {
+    static_assert(KC % PD == 0, "the x ring must divide the k chunks");
+    extern __shared__ __attribute__((aligned(16))) uint4 wl[];           // [MT * KC][64] fragments, MT * 16 bias floats, 8 output tiles
+    constexpr int OP = MT * 16 + 8;                                       // output tile row pitch (elements): rows 16 B off a bank period
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    // block id -> (walker, column block): the nb column blocks of one walker share id % 8, i.e. one XCD
+    const int b = blockIdx.x;
+    const int cb = (b >> 3) % nb;
+    const int walker = ((b >> 3) / nb) * 8 + (b & 7);
+    if (walker >= walkers) return;
+    const int m0 = cb * MT * 16;
+    const u16* w = static_cast<const u16*>(a.w);
+    const int K = a.K;
+    // resident weight block: fragment (mt, kc), lane l <- W[m0 + 16 mt + l % 16][32 kc + 8 (l / 16) .. + 7]
+    for (int i = tid; i < MT * KC * 64; i += ST_THREADS) {
+        const int l = i & 63, f = i >> 6, mt = f / KC, kc = f % KC;
+        const int m = m0 + mt * 16 + (l & 15);
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (m < a.M) v = *reinterpret_cast<const uint4*>(w + (int64_t)m * K + kc * 32 + 8 * (l >> 4));
+        wl[i] = v;
+    }
+    float* bl = reinterpret_cast<float*>(wl + MT * KC * 64);
+    u16* ot = reinterpret_cast<u16*>(bl + MT * 16) + wave * (16 * OP);   // this wave's 16-row output tile
+    for (int i = tid; i < MT * 16; i += ST_THREADS) bl[i] = (a.bias && m0 + i < a.M) ? a.bias[m0 + i] : 0.f;
+    __syncthreads();                                                      // the only barrier: waves are on their own from here
+
+    const u16* x = static_cast<const u16*>(a.x);
+    const int64_t ntiles = (a.rows + ST_ROWS - 1) / ST_ROWS;
+    const int64_t stride = (int64_t)walkers * 8;
+    int64_t tile = (int64_t)walker * 8 + wave;
+    if (tile >= ntiles) return;
+    // x ring: slot c % PD holds chunk c of the tile being computed, or of the next tile once consumed
+    uint4 xq[PD][2];
+    auto xrow = [&](int64_t t, int rt) {
+        const int64_t r = t * ST_ROWS + rt * 16 + r16;
+        return (r < a.rows ? r : a.rows - 1) * a.ldx + 8 * g;
+    };
+    int64_t o0 = xrow(tile, 0), o1 = xrow(tile, 1);
+#pragma unroll
+    for (int c = 0; c < PD; ++c) {
+        xq[c][0] = *reinterpret_cast<const uint4*>(x + o0 + c * 32);
+        xq[c][1] = *reinterpret_cast<const uint4*>(x + o1 + c * 32);
+    }
+    const u16* res = static_cast<const u16*>(a.res);
+    const u16* gate = static_cast<const u16*>(a.gate);
+    u16* y = static_cast<u16*>(a.y);
+    for (; tile < ntiles; tile += stride) {
+        const int64_t next = tile + stride;
+        const bool more = next < ntiles;
+        const int64_t n0 = more ? xrow(next, 0) : o0, n1 = more ? xrow(next, 1) : o1;
+        f32x4 acc[MT][2];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) { acc[mt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; acc[mt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const s16x8 x0 = __builtin_bit_cast(s16x8, xq[kc % PD][0]), x1 = __builtin_bit_cast(s16x8, xq[kc % PD][1]);
+            // refill the slot: chunk kc + PD of this tile, or chunk kc + PD - KC of the next one
+            if (kc + PD < KC) {
+                xq[kc % PD][0] = *reinterpret_cast<const uint4*>(x + o0 + (kc + PD) * 32);
+                xq[kc % PD][1] = *reinterpret_cast<const uint4*>(x + o1 + (kc + PD) * 32);
+            } else if (more) {
+                xq[kc % PD][0] = *reinterpret_cast<const uint4*>(x + n0 + (kc + PD - KC) * 32);
+                xq[kc % PD][1] = *reinterpret_cast<const uint4*>(x + n1 + (kc + PD - KC) * 32);
+            }
+            // fragments are read a pair ahead of their MFMAs and no further: without the pins the scheduler hoists
+            // every LDS read of the tile to the top and spills the accumulators
+#pragma unroll
+            for (int mt = 0; mt < MT; mt += 2) {
+                const s16x8 wf0 = __builtin_bit_cast(s16x8, wl[(mt * KC + kc) * 64 + lane]);
+                const s16x8 wf1 = __builtin_bit_cast(s16x8, wl[((mt + 1) * KC + kc) * 64 + lane]);
+                acc[mt][0] = DT::mfma32(wf0, x0, acc[mt][0]);
+                acc[mt][1] = DT::mfma32(wf0, x1, acc[mt][1]);
+                acc[mt + 1][0] = DT::mfma32(wf1, x0, acc[mt + 1][0]);
+                acc[mt + 1][1] = DT::mfma32(wf1, x1, acc[mt + 1][1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // epilogue: lane holds features m0 + 16 mt + 4 g .. + 3 of rows 16 rt + r16
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int64_t row = tile * ST_ROWS + rt * 16 + r16;
+            const bool rv = row < a.rows;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int col = m0 + mt * 16 + 4 * g;
+                const bool on = rv && col < a.M;
+                const float4 bv = *reinterpret_cast<const float4*>(bl + mt * 16 + 4 * g);
+                float o[4] = {acc[mt][rt][0] + bv.x, acc[mt][rt][1] + bv.y, acc[mt][rt][2] + bv.z, acc[mt][rt][3] + bv.w};
+                if (act == BSRL_ACT_RELU) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = fmaxf(o[e], 0.f);
+                } else if (act == BSRL_ACT_GELU) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = gelu_fast(o[e]);
+                }
+                if (res && on) {
+                    const uint2 rv2 = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
+                    o[0] += DT::to_f((u16)(rv2.x & 0xffff)); o[1] += DT::to_f((u16)(rv2.x >> 16));
+                    o[2] += DT::to_f((u16)(rv2.y & 0xffff)); o[3] += DT::to_f((u16)(rv2.y >> 16));
+                }
+                if (gate && on) {
+                    const uint2 gv = *reinterpret_cast<const uint2*>(gate + row * a.ldgate + col);
+                    if (!(DT::to_f((u16)(gv.x & 0xffff)) > 0.f)) o[0] = 0.f;
+                    if (!(DT::to_f((u16)(gv.x >> 16)) > 0.f)) o[1] = 0.f;
+                    if (!(DT::to_f((u16)(gv.y & 0xffff)) > 0.f)) o[2] = 0.f;
+                    if (!(DT::to_f((u16)(gv.y >> 16)) > 0.f)) o[3] = 0.f;
+                }
+                uint2 ov;
+                ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
+                ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                *reinterpret_cast<uint2*>(ot + r16 * OP + mt * 16 + 4 * g) = ov;
+            }
+            // the tile leaves row-major: 16-byte pieces, consecutive lanes on consecutive pieces of a row
+            constexpr int PPR = MT * 2;                                   // 16-byte pieces per row
+#pragma unroll 1
+            for (int c0 = 0; c0 < 16 * PPR; c0 += WAVE) {
+                const int c = c0 + lane;
+                const int r = c / PPR, pc = c % PPR;
+                const int64_t orow = tile * ST_ROWS + rt * 16 + r;
+                if (c < 16 * PPR && orow < a.rows && m0 + pc * 8 < a.M)
+                    *reinterpret_cast<uint4*>(y + lin_yoff(a, orow) + m0 + pc * 8) = *reinterpret_cast<const uint4*>(ot + r * OP + pc * 8);
+            }
+        }
+        o0 = n0; o1 = n1;
+    }
+}
+
+int device_cus() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        return n;
+    }();
+    return cus;
+}
+
+template <typename DT, int KC, int MT, int PD>
+bool launch(const LinArgs& a, int act, hipStream_t st) {
+    const size_t lds = (size_t)MT * KC * 1024 + (size_t)MT * 16 * sizeof(float) + (size_t)8 * 16 * (MT * 16 + 8) * sizeof(u16);
+    auto kern = linear_stream_kernel<DT, KC, MT, PD>;
+    // workgroups resident per CU (LDS and registers), 0 = this instantiation cannot run here
+    static const int per_cu = [&] {
+        int n = 0;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, ST_THREADS, lds) != hipSuccess) return 0;
+        return n;
+    }();
+    if (per_cu < 1) return false;
+    const int nb = (a.M + MT * 16 - 1) / (MT * 16);
+    const int64_t ntiles = (a.rows + ST_ROWS - 1) / ST_ROWS;
+    // every workgroup must be resident at once (the rows are split statically); the walkers of a column block come
+    // in whole groups of 8 block ids (one per XCD)
+    const int64_t slots = (int64_t)device_cus() * per_cu;
+    int64_t walkers = slots / nb / 8 * 8;
+    if (walkers < 8) return false;
+    const int64_t need = ((ntiles + 7) / 8 + 7) / 8 * 8;
+    if (walkers > need) walkers = need;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(walkers * nb)), dim3(ST_THREADS), lds, st, a, act, nb, (int)walkers);
+    return true;
+}
+
+template <typename DT>
+bool dispatch(const LinArgs& a, int act, hipStream_t st) {
+    switch (a.K / 32) {
+        case 4: return launch<DT, 4, 8, 4>(a, act, st);
+        case 6: return launch<DT, 6, 12, 3>(a, act, st);
+        case 8: return launch<DT, 8, 8, 8>(a, act, st);
+        case 12: return launch<DT, 12, 8, 6>(a, act, st);
+        case 16: return launch<DT, 16, 4, 8>(a, act, st);
+        case 24: return launch<DT, 24, 4, 8>(a, act, st);
+        case 32: return launch<DT, 32, 2, 8>(a, act, st);
+        case 48: return launch<DT, 48, 2, 8>(a, act, st);
+        default: return false;
+    }
+}
+
+}  // namespace
+
+bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st) {
+    // many rows, K a supported multiple of 32, 16-bit in and out, 8-byte aligned rows everywhere
+    if (a.out_f32 || a.y2 || a.rows < 8192 || a.K % 32 != 0 || a.M % 8 != 0) return false;
+    if (a.ldx % 8 != 0 || !bsrl_aligned(a.x, 16) || !bsrl_aligned(a.w, 16)) return false;
+    if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16)) return false;
+    if (a.res && (a.ldr % 4 != 0 || !bsrl_aligned(a.res, 8))) return false;
+    if (a.gate && (a.ldgate % 4 != 0 || !bsrl_aligned(a.gate, 8))) return false;
+    if (a.bias && !bsrl_aligned(a.bias, 4)) return false;
+    return dtype == BSRL_F16 ? dispatch<F16>(a, act, st) : dispatch<BF16>(a, act, st);
+}

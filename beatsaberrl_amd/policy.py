@@ -145,6 +145,24 @@ def note_geo(notes, sabers, z_asinh, flux, z_off):
     return torch.cat(base + blade, -1)
 
 
+def hl_target(v, centers, sigma: float):
+    """HL-Gauss target (reference python/policy.py:759-773): the mass of N(v, sigma^2) inside each of the K
+    equally spaced histogram bins, v clamped into the support, rows renormalised to 1.  v (B,) -> (B, K)."""
+    v = v.float()
+    width = centers[1] - centers[0]
+    edges = torch.cat([centers[:1] - 0.5 * width, centers + 0.5 * width])
+    v = v.clamp(edges[0], edges[-1])
+    cdf = 0.5 * (1.0 + torch.erf((edges.unsqueeze(0) - v.unsqueeze(1)) / (sigma * math.sqrt(2.0))))
+    p = cdf[:, 1:] - cdf[:, :-1]
+    return p / p.sum(-1, keepdim=True)
+
+
+def hl_loss(logits, v_tgt, centers, sigma: float):
+    """Cross-entropy between the critic's bin distribution and the HL-Gauss target, batch mean
+    (reference python/policy.py:776-781); logits (B, K) fp32 = `policy._value_logits` of the update forward."""
+    return -(hl_target(v_tgt, centers, sigma) * F.log_softmax(logits.float(), dim=-1)).sum(-1).mean()
+
+
 class Block(nn.Module):
     """Pre-LN transformer block; parameters as the reference's Block
     (python/policy.py:492-522): ln_attn, q/k/v/out_proj, ln_ffn, ffn.{0,2}."""

@@ -521,3 +521,44 @@ def test_attention_backward(dtype, T, TQ, H, dh, mask):
         assert torch.equal(dk[dead], torch.zeros_like(dk[dead])) and torch.equal(dv[dead], torch.zeros_like(dv[dead]))
     dq2, dk2, dv2 = ops.attn_bwd(q, k, v, dout, H, **kw)      # fresh contiguous outputs, same bits
     assert torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
+
+
+# ---------------------------------------------------------------- weight-resident streaming linear
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,K,M", [(8192, 128, 128), (8200, 128, 384), (9001, 192, 192), (8193, 192, 576), (8192, 192, 776),
+                                      (8300, 256, 1024), (8192, 384, 384), (8207, 512, 136), (8192, 768, 192),
+                                      (8192, 1024, 256), (8199, 1536, 384)])
+@pytest.mark.parametrize("act,use_res,use_bias", [(None, False, True), ("gelu", False, True), ("relu", True, False), (None, True, True)])
+def test_linear_many_rows_take_the_streaming_kernel(dtype, rows, K, M, act, use_res, use_bias):
+    """rows >= 8192 with K a multiple of 32 up to 1536 run the weight-resident streaming kernel (every K chunk
+    count it is built for, column blocks that overhang M, ragged last row tile): the same closed form, and the
+    same BITS as the direct-from-global kernel on row slices (all accumulate k in the same order)."""
+    x = _rand(rows, K, dtype=dtype, seed=rows)
+    w = _rand(M, K, dtype=dtype, seed=K + M, scale=1 / math.sqrt(K))
+    b = _rand(M, seed=M) if use_bias else None
+    res = _rand(rows, M, dtype=dtype, seed=7) if use_res else None
+    y = ops.linear(x, w, b, act=act, residual=res)
+    ref = _lin_ref(x, w, b if use_bias else torch.zeros(M, device=DEV), act, res)
+    assert (y.double() - ref).abs().max().item() <= 1.2 * EPS16[dtype] * ref.abs().max().item()
+    for lo, hi in ((0, 300), (rows // 2 - 5, rows // 2 + 200), (rows - 257, rows)):
+        small = ops.linear(x[lo:hi], w, b, act=act, residual=None if res is None else res[lo:hi])
+        assert torch.equal(small, y[lo:hi])
+
+
+def test_streaming_linear_gate_and_token_slice_output():
+    """The ReLU gate and the grouped (token-slice) output through the streaming kernel."""
+    rows, K, M = 8192, 192, 768
+    g = _rand(rows, K, dtype=torch.float16, seed=1)
+    wt = _rand(M, K, dtype=torch.float16, seed=2, scale=K ** -0.5)
+    hid = torch.relu(_rand(rows, M, dtype=torch.float16, seed=3))
+    out = ops.linear_gated(g, wt, hid)
+    assert torch.equal(out[:500], ops.linear_gated(g[:500], wt, hid[:500]))
+    assert torch.equal(out[hid <= 0], torch.zeros_like(out[hid <= 0]))
+    N, G, T = 512, 24, 29
+    x = _rand(N * G, 128, dtype=torch.float16, seed=4)
+    w = _rand(192, 128, dtype=torch.float16, seed=5, scale=0.09)
+    b = _rand(192, seed=6)
+    stream = torch.full((N, T, 192), 7.0, device=DEV, dtype=torch.float16)
+    ops.linear(x, w, b, act="relu", out=stream[:, 5:])
+    assert torch.equal(stream[:, 5:].reshape(N * G, 192), ops.linear(x, w, b, act="relu"))
+    assert torch.equal(stream[:, :5], torch.full_like(stream[:, :5], 7.0))
