@@ -75,20 +75,31 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
     u16* Ps = Vs + TP * DHP;
     u16* dSs = Ps + 16 * PP;
 
-    // stage the pair's q, dO (TQ rows) and k, v (T rows), zero rows up to the tile edge
-    auto stage = [&](u16* dst, const void* src, int64_t bs, int64_t rs, int nrows, int prows) {
-        const u16* sp = static_cast<const u16*>(src) + b * bs + h * DH;
-        for (int c = lane; c < prows * (DH / 8); c += WAVE) {
-            const int row = c / (DH / 8), part = c % (DH / 8);
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (row < nrows) val = *reinterpret_cast<const uint4*>(sp + (int64_t)row * rs + part * 8);
-            *reinterpret_cast<uint4*>(dst + row * DHP + part * 8) = val;
+    // stage the pair's q, dO (TQ rows) and k, v (T rows), zero rows up to the tile edge.  All global loads are
+    // issued before the first LDS write: one memory round trip for the four matrices instead of one per piece.
+    constexpr int PPR = DH / 8;                                     // 16-byte pieces per row
+    constexpr int NIT = (kMaxKT * 16 * PPR + WAVE - 1) / WAVE;      // pieces per lane and matrix, at most
+    uint4 buf[4][NIT];
+    const u16* srcs[4] = {static_cast<const u16*>(a.q) + b * a.q_bs + h * DH, static_cast<const u16*>(a.dout) + b * a.do_bs + h * DH,
+                          static_cast<const u16*>(a.k) + b * a.k_bs + h * DH, static_cast<const u16*>(a.v) + b * a.v_bs + h * DH};
+    const int64_t rss[4] = {a.q_rs, a.do_rs, a.k_rs, a.v_rs};
+    const int nrows[4] = {TQ, TQ, T, T}, prows[4] = {TQP, TQP, TP, TP};
+    u16* dsts[4] = {Qs, dOs, Ks, Vs};
+#pragma unroll
+    for (int mtx = 0; mtx < 4; ++mtx)
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int c = it * WAVE + lane, row = c / PPR, part = c % PPR;
+            buf[mtx][it] = make_uint4(0, 0, 0, 0);
+            if (row < nrows[mtx]) buf[mtx][it] = *reinterpret_cast<const uint4*>(srcs[mtx] + (int64_t)row * rss[mtx] + part * 8);
         }
-    };
-    stage(Qs, a.q, a.q_bs, a.q_rs, TQ, TQP);
-    stage(dOs, a.dout, a.do_bs, a.do_rs, TQ, TQP);
-    stage(Ks, a.k, a.k_bs, a.k_rs, T, TP);
-    stage(Vs, a.v, a.v_bs, a.v_rs, T, TP);
+#pragma unroll
+    for (int mtx = 0; mtx < 4; ++mtx)
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int c = it * WAVE + lane, row = c / PPR, part = c % PPR;
+            if (row < prows[mtx]) *reinterpret_cast<uint4*>(dsts[mtx] + row * DHP + part * 8) = buf[mtx][it];
+        }
 
     // additive bias / validity of keys 16 kt + 4 g + e, as the forward applies them
     float kb[kMaxKT][4];

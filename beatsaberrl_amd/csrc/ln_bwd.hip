@@ -129,20 +129,23 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(const void* __restrict__ x,
     }
 }
 
-// dw / db / dbb[col] = sum over the G partial rows, 4 interleaved running sums folded in a fixed order
+// dw / db / dbb[col] = sum over the G partial rows: a workgroup owns 16 columns, its 16 row slices run interleaved
+// sums that are folded in slice order (a fixed order: reproducible)
 __global__ __launch_bounds__(256) void ln_bwd_reduce_kernel(const float* __restrict__ part, int G, int nq, int d,
                                                             float* __restrict__ dw, float* __restrict__ db,
                                                             float* __restrict__ dbb) {
-    __shared__ float sm[4][64];
-    const int cl = threadIdx.x & 63, k = threadIdx.x >> 6;
-    const int q = blockIdx.y, col = blockIdx.x * 64 + cl;
+    __shared__ float sm[16][17];
+    const int cl = threadIdx.x & 15, k = threadIdx.x >> 4;
+    const int q = blockIdx.y, col = blockIdx.x * 16 + cl;
     float t = 0.f;
     if (col < d)
-        for (int gi = k; gi < G; gi += 4) t += part[((int64_t)gi * nq + q) * d + col];
+        for (int gi = k; gi < G; gi += 16) t += part[((int64_t)gi * nq + q) * d + col];
     sm[k][cl] = t;
     __syncthreads();
     if (k == 0 && col < d) {
-        const float v = (sm[0][cl] + sm[1][cl]) + (sm[2][cl] + sm[3][cl]);
+        float v = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v += sm[j][cl];
         (q == 0 ? dw : q == 1 ? db : dbb)[col] = v;
     }
 }
@@ -226,7 +229,7 @@ extern "C" int bsrl_ln_bwd(const void* x, const void* dy, const float* weight, c
     else if (dtype == BSRL_F16) rc = dispatch<F16>(x, dy, weight, mean, rstd, gx, dx, part, dbb != nullptr, rows, d, &grid, st);
     else rc = dispatch<BF16>(x, dy, weight, mean, rstd, gx, dx, part, dbb != nullptr, rows, d, &grid, st);
     if (rc != BSRL_OK) return rc;
-    hipLaunchKernelGGL(ln_bwd_reduce_kernel, dim3((unsigned)((d + 63) / 64), nq), dim3(256), 0, st, part, grid, nq, (int)d, dw, db, dbb);
+    hipLaunchKernelGGL(ln_bwd_reduce_kernel, dim3((unsigned)((d + 15) / 16), nq), dim3(256), 0, st, part, grid, nq, (int)d, dw, db, dbb);
     BSRL_CHECK_LAUNCH("bsrl_ln_bwd");
     return BSRL_OK;
 }
