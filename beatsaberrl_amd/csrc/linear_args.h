@@ -30,6 +30,6 @@ __device__ __forceinline__ int64_t lin_yoff(const LinArgs& a, int64_t row) {
 // shape is outside what it covers (the caller then takes the direct-from-global kernel).
 bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st);
 
-// Weight-resident streaming 16-bit kernel for many rows and K a multiple of 32 up to 1536 (linear_stream.hip);
+// Weight-resident streaming 16-bit kernel for many rows and K = 128 / 192 / 256 / 384 (linear_stream.hip);
 // false when the shape is outside what it covers.
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st);

@@ -1,7 +1,8 @@
 // Weight-resident streaming linear for many rows and a modest K: y = act(x W^T + b) (+ residual) (* ReLU gate).
 //
-// The policy's token-level Linears have millions of rows and K = 128 .. 1536, i.e. they are HBM streams
-// (x in, y out) with a small weight.  This kernel keeps a block of the weight - MT 16-feature tiles x all
+// The policy's token-level Linears have millions of rows and K = 128 .. 256 on their input side, i.e. they are
+// HBM streams (x in, y out) with a small weight.  (At larger K the resident block shrinks to a few 16-feature tiles
+// and x would be re-read once per column block: those shapes stay on the LDS-tiled kernel.)  This kernel keeps a block of the weight - MT 16-feature tiles x all
 // of K - resident in LDS in MFMA fragment order for the whole life of a persistent workgroup, and every
 // wave streams its own 32-row tiles of x STRAIGHT from global memory into MFMA B fragments (lane = row,
 // 16 bytes = 8 consecutive k): no LDS staging of activations, no workgroup barrier after the prologue,
@@ -195,11 +196,7 @@ bool dispatch(const LinArgs& a, int act, hipStream_t st) {
         case 4: return launch<DT, 4, 8, 4>(a, act, st);
         case 6: return launch<DT, 6, 12, 3>(a, act, st);
         case 8: return launch<DT, 8, 8, 8>(a, act, st);
-        case 12: return launch<DT, 12, 8, 6>(a, act, st);
-        case 16: return launch<DT, 16, 4, 8>(a, act, st);
-        case 24: return launch<DT, 24, 4, 8>(a, act, st);
-        case 32: return launch<DT, 32, 2, 8>(a, act, st);
-        case 48: return launch<DT, 48, 2, 8>(a, act, st);
+        case 12: return a.M <= 256 ? launch<DT, 12, 8, 6>(a, act, st) : false;
         default: return false;
     }
 }
@@ -207,7 +204,7 @@ bool dispatch(const LinArgs& a, int act, hipStream_t st) {
 }  // namespace
 
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st) {
-    // many rows, K a supported multiple of 32, 16-bit in and out, 8-byte aligned rows everywhere
+    // many rows, K = 128 / 192 / 256 (384 for narrow outputs), 16-bit in and out, 16-byte aligned rows
     if (a.out_f32 || a.y2 || a.rows < 8192 || a.K % 32 != 0 || a.M % 8 != 0) return false;
     if (a.ldx % 8 != 0 || !bsrl_aligned(a.x, 16) || !bsrl_aligned(a.w, 16)) return false;
     if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16)) return false;
