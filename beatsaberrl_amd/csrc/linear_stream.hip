@@ -4,10 +4,14 @@
 // HBM streams (x in, y out) with a small weight.  (At larger K the resident block shrinks to a few 16-feature tiles
 // and x would be re-read once per column block: those shapes stay on the LDS-tiled kernel.)  This kernel keeps a block of the weight - MT 16-feature tiles x all
 // of K - resident in LDS in MFMA fragment order for the whole life of a persistent workgroup, and every
-// wave streams its own 32-row tiles of x STRAIGHT from global memory into MFMA B fragments (lane = row,
-// 16 bytes = 8 consecutive k): no LDS staging of activations, no workgroup barrier after the prologue,
-// so the 8 waves of a workgroup drift freely and hide each other's memory latency.  A ring of PD
-// k-chunks of x per wave is always in flight, running ahead across tile boundaries.
+// wave streams its own 32-row tiles of x: whole rows, consecutive lanes on consecutive 16-byte pieces, one tile
+// ahead of the MFMAs, turned into B fragments through a small per-wave LDS tile.  (Loading the fragments straight
+// from global memory - lane = row, the 4 lanes of a row 16 lanes apart - touches 16 rows x 64 B per wave
+// instruction: with everything but the loads cut out the kernel read at 3.65 TB/s that way and reads at 4.8 TB/s
+// with whole-row loads; a plain 16-byte-per-lane read reaches 6.3 TB/s on this part.)  The register arrays
+// that live across the tile loop are native vector types: arrays of HIP's uint4 class stayed in scratch.  There is
+// no workgroup barrier after the prologue, so the 8 waves of a workgroup drift freely and hide each other's
+// memory latency.
 // Per 32-k chunk a wave reads MT fragments (1 KB each) from LDS for 2 MT MFMAs (two 16-row tiles share
 // each fragment): the LDS read path allows ~50 % of MFMA peak, which is above what the HBM stream needs
 // at these K.  Bias, activation, residual and gate are applied in registers (a lane holds 4 consecutive
@@ -26,12 +30,15 @@ namespace {
 
 constexpr int ST_THREADS = 512;                  // 8 waves share one resident weight block
 constexpr int ST_ROWS = 32;                      // rows per wave tile (2 MFMA row tiles)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <typename DT, int KC, int MT, int PD>
+template <typename DT, int KC, int MT>
 __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, int act, int nb, int walkers) {
-    static_assert(KC % PD == 0, "the x ring must divide the k chunks");
-    extern __shared__ __attribute__((aligned(16))) uint4 wl[];           // [MT * KC][64] fragments, MT * 16 bias floats, 8 output tiles
-    constexpr int OP = MT * 16 + 8;                                       // output tile row pitch (elements): rows 16 B off a bank period
+    extern __shared__ __attribute__((aligned(16))) uint4 wl[];           // [MT * KC][64] fragments, MT * 16 bias floats, 8 wave tiles
+    constexpr int KE = KC * 32;                                           // K
+    constexpr int TP = (KE > MT * 16 ? KE : MT * 16) + 8;                 // wave tile row pitch (elements): rows 16 B off a bank period
+    constexpr int PPR = KE / 8;                                           // 16-byte pieces per x row
+    constexpr int NLD = (16 * PPR + WAVE - 1) / WAVE;                     // pieces per lane for 16 rows of x
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
     // block id -> (walker, column block): the nb column blocks of one walker share id % 8, i.e. one XCD
@@ -41,17 +48,16 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
     if (walker >= walkers) return;
     const int m0 = cb * MT * 16;
     const u16* w = static_cast<const u16*>(a.w);
-    const int K = a.K;
     // resident weight block: fragment (mt, kc), lane l <- W[m0 + 16 mt + l % 16][32 kc + 8 (l / 16) .. + 7]
     for (int i = tid; i < MT * KC * 64; i += ST_THREADS) {
         const int l = i & 63, f = i >> 6, mt = f / KC, kc = f % KC;
         const int m = m0 + mt * 16 + (l & 15);
         uint4 v = make_uint4(0, 0, 0, 0);
-        if (m < a.M) v = *reinterpret_cast<const uint4*>(w + (int64_t)m * K + kc * 32 + 8 * (l >> 4));
+        if (m < a.M) v = *reinterpret_cast<const uint4*>(w + (int64_t)m * KE + kc * 32 + 8 * (l >> 4));
         wl[i] = v;
     }
     float* bl = reinterpret_cast<float*>(wl + MT * KC * 64);
-    u16* ot = reinterpret_cast<u16*>(bl + MT * 16) + wave * (16 * OP);   // this wave's 16-row output tile
+    u16* wt = reinterpret_cast<u16*>(bl + MT * 16) + wave * (16 * TP);   // this wave's 16-row tile: x on the way in, y on the way out
     for (int i = tid; i < MT * 16; i += ST_THREADS) bl[i] = (a.bias && m0 + i < a.M) ? a.bias[m0 + i] : 0.f;
     __syncthreads();                                                      // the only barrier: waves are on their own from here
 
@@ -60,39 +66,46 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
     const int64_t stride = (int64_t)walkers * 8;
     int64_t tile = (int64_t)walker * 8 + wave;
     if (tile >= ntiles) return;
-    // x ring: slot c % PD holds chunk c of the tile being computed, or of the next tile once consumed
-    uint4 xq[PD][2];
-    auto xrow = [&](int64_t t, int rt) {
-        const int64_t r = t * ST_ROWS + rt * 16 + r16;
-        return (r < a.rows ? r : a.rows - 1) * a.ldx + 8 * g;
-    };
-    int64_t o0 = xrow(tile, 0), o1 = xrow(tile, 1);
-#pragma unroll
-    for (int c = 0; c < PD; ++c) {
-        xq[c][0] = *reinterpret_cast<const uint4*>(x + o0 + c * 32);
-        xq[c][1] = *reinterpret_cast<const uint4*>(x + o1 + c * 32);
+    // x arrives as whole rows: consecutive lanes load consecutive 16-byte pieces (a wave instruction = 1 KB of
+    // contiguous memory when rows are dense), one 32-row tile ahead of the MFMAs
+    u32x4 pa[NLD], pb[NLD];                                               // rows 0..15 and 16..31 of the tile in flight
+#define ST_FETCH(t)                                                                                                   \
+    _Pragma("unroll") for (int it = 0; it < NLD; ++it) {                                                               \
+        const int p = it * WAVE + lane, r = p / PPR, part = p % PPR;                                                  \
+        int64_t ra = (t) * ST_ROWS + r, rb = ra + 16;                                                                 \
+        ra = ra < a.rows ? ra : a.rows - 1;                                                                           \
+        rb = rb < a.rows ? rb : a.rows - 1;                                                                           \
+        pa[it] = *reinterpret_cast<const u32x4*>(x + ra * a.ldx + part * 8);                                          \
+        pb[it] = *reinterpret_cast<const u32x4*>(x + rb * a.ldx + part * 8);                                          \
     }
+    ST_FETCH(tile)
     const u16* res = static_cast<const u16*>(a.res);
     const u16* gate = static_cast<const u16*>(a.gate);
     u16* y = static_cast<u16*>(a.y);
     for (; tile < ntiles; tile += stride) {
-        const int64_t next = tile + stride;
-        const bool more = next < ntiles;
-        const int64_t n0 = more ? xrow(next, 0) : o0, n1 = more ? xrow(next, 1) : o1;
+        // rows -> B fragments through the wave tile: lane (r16, g) of chunk kc holds x[16 h + r16][32 kc + 8 g .. + 7]
+        u32x4 xf0[KC], xf1[KC];
+#pragma unroll
+        for (int it = 0; it < NLD; ++it) {
+            const int p = it * WAVE + lane;
+            if (NLD * WAVE == 16 * PPR || p < 16 * PPR) *reinterpret_cast<u32x4*>(wt + (p / PPR) * TP + (p % PPR) * 8) = pa[it];
+        }
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) xf0[kc] = *reinterpret_cast<const u32x4*>(wt + r16 * TP + kc * 32 + 8 * g);
+#pragma unroll
+        for (int it = 0; it < NLD; ++it) {
+            const int p = it * WAVE + lane;
+            if (NLD * WAVE == 16 * PPR || p < 16 * PPR) *reinterpret_cast<u32x4*>(wt + (p / PPR) * TP + (p % PPR) * 8) = pb[it];
+        }
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) xf1[kc] = *reinterpret_cast<const u32x4*>(wt + r16 * TP + kc * 32 + 8 * g);
+        ST_FETCH(tile + stride)                                         // rows past the end clamp to the last row: always a valid load
         f32x4 acc[MT][2];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) { acc[mt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; acc[mt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc) {
-            const s16x8 x0 = __builtin_bit_cast(s16x8, xq[kc % PD][0]), x1 = __builtin_bit_cast(s16x8, xq[kc % PD][1]);
-            // refill the slot: chunk kc + PD of this tile, or chunk kc + PD - KC of the next one
-            if (kc + PD < KC) {
-                xq[kc % PD][0] = *reinterpret_cast<const uint4*>(x + o0 + (kc + PD) * 32);
-                xq[kc % PD][1] = *reinterpret_cast<const uint4*>(x + o1 + (kc + PD) * 32);
-            } else if (more) {
-                xq[kc % PD][0] = *reinterpret_cast<const uint4*>(x + n0 + (kc + PD - KC) * 32);
-                xq[kc % PD][1] = *reinterpret_cast<const uint4*>(x + n1 + (kc + PD - KC) * 32);
-            }
+            const s16x8 x0 = __builtin_bit_cast(s16x8, xf0[kc]), x1 = __builtin_bit_cast(s16x8, xf1[kc]);
             // fragments are read a pair ahead of their MFMAs and no further: without the pins the scheduler hoists
             // every LDS read of the tile to the top and spills the accumulators
 #pragma unroll
@@ -139,22 +152,22 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
                 uint2 ov;
                 ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
                 ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
-                *reinterpret_cast<uint2*>(ot + r16 * OP + mt * 16 + 4 * g) = ov;
+                *reinterpret_cast<uint2*>(wt + r16 * TP + mt * 16 + 4 * g) = ov;
             }
             // the tile leaves row-major: 16-byte pieces, consecutive lanes on consecutive pieces of a row
-            constexpr int PPR = MT * 2;                                   // 16-byte pieces per row
+            constexpr int OPR = MT * 2;                                   // 16-byte pieces per output row
 #pragma unroll 1
-            for (int c0 = 0; c0 < 16 * PPR; c0 += WAVE) {
+            for (int c0 = 0; c0 < 16 * OPR; c0 += WAVE) {
                 const int c = c0 + lane;
-                const int r = c / PPR, pc = c % PPR;
+                const int r = c / OPR, pc = c % OPR;
                 const int64_t orow = tile * ST_ROWS + rt * 16 + r;
-                if (c < 16 * PPR && orow < a.rows && m0 + pc * 8 < a.M)
-                    *reinterpret_cast<uint4*>(y + lin_yoff(a, orow) + m0 + pc * 8) = *reinterpret_cast<const uint4*>(ot + r * OP + pc * 8);
+                if (c < 16 * OPR && orow < a.rows && m0 + pc * 8 < a.M)
+                    *reinterpret_cast<uint4*>(y + lin_yoff(a, orow) + m0 + pc * 8) = *reinterpret_cast<const uint4*>(wt + r * TP + pc * 8);
             }
         }
-        o0 = n0; o1 = n1;
     }
 }
+#undef ST_FETCH
 
 int device_cus() {
     static const int cus = [] {
@@ -165,10 +178,11 @@ int device_cus() {
     return cus;
 }
 
-template <typename DT, int KC, int MT, int PD>
+template <typename DT, int KC, int MT>
 bool launch(const LinArgs& a, int act, hipStream_t st) {
-    const size_t lds = (size_t)MT * KC * 1024 + (size_t)MT * 16 * sizeof(float) + (size_t)8 * 16 * (MT * 16 + 8) * sizeof(u16);
-    auto kern = linear_stream_kernel<DT, KC, MT, PD>;
+    constexpr int TP = (KC * 32 > MT * 16 ? KC * 32 : MT * 16) + 8;
+    const size_t lds = (size_t)MT * KC * 1024 + (size_t)MT * 16 * sizeof(float) + (size_t)8 * 16 * TP * sizeof(u16);
+    auto kern = linear_stream_kernel<DT, KC, MT>;
     // workgroups resident per CU (LDS and registers), 0 = this instantiation cannot run here
     static const int per_cu = [&] {
         int n = 0;
@@ -193,10 +207,9 @@ bool launch(const LinArgs& a, int act, hipStream_t st) {
 template <typename DT>
 bool dispatch(const LinArgs& a, int act, hipStream_t st) {
     switch (a.K / 32) {
-        case 4: return launch<DT, 4, 8, 4>(a, act, st);
-        case 6: return launch<DT, 6, 12, 3>(a, act, st);
-        case 8: return launch<DT, 8, 8, 8>(a, act, st);
-        case 12: return a.M <= 256 ? launch<DT, 12, 8, 6>(a, act, st) : false;
+        case 4: return launch<DT, 4, 8>(a, act, st);
+        case 6: return launch<DT, 6, 12>(a, act, st);
+        case 8: return launch<DT, 8, 8>(a, act, st);
         default: return false;
     }
 }
@@ -204,7 +217,7 @@ bool dispatch(const LinArgs& a, int act, hipStream_t st) {
 }  // namespace
 
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st) {
-    // many rows, K = 128 / 192 / 256 (384 for narrow outputs), 16-bit in and out, 16-byte aligned rows
+    // many rows, K = 128 / 192 / 256, 16-bit in and out, 16-byte aligned rows
     if (a.out_f32 || a.y2 || a.rows < 8192 || a.K % 32 != 0 || a.M % 8 != 0) return false;
     if (a.ldx % 8 != 0 || !bsrl_aligned(a.x, 16) || !bsrl_aligned(a.w, 16)) return false;
     if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16)) return false;
