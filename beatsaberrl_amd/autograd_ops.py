@@ -62,6 +62,25 @@ class LnFn(torch.autograd.Function):
         return dx, dw, db, None
 
 
+class LnResFn(torch.autograd.Function):
+    """(x, LayerNorm(x)) for a pre-LN residual stream: x is handed back as it came so that the residual branch
+    hangs off this node, and the backward forms grad(x) + LN's dx in ln_bwd's store loop (one rounding, no
+    separate add pass over the stream) - the saving the reference takes through `_LnAddFn`
+    (python/fused_ln.py:71-108) on its deferred-residual block layout."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        y, mean, rstd = ops.ln_fwd(x, weight.detach(), bias.detach(), eps, want_stats=True)
+        ctx.save_for_backward(x, weight, mean, rstd)
+        return x.view_as(x), y
+
+    @staticmethod
+    def backward(ctx, gx, gy):
+        x, weight, mean, rstd = ctx.saved_tensors
+        dx, dw, db = ops.ln_bwd(x, gy.contiguous(), weight.detach(), mean, rstd, gx=gx.contiguous())
+        return dx, dw, db, None
+
+
 class LnAddFn(torch.autograd.Function):
     """(x, y) = (a + b (+ b_bias), LayerNorm(x)) (reference python/fused_ln.py:71-108): d/da == d/db ==
     grad(x) + LN's dx, formed in one rounding inside ln_bwd; d/d(b_bias) = its column sums."""

@@ -19,6 +19,9 @@
 // S chunks per tile; split s of every tile is mapped to consecutive block ids of ONE XCD (id % 8),
 // so the tiles that re-read the same dy / x rows share that XCD's L2.  Partials land in the
 // caller's workspace and a second kernel folds them in split order (reproducible, no atomics).
+// One step of both operands is prefetched in registers; a 3-step register ring was measured and dropped: at 206
+// VGPRs two workgroups fit a CU instead of four and the kernel ran 1.5 - 1.8x slower - occupancy, not prefetch
+// depth, is what hides the step latency here.
 #include "bsrl_common.h"
 
 namespace {

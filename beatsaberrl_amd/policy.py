@@ -40,7 +40,7 @@ import torch.nn.functional as F
 from . import fp16_linear as _fl
 from . import obs_layout as L
 from . import ops
-from .autograd_ops import AttnPackedFn, AttnQKVFn, ChainFn, LinearFn
+from .autograd_ops import AttnPackedFn, AttnQKVFn, ChainFn, LinearFn, LnResFn
 from .fused_ln import FusedLayerNorm
 
 OBS_DIM = L.OBS_DIM
@@ -231,7 +231,8 @@ def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False):
     """Block.forward under autograd (update path): the same kernels in the same order as the per-op
     rollout route without the fused FFN, each paired with its backward; returns x_out (, v)."""
     d = self.d
-    h = self.ln_attn(x)
+    # each LayerNorm hands the stream back with it: the residual branch's gradient joins LN's inside ln_bwd
+    x, h = LnResFn.apply(x.contiguous(), self.ln_attn.weight, self.ln_attn.bias, self.ln_attn.eps)
     if n_queries:
         kv = _packed_t([self.k_proj, self.v_proj], h)
         v = kv[..., d:]
@@ -247,7 +248,8 @@ def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False):
             qkv = torch.cat([qkv[..., :2 * d], torch.addcmul(v * self.vres_a, v0, self.vres_b).to(v.dtype)], -1)
         att = AttnPackedFn.apply(qkv, attn_bias, self.n_heads)
     x = _lin_t(self.out_proj, att, residual=x)
-    x = _seq_t(self.ffn, self.ln_ffn(x), residual=x)
+    x, h2 = LnResFn.apply(x, self.ln_ffn.weight, self.ln_ffn.bias, self.ln_ffn.eps)
+    x = _seq_t(self.ffn, h2, residual=x)
     return (x, v) if want_v else x
 
 
