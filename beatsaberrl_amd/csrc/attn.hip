@@ -54,12 +54,21 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnArgs a) {
     const u16* vp = static_cast<const u16*>(a.v) + b * a.v_bs + h * DH;
     u16* myv = vs[wave];
 
-    // V rows -> LDS (zero rows beyond T: their probabilities are 0, but 0 * junk must stay 0)
-    for (int c = lane; c < nkt * 16 * (DH / 8); c += WAVE) {
-        const int row = c / (DH / 8), part = c % (DH / 8);
-        uint4 val = make_uint4(0, 0, 0, 0);
-        if (row < T) val = *reinterpret_cast<const uint4*>(vp + (int64_t)row * a.v_rs + part * 8);
-        *reinterpret_cast<uint4*>(myv + row * VLD + part * 8) = val;
+    // V rows -> LDS (zero rows beyond T: their probabilities are 0, but 0 * junk must stay 0); every load is
+    // issued before the first LDS write, so the staging costs one memory round trip, not one per piece
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int VPR = DH / 8, VNIT = (kMaxKT * 16 * VPR + WAVE - 1) / WAVE;
+    u32x4 vbuf[VNIT];
+#pragma unroll
+    for (int it = 0; it < VNIT; ++it) {
+        const int c = it * WAVE + lane, row = c / VPR, part = c % VPR;
+        vbuf[it] = (u32x4){0u, 0u, 0u, 0u};
+        if (row < T) vbuf[it] = *reinterpret_cast<const u32x4*>(vp + (int64_t)row * a.v_rs + part * 8);
+    }
+#pragma unroll
+    for (int it = 0; it < VNIT; ++it) {
+        const int c = it * WAVE + lane, row = c / VPR, part = c % VPR;
+        if (row < nkt * 16) *reinterpret_cast<u32x4*>(myv + row * VLD + part * 8) = vbuf[it];
     }
     // K fragments (A operand): lane (key = r16, k-block g)
     s16x8 kf[kMaxKT]; s16x4 kf2[kMaxKT];
