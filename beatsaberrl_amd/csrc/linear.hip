@@ -246,6 +246,8 @@ int lin_dispatch(const LinArgs& a, int act, int dtype, int out_dtype, hipStream_
                          (!a.gate || (a.ldgate % 4 == 0 && bsrl_aligned(a.gate, 8)));
         if (vec && bsrl_linear_stream(a, act, dtype, st)) {
             // many rows, modest K: the weight-resident streaming kernel
+        } else if (vec && bsrl_linear_ring(a, act, dtype, st)) {
+            // large, aligned, 16-bit-out problems with K a multiple of 32: operands straight into an LDS ring
         } else if (vec && bsrl_linear_tiled(a, act, dtype, st)) {
             // large, aligned, 16-bit-out problems: the LDS-tiled kernel
         } else if (dtype == BSRL_F16) launch16<F16>(a, act, fast, vec, st);

@@ -33,3 +33,7 @@ bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st);
 // Weight-resident streaming 16-bit kernel for many rows and K = 128 / 192 / 256 / 384 (linear_stream.hip);
 // false when the shape is outside what it covers.
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st);
+
+// Ring-buffered 16-bit kernel for large row counts and K a multiple of 32 (linear_ring.hip): operands go from
+// global memory straight into an LDS ring; false when the shape is outside what it covers.
+bool bsrl_linear_ring(const LinArgs& a, int act, int dtype, hipStream_t st);

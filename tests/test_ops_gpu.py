@@ -142,11 +142,13 @@ def test_linear_strided_views_split_and_packing(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rows,K,M", [(4096, 128, 128), (5000, 128, 384), (4097, 384, 1152), (8192, 1536, 384),
-                                      (6000, 192, 576), (4100, 40, 192), (9000, 256, 1024), (4099, 128, 136)])
+                                      (6000, 192, 576), (4100, 40, 192), (9000, 256, 1024), (4099, 128, 136),
+                                      (4200, 96, 1024), (4500, 512, 1280)])
 @pytest.mark.parametrize("act,use_res", [(None, False), ("gelu", False), ("relu", True), (None, True)])
 def test_linear_large_row_counts_take_the_tiled_kernel(dtype, rows, K, M, act, use_res):
-    """rows >= 4096 with aligned shapes run the LDS-tiled kernel: same closed form, and the same
-    BITS as the direct-from-global kernel on a slice (both accumulate k in the same order)."""
+    """rows >= 4096 with aligned shapes run the LDS kernels (K a multiple of 32: the ring-buffered kernel, 256- or
+    128-column tiles by M and K; otherwise the register-staged tiled kernel): same closed form, and the same BITS as
+    the direct-from-global kernel on a slice (all accumulate k in the same order)."""
     x = _rand(rows, K, dtype=dtype, seed=rows)
     w = _rand(M, K, dtype=dtype, seed=K + M, scale=1 / math.sqrt(K))
     b = _rand(M, seed=M)
@@ -471,7 +473,7 @@ def test_wgrad_strided_operands_and_empty_batch():
 
 # ---------------------------------------------------------------- data gradient through a ReLU
 @pytest.mark.parametrize("dtype", DTS)
-@pytest.mark.parametrize("rows,K,M", [(1, 8, 8), (77, 192, 768), (5000, 192, 768), (4096, 128, 512), (333, 40, 101), (129, 256, 96)])
+@pytest.mark.parametrize("rows,K,M", [(1, 8, 8), (77, 192, 768), (5000, 192, 768), (4096, 128, 512), (4300, 768, 192), (333, 40, 101), (129, 256, 96)])
 def test_linear_gated(dtype, rows, K, M):
     """(g @ W) * [hidden > 0] == autograd through relu(h @ W1^T) @ W2^T at the hidden (python/fp16_linear.py:719-727)."""
     g = _rand(rows, K, dtype=dtype, seed=rows + K)
