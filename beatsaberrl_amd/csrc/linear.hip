@@ -244,7 +244,11 @@ int lin_dispatch(const LinArgs& a, int act, int dtype, int out_dtype, hipStream_
                          (!a.bias || bsrl_aligned(a.bias, 16)) &&
                          (!a.res || (a.ldr % 4 == 0 && bsrl_aligned(a.res, 8))) &&
                          (!a.gate || (a.ldgate % 4 == 0 && bsrl_aligned(a.gate, 8)));
-        if (vec && bsrl_linear_stream(a, act, dtype, st)) {
+        if (vec && a.res && bsrl_linear_ring(a, act, dtype, st)) {
+            // with a residual the ring kernel's epilogue (all residual loads of a wave tile in flight at once)
+            // beats the streaming kernel at every K measured (75 vs 97 us at 128 -> 128, 150 vs 192 at 192 -> 192,
+            // 475k rows)
+        } else if (vec && bsrl_linear_stream(a, act, dtype, st)) {
             // many rows, modest K: the weight-resident streaming kernel
         } else if (vec && bsrl_linear_ring(a, act, dtype, st)) {
             // large, aligned, 16-bit-out problems with K a multiple of 32: operands straight into an LDS ring
