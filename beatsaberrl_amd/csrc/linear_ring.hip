@@ -11,13 +11,15 @@
 //   BK = 64: a block is 8 rows x 128 B (whole cache lines: half as many requests to L2, ~11 % faster per k);
 //            lane l fetches row l / 8, k piece (l % 8) ^ row.
 //
-// Two geometries, picked by the column count:
+// Three geometries, picked by the column count:
 //   narrow: 256 x 128 tile, 4 waves, BK 32 x 3 stages = 72 KB, two workgroups per CU (the epilogue and ring fill
 //           of one overlap the main loop of the other);
 //   wide:   256 x 256 tile, 8 waves (4 row slabs x 2 column slabs), BK 64 x 2 stages = 128 KB, one workgroup per
 //           CU.  What bounds the main loop is the rate at which a CU pulls operands from L2 (~16 B/clk/CU measured
 //           with either geometry, against 48 B/clk that 256 x 128 tiles would need at full MFMA rate and 32 for
 //           256 x 256): a stage of the wide tile moves 2/3 of the bytes per MFMA.
+//   192:    256 x 192 tile, 8 waves of 64 x 96, BK 64 x 2 stages = 112 KB: one column block for the d = 192
+//           shapes, where 128-column tiles take two (the second half empty) and pull x from L2 twice.
 // Workgroup ids are remapped so that all column blocks of a row block run on the same XCD one after the other:
 // the row block's x tile crosses the fabric once and then hits in that XCD's L2.
 //
@@ -33,13 +35,14 @@
 namespace {
 
 constexpr int BM = 256;
-constexpr int EP_LD = 128 + 4;                                // epilogue row pitch (floats): a wave stages 16 x 128
+constexpr int EP_LD = 128 + 4;                                // epilogue row pitch (floats): a wave stages 16 x <= 128
 
-// Geometry of one instantiation: WC wave columns of 128 (workgroup tile 256 x 128 WC, 4 WC waves), BK k per stage
-// (32: a load covers 16 rows x 64 B; 64: 8 rows x 128 B), NS stages.
-template <int WC, int BK, int NS>
+// Geometry of one instantiation: WC wave columns of 16 CT (workgroup tile 256 x 16 CT WC, 4 WC waves), BK k per
+// stage (32: a load covers 16 rows x 64 B; 64: 8 rows x 128 B), NS stages.
+template <int WC, int BK, int NS, int CT = 8>
 struct Geo {
-    static constexpr int BN = 128 * WC, NW = 4 * WC, NT = 64 * NW;
+    static constexpr int CW = 16 * CT;                                   // columns per wave
+    static constexpr int BN = CW * WC, NW = 4 * WC, NT = 64 * NW;
     static constexpr int KCH = BK / 32;                                  // 32-wide k chunks per stage
     static constexpr int RPL = 512 / BK, LPR = 64 / RPL;                 // rows per load instruction, lanes per row
     static constexpr int XB = BM / RPL, WB = BN / RPL, NB = XB + WB;     // 1 KB blocks per stage
@@ -59,14 +62,15 @@ __device__ __forceinline__ void frag_load(uint32_t voff, const void* sbase, uint
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-template <typename DT, int ACT, int WC, int BK, int NS>
-__global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear_ring_kernel(LinArgs a, int ncb, int nrb) {
-    typedef Geo<WC, BK, NS> G;
+template <typename DT, int ACT, int WC, int BK, int NS, int CT>
+__global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void linear_ring_kernel(LinArgs a, int ncb, int nrb) {
+    typedef Geo<WC, BK, NS, CT> G;
+    constexpr int CW = G::CW;
     constexpr int BN = G::BN, NW = G::NW, KCH = G::KCH, RPL = G::RPL, LPR = G::LPR, XB = G::XB, STAGE_U4 = G::STAGE_U4;
     constexpr int NLX = G::NLX, NLW = G::NLW, NLD = G::NLD;
     extern __shared__ __attribute__((aligned(16))) u32x4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave & 3, wc = wave >> 2;                   // the wave's 64-row slab and 128-column slab
+    const int wr = wave & 3, wc = wave >> 2;                   // the wave's 64-row slab and column slab
     const int r16 = lane & 15, g = lane >> 4;
     // workgroup id -> (row block, column block): ids go round-robin over the 8 XCDs; inside an XCD consecutive
     // workgroups walk the column blocks of one row block
@@ -104,9 +108,9 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear
         xs += 2 * BK; ws += 2 * BK;
     };
 
-    f32x4 acc[8][4];                               // [column tile][row tile]
+    f32x4 acc[CT][4];                              // [column tile][row tile]
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < CT; ++i)
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) acc[i][jj] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
@@ -131,8 +135,8 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj) xf[jj] = __builtin_bit_cast(s16x8, st[rd(wr * 4 + jj, c)]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const s16x8 wf = __builtin_bit_cast(s16x8, st[XB * 64 + rd(wc * 8 + i, c)]);
+            for (int i = 0; i < CT; ++i) {
+                const s16x8 wf = __builtin_bit_cast(s16x8, st[XB * 64 + rd(wc * CT + i, c)]);
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) acc[i][jj] = DT::mfma32(wf, xf[jj], acc[i][jj]);
             }
@@ -145,8 +149,8 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear
     // residual (or, without one, the gate) for the whole 64 x 128 wave tile is requested up front, 16 loads in
     // flight, so that its latency is paid once per tile and not once per row group.
     const int m16 = lane & 15, rq = lane >> 4;
-    const int colw = col0 + wc * 128 + 8 * m16;                  // M % 8 == 0: the 8 columns are in or out together
-    const bool col_ok = colw < a.M;
+    const int colw = col0 + wc * CW + 8 * m16;                   // M % 8 == 0: the 8 columns are in or out together
+    const bool col_ok = 8 * m16 < CW && colw < a.M;              // 96-column slabs leave lanes 12..15 of a row idle
     const u16* aux = static_cast<const u16*>(a.res ? a.res : a.gate);
     const int64_t ldaux = a.res ? a.ldr : a.ldgate;
     const bool gate_inline = a.res && a.gate;
@@ -172,7 +176,7 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < CT; ++i)
             *reinterpret_cast<float4*>(ep + r16 * EP_LD + i * 16 + 4 * g) = make_float4(acc[i][jj][0], acc[i][jj][1], acc[i][jj][2], acc[i][jj][3]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -207,10 +211,10 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS>::WG_PER_CU)) void linear
     }
 }
 
-template <typename DT, int ACT, int WC, int BK, int NS>
+template <typename DT, int ACT, int WC, int BK, int NS, int CT>
 bool launch_geo(const LinArgs& a, hipStream_t st) {
-    typedef Geo<WC, BK, NS> G;
-    auto kern = linear_ring_kernel<DT, ACT, WC, BK, NS>;
+    typedef Geo<WC, BK, NS, CT> G;
+    auto kern = linear_ring_kernel<DT, ACT, WC, BK, NS, CT>;
     static bool ready = false;                     // per instantiation; the attribute is process-wide per function
     if (!ready) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES) != hipSuccess) {
@@ -229,8 +233,12 @@ bool launch_geo(const LinArgs& a, hipStream_t st) {
 template <typename DT, int ACT>
 bool launch_one(const LinArgs& a, hipStream_t st) {
     // 256-column tiles (half the operand traffic per MFMA) when the columns fill them
-    if ((a.M % 256 == 0 || a.M >= 1024) && a.K % 64 == 0) return launch_geo<DT, ACT, 2, 64, 2>(a, st);
-    return launch_geo<DT, ACT, 1, 32, 3>(a, st);
+    if ((a.M % 256 == 0 || a.M >= 1024) && a.K % 64 == 0) return launch_geo<DT, ACT, 2, 64, 2, 8>(a, st);
+    // 192-column tiles: one column block where 128-column tiles take two (the second half empty) and read x twice
+    // (with more than one block of them and a short K the two-workgroups-per-CU narrow tiles win: 0.47 vs 0.51 ms
+    // at K = M = 384, 786k rows; at K = 1536 it is 1.24 vs 1.14 the other way)
+    if ((a.M == 192 || (a.M % 192 == 0 && a.M <= 768 && a.K >= 512)) && a.K % 64 == 0) return launch_geo<DT, ACT, 2, 64, 2, 6>(a, st);
+    return launch_geo<DT, ACT, 1, 32, 3, 8>(a, st);
 }
 
 template <typename DT>
