@@ -51,14 +51,19 @@ struct Geo {
     static constexpr int NLX = XB / NW, NLW = WB / NW, NLD = NLX + NLW;  // loads per wave and stage
     static constexpr int WG_PER_CU = LDS_BYTES <= 80 * 1024 ? 2 : 1;
     static_assert(XB % NW == 0 && WB % NW == 0, "blocks must divide over the waves");
+    static_assert(NLD <= KCH * CT, "a stage's loads are spread over its MFMA groups");
     static_assert(16 * EP_LD * 4 * NW <= LDS_BYTES, "epilogue staging must fit in the operand ring");
 };
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// one block load: 64 lanes x 16 bytes from sbase + voff (bytes) to LDS bytes [lds_addr, lds_addr + 1024)
+// one block load: 64 lanes x 16 bytes from sbase + voff (bytes) to LDS bytes [lds_addr, lds_addr + 1024).  No "memory"
+// clobber: what orders these asynchronous LDS writes against the fragment reads is the vmcnt wait + barrier of the
+// stage loop (both compiler barriers), never program order - and with the clobber the compiler kept every fragment
+// read behind the load issued before it, one LDS latency per MFMA group.  volatile keeps the loads in order among
+// themselves and against the waits.
 __device__ __forceinline__ void frag_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "m0");
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
@@ -107,6 +112,14 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
         for (int i = 0; i < NLW; ++i) frag_load(voff[NLX + i], ws, sb + (XB + wave + NW * i) * 1024);
         xs += 2 * BK; ws += 2 * BK;
     };
+    // the same loads one at a time, for spreading over the MFMAs of a stage: issued in one burst after the barrier, the
+    // 8 waves' loads queue behind each other in the CU's address unit and every wave stalls in its issue phase
+    auto issue_one = [&](int slot, int idx) __attribute__((always_inline)) {
+        const uint32_t sb = lds_base + slot * (STAGE_U4 * 16);
+        if (idx < NLX) frag_load(voff[idx], xs, sb + (wave + NW * idx) * 1024);
+        else frag_load(voff[idx], ws, sb + (XB + wave + NW * (idx - NLX)) * 1024);
+        if (idx == NLD - 1) { xs += 2 * BK; ws += 2 * BK; }
+    };
 
     f32x4 acc[CT][4];                              // [column tile][row tile]
 #pragma unroll
@@ -124,26 +137,36 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) if (s < nsteps) issue(s);
     int slot = 0, fill = NS - 1;                                 // slot of step s; slot that step s + NS - 1 goes to
-    for (int s = 0; s < nsteps; ++s) {
-        if (s + NS - 2 < nsteps) wait_loads<NLD * (NS - 2)>(); else wait_loads<0>();
+    // one stage: the fragment reads and MFMAs of slot `slot`, with the loads of stage s + NS - 1 spread over the
+    // MFMA groups when MORE.  Two loops (main with loads, tail without) rather than a branch inside one: with the
+    // branch the fragment reads were no longer issued ahead of the previous group's MFMAs.
+#define RING_STAGE(MORE)                                                                                        \
+    do {                                                                                                        \
+        const u32x4* st = lds + slot * STAGE_U4;                                                                \
+        _Pragma("unroll") for (int c = 0; c < KCH; ++c) {                                                       \
+            s16x8 xf[4];                                                                                        \
+            _Pragma("unroll") for (int jj = 0; jj < 4; ++jj) xf[jj] = __builtin_bit_cast(s16x8, st[rd(wr * 4 + jj, c)]); \
+            _Pragma("unroll") for (int i = 0; i < CT; ++i) {                                                    \
+                const s16x8 wf = __builtin_bit_cast(s16x8, st[XB * 64 + rd(wc * CT + i, c)]);                   \
+                _Pragma("unroll") for (int jj = 0; jj < 4; ++jj) acc[i][jj] = DT::mfma32(wf, xf[jj], acc[i][jj]); \
+                if (MORE && c * CT + i < NLD) issue_one(fill, c * CT + i);                                      \
+            }                                                                                                   \
+        }                                                                                                       \
+        slot = slot + 1 == NS ? 0 : slot + 1;                                                                   \
+        fill = fill + 1 == NS ? 0 : fill + 1;                                                                   \
+    } while (0)
+    int s = 0;
+    for (; s + NS - 1 < nsteps; ++s) {
+        wait_loads<NLD * (NS - 2)>();
         __syncthreads();                           // step s has landed for every wave; slot `fill` is no longer read
-        if (s + NS - 1 < nsteps) issue(fill);
-        const u32x4* st = lds + slot * STAGE_U4;
-#pragma unroll
-        for (int c = 0; c < KCH; ++c) {
-            s16x8 xf[4];
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) xf[jj] = __builtin_bit_cast(s16x8, st[rd(wr * 4 + jj, c)]);
-#pragma unroll
-            for (int i = 0; i < CT; ++i) {
-                const s16x8 wf = __builtin_bit_cast(s16x8, st[XB * 64 + rd(wc * CT + i, c)]);
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) acc[i][jj] = DT::mfma32(wf, xf[jj], acc[i][jj]);
-            }
-        }
-        slot = slot + 1 == NS ? 0 : slot + 1;
-        fill = fill + 1 == NS ? 0 : fill + 1;
+        RING_STAGE(true);
     }
+    for (; s < nsteps; ++s) {
+        if (s + NS - 2 < nsteps) wait_loads<NLD * (NS - 2)>(); else wait_loads<0>();
+        __syncthreads();
+        RING_STAGE(false);
+    }
+#undef RING_STAGE
     // epilogue.  After a transpose through LDS lane (rq, m) = (lane / 16, lane % 16) owns 8 consecutive columns
     // 8 m .. 8 m + 7 of rows rq + 4 q: 16 lanes write (and read the residual of) one 256-byte row segment.  The
     // residual (or, without one, the gate) for the whole 64 x 128 wave tile is requested up front, 16 loads in
@@ -153,7 +176,6 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
     const bool col_ok = 8 * m16 < CW && colw < a.M;              // 96-column slabs leave lanes 12..15 of a row idle
     const u16* aux = static_cast<const u16*>(a.res ? a.res : a.gate);
     const int64_t ldaux = a.res ? a.ldr : a.ldgate;
-    const bool gate_inline = a.res && a.gate;
     u32x4 pre[16];
     if (aux) {
 #pragma unroll
@@ -193,8 +215,7 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
                 for (int e = 0; e < 4; ++e) { v[2 * e] += DT::to_f((u16)(p[e] & 0xffff)); v[2 * e + 1] += DT::to_f((u16)(p[e] >> 16)); }
             }
             if (a.gate && col_ok && row < a.rows) {
-                u32x4 gv = p;
-                if (gate_inline) gv = *reinterpret_cast<const u32x4*>(static_cast<const u16*>(a.gate) + row * a.ldgate + colw);
+                const u32x4 gv = p;                    // residual and gate together are not taken (entry check)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     if (!(DT::to_f((u16)(gv[e] & 0xffff)) > 0.f)) v[2 * e] = 0.f;
@@ -254,6 +275,8 @@ bool bsrl_linear_ring(const LinArgs& a, int act, int dtype, hipStream_t st) {
     if (a.out_f32 || a.y2 || a.rows < 4096 || a.M % 8 != 0 || a.K % 32 != 0) return false;
     if (a.ldx % 8 != 0 || !bsrl_aligned(a.x, 16) || !bsrl_aligned(a.w, 16) || a.ldx > (1 << 22) || a.K > (1 << 22)) return false;
     if (a.ldy % 8 != 0 || a.y_gstride % 8 != 0 || !bsrl_aligned(a.y, 16) || (a.res && (a.ldr % 8 != 0 || !bsrl_aligned(a.res, 16)))) return false;
-    if (a.gate && (a.ldgate % 8 != 0 || !bsrl_aligned(a.gate, 16))) return false;
+    // a load inside the row-group loop would put a vmcnt(0) wait there, and on this part that also waits for the
+    // previous group's stores: residual and gate together go to the tiled kernel
+    if (a.gate && (a.res || a.ldgate % 8 != 0 || !bsrl_aligned(a.gate, 16))) return false;
     return dtype == BSRL_F16 ? launch<F16>(a, act, st) : launch<BF16>(a, act, st);
 }
