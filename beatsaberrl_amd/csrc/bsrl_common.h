@@ -101,6 +101,12 @@ template <int ACT> __device__ __forceinline__ float act16_tail(float x, Act16Hea
     }
     return x;
 }
+// Pins an fp32 value in a register.  Where an activation's last multiply is followed directly by the conversion to
+// fp16, the compiler fuses the two into v_fma_mixlo_f16 (ONE rounding); kernels in which a branch or another op sits
+// between them round twice.  All linear kernels must produce the same bits for a row (a row's result may not depend
+// on which kernel its batch size selects), so the fused form is kept out where the pattern can arise.
+__device__ __forceinline__ float keep_f32(float v) { asm("" : "+v"(v)); return v; }
+
 // activation for values about to be rounded to fp16 / bf16
 template <int ACT> __device__ __forceinline__ float apply_act16(float x) {
     if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);

@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
             const float4 f1 = *reinterpret_cast<const float4*>(ep + rl * EP_LD + 8 * m16 + 4);
             float v[8] = {f0.x, f0.y, f0.z, f0.w, f1.x, f1.y, f1.z, f1.w};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = apply_act16<ACT>(v[e] + bv[e]);
+            for (int e = 0; e < 8; ++e) v[e] = keep_f32(apply_act16<ACT>(v[e] + bv[e]));
             const u32x4 p = pre[jj * 4 + q];
             if (a.res) {
 #pragma unroll

@@ -32,8 +32,11 @@ constexpr int ST_THREADS = 512;                  // 8 waves share one resident w
 constexpr int ST_ROWS = 32;                      // rows per wave tile (2 MFMA row tiles)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <typename DT, int KC, int MT>
-__global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, int act, int nb, int walkers) {
+// ACT and AUX (0 none, 1 residual, 2 ReLU gate) are compile-time: with run-time switches the epilogue was 2270 VALU
+// instructions and 248 branches per 32-row tile and took 12k of a tile's 18.5k cycles (traced with s_memtime), twice
+// what its 144 MFMAs took.
+template <typename DT, int KC, int MT, int ACT, int AUX>
+__global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, int nb, int walkers) {
     extern __shared__ __attribute__((aligned(16))) uint4 wl[];           // [MT * KC][64] fragments, MT * 16 bias floats, 8 wave tiles
     constexpr int KE = KC * 32;                                           // K
     constexpr int TP = (KE > MT * 16 ? KE : MT * 16) + 8;                 // wave tile row pitch (elements): rows 16 B off a bank period
@@ -130,19 +133,14 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
                 const bool on = rv && col < a.M;
                 const float4 bv = *reinterpret_cast<const float4*>(bl + mt * 16 + 4 * g);
                 float o[4] = {acc[mt][rt][0] + bv.x, acc[mt][rt][1] + bv.y, acc[mt][rt][2] + bv.z, acc[mt][rt][3] + bv.w};
-                if (act == BSRL_ACT_RELU) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = fmaxf(o[e], 0.f);
-                } else if (act == BSRL_ACT_GELU) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = gelu_fast(o[e]);
-                }
-                if (res && on) {
+                for (int e = 0; e < 4; ++e) o[e] = keep_f32(apply_act16<ACT>(o[e]));
+                if (AUX == 1 && on) {
                     const uint2 rv2 = *reinterpret_cast<const uint2*>(res + row * a.ldr + col);
                     o[0] += DT::to_f((u16)(rv2.x & 0xffff)); o[1] += DT::to_f((u16)(rv2.x >> 16));
                     o[2] += DT::to_f((u16)(rv2.y & 0xffff)); o[3] += DT::to_f((u16)(rv2.y >> 16));
                 }
-                if (gate && on) {
+                if (AUX == 2 && on) {
                     const uint2 gv = *reinterpret_cast<const uint2*>(gate + row * a.ldgate + col);
                     if (!(DT::to_f((u16)(gv.x & 0xffff)) > 0.f)) o[0] = 0.f;
                     if (!(DT::to_f((u16)(gv.x >> 16)) > 0.f)) o[1] = 0.f;
@@ -178,11 +176,11 @@ int device_cus() {
     return cus;
 }
 
-template <typename DT, int KC, int MT>
-bool launch(const LinArgs& a, int act, hipStream_t st) {
+template <typename DT, int KC, int MT, int ACT, int AUX>
+bool launch(const LinArgs& a, hipStream_t st) {
     constexpr int TP = (KC * 32 > MT * 16 ? KC * 32 : MT * 16) + 8;
     const size_t lds = (size_t)MT * KC * 1024 + (size_t)MT * 16 * sizeof(float) + (size_t)8 * 16 * TP * sizeof(u16);
-    auto kern = linear_stream_kernel<DT, KC, MT>;
+    auto kern = linear_stream_kernel<DT, KC, MT, ACT, AUX>;
     // workgroups resident per CU (LDS and registers), 0 = this instantiation cannot run here
     static const int per_cu = [&] {
         int n = 0;
@@ -200,18 +198,29 @@ bool launch(const LinArgs& a, int act, hipStream_t st) {
     if (walkers < 8) return false;
     const int64_t need = ((ntiles + 7) / 8 + 7) / 8 * 8;
     if (walkers > need) walkers = need;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(walkers * nb)), dim3(ST_THREADS), lds, st, a, act, nb, (int)walkers);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(walkers * nb)), dim3(ST_THREADS), lds, st, a, nb, (int)walkers);
     return true;
+}
+
+template <typename DT, int ACT, int AUX>
+bool by_k(const LinArgs& a, hipStream_t st) {
+    switch (a.K / 32) {
+        case 4: return launch<DT, 4, 8, ACT, AUX>(a, st);
+        case 6: return launch<DT, 6, 12, ACT, AUX>(a, st);
+        case 8: return launch<DT, 8, 8, ACT, AUX>(a, st);
+        default: return false;
+    }
 }
 
 template <typename DT>
 bool dispatch(const LinArgs& a, int act, hipStream_t st) {
-    switch (a.K / 32) {
-        case 4: return launch<DT, 4, 8>(a, act, st);
-        case 6: return launch<DT, 6, 12>(a, act, st);
-        case 8: return launch<DT, 8, 8>(a, act, st);
-        default: return false;
-    }
+    // the combinations the policy uses: any activation alone, a residual without one, the gate without one
+    if (a.res && a.gate) return false;
+    if (a.gate) return act == BSRL_ACT_NONE ? by_k<DT, BSRL_ACT_NONE, 2>(a, st) : false;
+    if (a.res) return act == BSRL_ACT_NONE ? by_k<DT, BSRL_ACT_NONE, 1>(a, st) : false;
+    if (act == BSRL_ACT_RELU) return by_k<DT, BSRL_ACT_RELU, 0>(a, st);
+    if (act == BSRL_ACT_GELU) return by_k<DT, BSRL_ACT_GELU, 0>(a, st);
+    return by_k<DT, BSRL_ACT_NONE, 0>(a, st);
 }
 
 }  // namespace
