@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -68,6 +68,7 @@ SIGNATURES = {
     "bsrl_counter_add": (_i32, [_p, C.c_uint64, _p]),
     "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _p, _i32,
                                  _p, _p, _p, _p, _p, _p]),
+    "bsrl_critic_pool": (_i32, [_p, _p, _p, C.c_float, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_ln_bwd_workspace_size": (_i64, [_i64]),
     "bsrl_ln_bwd": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i32, _p]),
     "bsrl_attn_bwd": (_i32, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _i64,

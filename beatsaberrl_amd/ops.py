@@ -317,6 +317,30 @@ def attn_bwd(q, k, v, dout, n_heads, key_bias=None, n_valid=None, out=None):
     return dq, dk, dv
 
 
+def critic_pool_supported(T, d, n_heads, dtype) -> bool:
+    """Shapes bsrl_critic_pool covers (16-bit streams; the fp32 parity path keeps the reference's op order)."""
+    return dtype in (torch.float16, torch.bfloat16) and T <= 32 and n_heads <= 16 and d in (128, 192, 256) and d % n_heads == 0
+
+
+def critic_pool(x_res, ln_weight, ln_bias, eps, qk, key_bias, n_heads):
+    """pooled (B, H, d) = per-head attention pool of LN(x_res) under the single query folded into qk (B, H, d)
+    (see bsrl_critic_pool: the adapool critic's attention without materialised keys / values)."""
+    _need_cuda(x_res, ln_weight, ln_bias, qk, key_bias)
+    B, T, d = x_res.shape
+    if qk.shape != (B, n_heads, d) or qk.dtype is not x_res.dtype or not (x_res.is_contiguous() and qk.is_contiguous()):
+        raise TypeError("critic_pool: x_res (B, T, d) and qk (B, H, d) must be contiguous in one dtype")
+    if key_bias is not None and (key_bias.shape != (B, T) or key_bias.dtype is not x_res.dtype or not key_bias.is_contiguous()):
+        raise TypeError("critic_pool: key_bias must be contiguous (B, T) in x_res's dtype")
+    pooled = torch.empty(B, n_heads, d, device=x_res.device, dtype=x_res.dtype)
+    with torch.cuda.device(x_res.device):
+        rc = _lib.load().bsrl_critic_pool(x_res.data_ptr(), _f32c(ln_weight, "ln weight").data_ptr(),
+                                          _f32c(ln_bias, "ln bias").data_ptr(), float(eps), qk.data_ptr(), _ptr(key_bias),
+                                          pooled.data_ptr(), B, T, d, n_heads, dt_code(x_res.dtype), _stream(x_res))
+    if not _lib.check(rc, "bsrl_critic_pool"):
+        raise Unsupported(f"critic_pool T={T} d={d} H={n_heads} dtype={x_res.dtype}")
+    return pooled
+
+
 def ffn_fused_supported(d, F, dtype) -> bool:
     return bool(_lib.load().bsrl_ffn_fused_supported(d, F, dt_code(dtype)))
 

@@ -375,6 +375,10 @@ class NotePolicy(nn.Module):
         # shape has one (ops.blocks_pack_size > 0); "off": always the per-op launch train
         self.fused_blocks = "auto"
         self._blocks_image = None               # [weights version, dtype, uint8 image]
+        # True: the critic's one-query attention runs as a pool over LN(x_res) with the k | v projections folded
+        # around it (no (B T, 2d) keys / values); False: the reference's op order
+        self.critic_pool = True
+        self._critic_pool_cache = None
         # sampling-call counter of the in-kernel Philox stream; on the device so that a captured
         # get_action_and_value draws fresh noise on every replay
         self.register_buffer("_sample_ctr", torch.zeros(1, dtype=torch.int64), persistent=False)
@@ -444,6 +448,8 @@ class NotePolicy(nn.Module):
             _fl.packed_halves([blk.k_proj, blk.v_proj], dt)
         _fl.packed_halves([self.critic_k, self.critic_v], dt)
         _fl.packed_halves(list(self.heads), dt)
+        if self.critic_pool:
+            self._critic_pool_weights(dt)
 
     def load_state_dict(self, *a, **k):
         r = super().load_state_dict(*a, **k)
@@ -615,15 +621,47 @@ class NotePolicy(nn.Module):
         r = _lin(self.trunk_fc1, u, act="relu")
         return self.trunk_ln2(_lin(self.trunk_fc2, r, residual=t))
 
+    def _critic_pool_weights(self, dt):
+        """Block-structured weights of the pooled critic attention, rebuilt in place per weights version (their
+        addresses stay put under a captured graph): wqk (H d, d) with wqk[h d + e, h dh + c] = Wk[h dh + c, e] maps the
+        query to the H per-head key-space vectors, wvo (d, H d) with wvo[h dh + c, h d + e] = Wv[h dh + c, e] maps the H
+        pooled vectors to the attention output; zeros elsewhere."""
+        d, H = self.embed, self.n_heads
+        dh = d // H
+        c = self._critic_pool_cache
+        dev = self.critic_k.weight.device
+        if c is None or c[1] is not dt or c[2].device != dev:
+            c = self._critic_pool_cache = [-1, dt, torch.zeros(H, d, H, dh, device=dev, dtype=dt),
+                                           torch.zeros(H, dh, H, d, device=dev, dtype=dt),
+                                           torch.empty(d, device=dev, dtype=torch.float32)]
+        if c[0] != _fl._weights_version:
+            wk, wv = self.critic_k.weight.detach(), self.critic_v.weight.detach()
+            for h in range(H):
+                c[2][h, :, h, :].copy_(wk[h * dh:(h + 1) * dh].t())
+                c[3][h, :, h, :].copy_(wv[h * dh:(h + 1) * dh])
+            c[4].copy_(self.critic_v.bias.detach())
+            c[0] = _fl._weights_version
+        return c[2].view(H * d, d), c[3].view(d, H * d), c[4]
+
     def _critic(self, x_res, hfeat, attn_bias):
         """adapool_v1 value path (policy.py:1346-1403): LN -> query from the torso token ->
         packed k|v -> 1-query attention pool -> out -> MLP -> HL-Gauss expectation."""
         B, T, d = x_res.shape
-        hv = self.critic_ln(x_res)
-        q = _lin(self.critic_q, hv[:, 2:3])                                # (B, 1, d)
-        wkv, bkv = _fl.packed_halves([self.critic_k, self.critic_v], x_res.dtype)
-        kv = ops.linear(hv, wkv, bkv)
-        a = ops.attn_fwd(q, kv[..., :d], kv[..., d:], self.n_heads, key_bias=attn_bias).view(B, d)
+        H = self.n_heads
+        if self.critic_pool and ops.critic_pool_supported(T, d, H, x_res.dtype):
+            # one query per env: the k | v projections commute with the pool, so keys and values are never formed
+            wqk, wvo, bvo = self._critic_pool_weights(x_res.dtype)
+            q = _lin(self.critic_q, self.critic_ln(x_res[:, 2].contiguous()))          # (B, d), the torso token's query
+            qk = ops.linear(q, wqk).view(B, H, d)                                      # Wk_h^T q_h per head
+            pooled = ops.critic_pool(x_res.contiguous(), self.critic_ln.weight.detach(), self.critic_ln.bias.detach(),
+                                     self.critic_ln.eps, qk, attn_bias, H)
+            a = ops.linear(pooled.view(B, H * d), wvo, bvo)                            # Wv_h pooled_h + bv_h
+        else:
+            hv = self.critic_ln(x_res)
+            q = _lin(self.critic_q, hv[:, 2:3])                                # (B, 1, d)
+            wkv, bkv = _fl.packed_halves([self.critic_k, self.critic_v], x_res.dtype)
+            kv = ops.linear(hv, wkv, bkv)
+            a = ops.attn_fwd(q, kv[..., :d], kv[..., d:], H, key_bias=attn_bias).view(B, d)
         a = _lin(self.critic_out, a)
         z = torch.cat([a, hfeat], dim=-1)
         z = _lin(self.critic_mlp[0], z, act="relu")

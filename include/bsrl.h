@@ -280,6 +280,21 @@ int bsrl_blocks_forward(const bsrl_blocks_desc* desc, const void* packed,
                         const void* x_in, const void* key_bias,
                         void* x_res, void* x_out, int64_t B, bsrl_stream stream);
 
+/* ---- Critic attention pool (one query per env) ----------------------------------
+ * The attention of the reference's adapool critic (NotePolicy._critic, python/policy.py:1346-1403: critic_ln, k|v
+ * projection of all T tokens, 1-query multi-head attention) without the (B T, 2d) keys and values: with one query
+ * the projections commute with the pool.  Given qk (B, H, d) with qk[b, h] = Wk[h rows]^T q[b, h cols] this computes
+ *   hv_j = LN(x_res[b, j]) (rounded to `dtype`), p[h] = softmax_j(hv_j . qk[b, h] / sqrt(d / H) + key_bias[b, j]),
+ *   pooled[b, h, :] = sum_j p[h][j] hv_j
+ * (q_h . bk_h is constant over j and cancels; the caller finishes a_h = Wv[h rows] pooled_h + bv_h because the
+ * probabilities sum to 1).  x_res (B, T, d), qk (B, H, d), key_bias (B, T) or NULL, pooled (B, H, d): contiguous in
+ * `dtype`; ln_weight / ln_bias fp32 (d).  16-bit dtypes, T <= 32, H <= 16, d = 128 / 192 / 256 (the scores and the
+ * pool run as MFMAs, one wave per env); BSRL_UNSUPPORTED beyond - the caller then takes the k|v projection and
+ * bsrl_attn_fwd. */
+int bsrl_critic_pool(const void* x_res, const float* ln_weight, const float* ln_bias, float eps,
+                     const void* qk, const void* key_bias, void* pooled,
+                     int64_t B, int64_t T, int64_t d, int64_t H, int dtype, bsrl_stream stream);
+
 /* ---- LayerNorm backward --------------------------------------------------------
  * Replaces layer_norm_cuda.ln_bwd(x, dy, w, mean, rstd, gx=None, want_dbb=False)
  * (python/beat_arena_env/csrc/layer_norm.cu:645-729), the backward of both

@@ -162,6 +162,31 @@ def test_value_residual_at_init_is_bitwise_the_plain_policy(dtype):
     assert not torch.equal(lq, lp)                              # and with b != 0 block 0's values do get through
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_pooled_critic_matches_the_reference_op_order(dtype):
+    """`critic_pool` (keys / values never formed) against the k | v projection + 1-query attention path of the same
+    build: identical logits, values equal to the rounding of the path (python/policy.py:1346-1403)."""
+    m, sd = _big(13, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True)
+    m = m.to(DEV)
+    if dtype != "f32":
+        m.fp16 = True
+        m.stream_dtype = torch.float16 if dtype == "f16" else torch.bfloat16
+    obs = _make_obs(200, 5)
+    od = obs.to(DEV)
+    m.critic_pool = True
+    lg1, v1 = m.forward_stacked(od)
+    m.critic_pool = False
+    lg0, v0 = m.forward_stacked(od)
+    assert torch.equal(lg0, lg1)
+    _, ref_v = nr.forward(sd, m.arch, obs)
+    e_pool, e_ref = (v1.cpu() - ref_v).abs().max().item(), (v0.cpu() - ref_v).abs().max().item()
+    print(f"\n[{dtype}] value vs fp32 oracle: pooled {e_pool:.2e}, reference op order {e_ref:.2e}")
+    if dtype == "f32":
+        assert e_pool <= 1e-5 * (ref_v.abs().max().item() + 1) and e_ref <= 1e-5 * (ref_v.abs().max().item() + 1)
+    else:
+        assert e_pool <= max(1.25 * e_ref, 2e-3)
+
+
 @pytest.mark.parametrize("blocks", ["auto", "off"])
 def test_invariants_and_sampling_epilogue(blocks):
     m, sd = _big(9, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,

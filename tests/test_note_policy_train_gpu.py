@@ -131,11 +131,17 @@ def test_update_forward_is_bitwise_the_per_op_rollout_forward(dtype):
                 head_gears=tuple(7 if j == 4 else 5 for j in range(29))).to(DEV)
     m.fp16 = dtype == "f16"
     m.fused_blocks = "off"
+    m.critic_pool = False          # the update keeps the reference's critic op order; the rollout's pooled form rounds differently
     od = _obs(40, 8).to(DEV)
     with torch.no_grad():
         lg0, v0 = m.forward_stacked(od)
     lg1, v1 = m.forward_stacked(od)
     assert lg1.requires_grad and torch.equal(lg0, lg1.detach()) and torch.equal(v0, v1.detach())
+    if dtype == "f16":             # with the pool the logits are untouched and the value moves by rounding only
+        m.critic_pool = True
+        with torch.no_grad():
+            lg2, v2 = m.forward_stacked(od)
+        assert torch.equal(lg0, lg2) and (v2 - v0).abs().max().item() <= 5e-3
     # evaluation of given actions: the torch-op log-prob / entropy of the update == the sampling kernel's
     with torch.no_grad():
         act, lp0, ent0, _ = m.get_action_and_value(od)

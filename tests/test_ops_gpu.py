@@ -564,3 +564,62 @@ def test_streaming_linear_gate_and_token_slice_output():
     ops.linear(x, w, b, act="relu", out=stream[:, 5:])
     assert torch.equal(stream[:, 5:].reshape(N * G, 192), ops.linear(x, w, b, act="relu"))
     assert torch.equal(stream[:, :5], torch.full_like(stream[:, :5], 7.0))
+
+
+# ---------------------------------------------------------------- critic attention pool
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,T,d,H", [(1, 29, 192, 4), (37, 29, 192, 4), (9, 29, 128, 4), (5, 32, 128, 2), (4, 16, 256, 8), (3, 17, 192, 3), (6, 7, 256, 16),
+                                     (4101, 29, 192, 4)])
+@pytest.mark.parametrize("masked", [False, True])
+def test_critic_pool(dtype, B, T, d, H, masked):
+    """The pooled form against the reference's op order in fp64 (python/policy.py:1346-1403): LN, k = Wk hv + bk,
+    v = Wv hv + bv, one query per env, softmax(q.k / sqrt(dh) + bias) v - rebuilt from the pool as Wv pooled + bv."""
+    dh = d // H
+    x = _rand(B, T, d, dtype=dtype, seed=B + T, scale=1.5)
+    lw, lb = _rand(d, seed=1) * 0.3 + 1.0, _rand(d, seed=2) * 0.3
+    wk, wv = _rand(d, d, seed=3, scale=d ** -0.5), _rand(d, d, seed=4, scale=d ** -0.5)
+    bk, bv = _rand(d, seed=5), _rand(d, seed=6)
+    q = _rand(B, d, seed=7)
+    bias = None
+    if masked:
+        valid = torch.rand(B, T, generator=torch.Generator().manual_seed(3)) < 0.6
+        valid[:, :5] = True
+        bias = ((valid.float() - 1.0) * 16384.0).to(dtype).to(DEV)
+    qk = torch.stack([q[:, h * dh:(h + 1) * dh] @ wk[h * dh:(h + 1) * dh] for h in range(H)], 1).to(dtype).contiguous()
+    pooled = ops.critic_pool(x, lw, lb, 1e-5, qk, bias, H)
+    assert pooled.shape == (B, H, d) and pooled.dtype is dtype
+    # reference order on the same rounded operands
+    hv = F.layer_norm(x.double(), (d,), lw.double(), lb.double(), 1e-5).to(dtype).double()
+    k = hv @ wk.double().t() + bk.double()
+    v = hv @ wv.double().t() + bv.double()
+    out_ref = torch.empty(B, d, dtype=torch.float64, device=DEV)
+    out = torch.empty(B, d, dtype=torch.float64, device=DEV)
+    for h in range(H):
+        sl = slice(h * dh, (h + 1) * dh)
+        s = (k[..., sl] @ q.double()[:, sl, None]).squeeze(-1) / math.sqrt(dh)
+        if bias is not None:
+            s = s + bias.double()
+        p = torch.softmax(s, -1)
+        out_ref[:, sl] = (p[:, None, :] @ v[..., sl]).squeeze(1)
+        out[:, sl] = pooled[:, h].double() @ wv.double()[sl].t() + bv.double()[sl]
+        # the pool itself: rows of probabilities that sum to 1 applied to hv
+        s2 = (hv @ qk[:, h].double()[:, :, None]).squeeze(-1) / math.sqrt(dh) + (bias.double() if bias is not None else 0.0)
+        ref_pool = (torch.softmax(s2, -1)[:, None, :] @ hv).squeeze(1)
+        tol_p = 2e-5 if dtype is torch.float32 else 1.5 * EPS16[dtype]
+        assert (pooled[:, h].double() - ref_pool).abs().max().item() <= tol_p * (ref_pool.abs().max().item() + 1.0)
+    tol = 1e-4 if dtype is torch.float32 else 6 * EPS16[dtype]
+    assert (out - out_ref).abs().max().item() <= tol * (out_ref.abs().max().item() + 1.0)
+    if masked:      # junk in masked tokens cannot move the pool
+        x2 = x.clone()
+        x2[~valid.to(DEV)] = 9.0
+        assert torch.equal(ops.critic_pool(x2, lw, lb, 1e-5, qk, bias, H), pooled)
+
+
+def test_critic_pool_unsupported_shapes_say_so():
+    """fp32 streams, T > 32 and widths other than 128 / 192 / 256 are reported, not computed some other way."""
+    for dtype, T, d, H in ((torch.float32, 29, 192, 4), (torch.float16, 33, 192, 4), (torch.float16, 29, 96, 3)):
+        assert not ops.critic_pool_supported(T, d, H, dtype)
+        x = _rand(2, T, d, dtype=dtype, seed=1)
+        qk = _rand(2, H, d, dtype=dtype, seed=2)
+        with pytest.raises(ops.Unsupported):
+            ops.critic_pool(x, _rand(d, seed=3), _rand(d, seed=4), 1e-5, qk, None, H)
