@@ -8,7 +8,8 @@
 // and the three gradients are written through strides, so they may be column slices of one packed
 // q|k|v gradient buffer (what the reference's callers pass).
 //
-// 16-bit path: one wave64 per (env, head), 2 waves per workgroup.  q, k, v, dO of the pair are
+// 16-bit path: one wave64 per (env, head); a workgroup is the H heads of one env where they fit (persistent, the next
+// env's rows prefetched in registers), else 2 independent pairs.  q, k, v, dO are
 // staged once in LDS as they lie in memory (rows = tokens); every product is a chain of
 // v_mfma_f32_16x16x16 with the operand orientation each one needs:
 //   S^T = K Q^T and dP^T = V dO^T contract over features: both operands are plain 8-byte row reads;
@@ -17,8 +18,10 @@
 //   dQ^T = K^T dS^T, whose A operand (K^T) is an LDS transpose load (ds_read_b64_tr_b16);
 //   dV^T = dO^T P and dK^T = Q^T dS contract over QUERIES: P and dS of the current 16-query tile go
 //   through a 16-row LDS tile and both operands come back through transpose loads.
-// Every output lane holds 4 consecutive features of one token: 8-byte stores.  dK^T / dV^T stay in
-// accumulators across the query tiles.  HBM traffic: q, k, v, dO read once, dq, dk, dv written once.
+// Every output lane holds 4 consecutive features of one token; the gradients take the place of q, k, v in LDS and
+// leave as 16-byte pieces of whole rows.  dK^T / dV^T stay in accumulators across the query tiles.  HBM traffic:
+// q, k, v, dO read once, dq, dk, dv written once.  B = 16384, T = 29, 4 x 48: 454 us with per-wave slices and 8-byte
+// stores, 417 us with whole rows per workgroup, 319 us (4.0 TB/s) with the persistent prefetching form.
 //
 // fp32 path (parity configuration): one wave per (env, head) on LDS-staged fp32 tiles, plain FMA loops.
 #include "bsrl_common.h"
@@ -34,10 +37,12 @@ struct AttnBwdArgs {
     int64_t B; int T, TQ, H;
     float scale;
     int wave_elems;            // 16-bit path: LDS elements per wave
+    int out16;                 // 16-bit path: gradient rows may leave as 16-byte pieces (else 8-byte)
 };
 
 constexpr int kMaxKT = 3;      // key tiles of 16 (T <= 48)
 typedef short s16x4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
 
 // 16x16x16 operand whose contraction index runs over the ROWS of a row-major LDS tile: lane (i = lane % 16,
 // g = lane / 16) ends with rows k0 + 4 g + {0..3} of column c0 + i.  Lanes 4 r + s of a 16-lane group present
@@ -54,17 +59,31 @@ __device__ __forceinline__ s16x4 row16(const u16* tile, int pitch, int r0, int c
     return *reinterpret_cast<const s16x4*>(tile + (r0 + (lane & 15)) * pitch + c0 + 4 * (lane >> 4));
 }
 
-template <typename DT, int DH>
-__global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
+// COOP: a workgroup is the H heads of ONE env (wave = head) and moves the env's rows together: q, k, v, dO come in and
+// dq, dk, dv leave as whole d-wide rows (consecutive threads on consecutive 16-byte pieces), through the per-head LDS
+// tiles.  Otherwise (H > 8, or H heads do not fit the LDS) a workgroup is 2 independent (env, head) pairs and every wave
+// moves its own dh-wide slices.  Written straight from the accumulators (a lane holds 4 consecutive features of one
+// token) the gradients left as 32-byte pieces and the stores cost 130 us of a 450 us kernel at B = 16384, T = 29, 4 x 48.
+// NKT: key tiles of 16 the instantiation is sized for (2 for T <= 32: 60 fewer registers than 3, which is what lets the
+// persistent form keep the next env's rows in registers without spilling)
+template <typename DT, int DH, bool COOP, int NKT>
+__global__ __launch_bounds__(COOP ? 512 : 128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
     constexpr int DHP = DH == 32 ? 48 : 56;     // LDS row pitch of the token tiles (elements)
     constexpr int FT = DH / 16;
     extern __shared__ __attribute__((aligned(16))) u16 smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, g = lane >> 4;
-    const int64_t pair = (int64_t)blockIdx.x * 2 + wave;
-    if (pair >= a.B * a.H) return;                                   // waves are independent: no workgroup barrier below
-    const int64_t b = pair / a.H;
-    const int h = (int)(pair % a.H);
+    int64_t b; int h;
+    if (COOP) { b = blockIdx.x; h = wave; }
+    else {
+        const int64_t pair = (int64_t)blockIdx.x * 2 + wave;
+        if (pair >= a.B * a.H) return;                               // waves are independent: no workgroup barrier in this mode
+        b = pair / a.H;
+        h = (int)(pair % a.H);
+    }
+    // the group that moves rows together: all threads and all heads of the workgroup (COOP) or this wave and its head
+    const int gh = COOP ? a.H : 1, h0 = COOP ? 0 : h;
+    const int gthreads = COOP ? (int)blockDim.x : WAVE, gt = COOP ? (int)threadIdx.x : lane;
     const int T = a.T, TQ = a.TQ;
     const int nkt = (T + 15) >> 4, nqt = (TQ + 15) >> 4;
     const int TP = nkt * 16, TQP = nqt * 16, PP = TP + 8;
@@ -78,59 +97,89 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
     // stage the pair's q, dO (TQ rows) and k, v (T rows), zero rows up to the tile edge.  All global loads are
     // issued before the first LDS write: one memory round trip for the four matrices instead of one per piece.
     constexpr int PPR = DH / 8;                                     // 16-byte pieces per row
-    constexpr int NIT = (kMaxKT * 16 * PPR + WAVE - 1) / WAVE;      // pieces per lane and matrix, at most
-    uint4 buf[4][NIT];
-    const u16* srcs[4] = {static_cast<const u16*>(a.q) + b * a.q_bs + h * DH, static_cast<const u16*>(a.dout) + b * a.do_bs + h * DH,
-                          static_cast<const u16*>(a.k) + b * a.k_bs + h * DH, static_cast<const u16*>(a.v) + b * a.v_bs + h * DH};
+    constexpr int NIT = (NKT * 16 * PPR + WAVE - 1) / WAVE;      // pieces per lane and matrix, at most
+    u32x4v buf[4][NIT];                                             // native vectors: arrays of the uint4 class that live across a loop stay in scratch
+    u16 kraw[NKT][4];                                            // key bias of keys 16 kt + 4 g + e, raw
+    int nv_next = 0;
     const int64_t rss[4] = {a.q_rs, a.do_rs, a.k_rs, a.v_rs};
     const int nrows[4] = {TQ, TQ, T, T}, prows[4] = {TQP, TQP, TP, TP};
-    u16* dsts[4] = {Qs, dOs, Ks, Vs};
+    const int offs[4] = {0, TQP * DHP, 2 * TQP * DHP, 2 * TQP * DHP + TP * DHP};          // Qs, dOs, Ks, Vs inside a wave's region
+    // piece c = it * gthreads + gt of a matrix is (row c / rp, head (c % rp) / PPR, part (c % rp) % PPR)
+    const int rp = gh * PPR;
+    const int row_step = gthreads / rp, cp_step = gthreads % rp;
+    const int row_first = gt / rp, cp_first = gt % rp;
+    auto tile_of = [&](int hh) __attribute__((always_inline)) { return smem + (int64_t)(COOP ? hh : wave) * a.wave_elems; };
+    // all global loads of an env (the four matrices, the key bias, the valid count) are issued together
+    auto fetch = [&](int64_t be) __attribute__((always_inline)) {
+        const u16* srcs[4] = {static_cast<const u16*>(a.q) + be * a.q_bs + h0 * DH, static_cast<const u16*>(a.dout) + be * a.do_bs + h0 * DH,
+                              static_cast<const u16*>(a.k) + be * a.k_bs + h0 * DH, static_cast<const u16*>(a.v) + be * a.v_bs + h0 * DH};
 #pragma unroll
-    for (int mtx = 0; mtx < 4; ++mtx)
+        for (int mtx = 0; mtx < 4; ++mtx) {
+            int row = row_first, cp = cp_first;
 #pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-            const int c = it * WAVE + lane, row = c / PPR, part = c % PPR;
-            buf[mtx][it] = make_uint4(0, 0, 0, 0);
-            if (row < nrows[mtx]) buf[mtx][it] = *reinterpret_cast<const uint4*>(srcs[mtx] + (int64_t)row * rss[mtx] + part * 8);
+            for (int it = 0; it < NIT; ++it) {
+                buf[mtx][it] = (u32x4v){0u, 0u, 0u, 0u};
+                if (row < nrows[mtx]) buf[mtx][it] = *reinterpret_cast<const u32x4v*>(srcs[mtx] + (int64_t)row * rss[mtx] + (cp / PPR) * DH + (cp % PPR) * 8);
+                row += row_step; cp += cp_step;
+                if (cp >= rp) { cp -= rp; ++row; }
+            }
         }
 #pragma unroll
-    for (int mtx = 0; mtx < 4; ++mtx)
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int key = kt * 16 + g * 4 + e;
+                kraw[kt][e] = 0;
+                if (a.key_bias && key < T) kraw[kt][e] = static_cast<const u16*>(a.key_bias)[be * T + key];
+            }
+        nv_next = a.n_valid ? a.n_valid[be] : T;
+    };
+    fetch(b);
+  for (;;) {                                                        // COOP: a persistent workgroup walks envs b, b + grid, ...
+#pragma unroll
+    for (int mtx = 0; mtx < 4; ++mtx) {
+        int row = row_first, cp = cp_first;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
-            const int c = it * WAVE + lane, row = c / PPR, part = c % PPR;
-            if (row < prows[mtx]) *reinterpret_cast<uint4*>(dsts[mtx] + row * DHP + part * 8) = buf[mtx][it];
+            if (row < prows[mtx]) *reinterpret_cast<u32x4v*>(tile_of(cp / PPR) + offs[mtx] + row * DHP + (cp % PPR) * 8) = buf[mtx][it];
+            row += row_step; cp += cp_step;
+            if (cp >= rp) { cp -= rp; ++row; }
         }
-
+    }
     // additive bias / validity of keys 16 kt + 4 g + e, as the forward applies them
-    float kb[kMaxKT][4];
-    const int nv = a.n_valid ? a.n_valid[b] : T;
+    float kb[NKT][4];
+    const int nv = nv_next;
 #pragma unroll
-    for (int kt = 0; kt < kMaxKT; ++kt)
+    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int key = kt * 16 + g * 4 + e;
             float bias = 0.f;
             if (key >= T || key > nv) bias = -INFINITY;
             else if (a.key_bias) {
-                const float kbv = DT::to_f(static_cast<const u16*>(a.key_bias)[b * T + key]);
+                const float kbv = DT::to_f(kraw[kt][e]);
                 bias = kbv < -0.5f * BSRL_MASK_BIAS ? -INFINITY : kbv;
             }
             kb[kt][e] = bias;
         }
+    if (COOP) __syncthreads();
+    // the next env's loads fly during this env's arithmetic (their registers are free until the next tile fill)
+    const int64_t b_next = b + gridDim.x;
+    const bool more = COOP && b_next < a.B;
+    if (more) fetch(b_next);
 
-    f32x4 dkt[FT][kMaxKT], dvt[FT][kMaxKT];      // dK^T, dV^T: lane holds features 16 ft + 4 g + e of key 16 kt + r16
+    f32x4 dkt[FT][NKT], dvt[FT][NKT];      // dK^T, dV^T: lane holds features 16 ft + 4 g + e of key 16 kt + r16
 #pragma unroll
     for (int ft = 0; ft < FT; ++ft)
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt) { dkt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; dvt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+        for (int kt = 0; kt < NKT; ++kt) { dkt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; dvt[ft][kt] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
 
-    u16* dqp = static_cast<u16*>(a.dq) + b * a.dq_bs + h * DH;
     for (int qt = 0; qt < nqt; ++qt) {
         // S^T and dP^T tiles: lane holds keys 16 kt + 4 g + e of query 16 qt + r16
-        float s[kMaxKT][4], dp[kMaxKT][4];
+        float s[NKT][4], dp[NKT][4];
         float m = -INFINITY;
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt) {
+        for (int kt = 0; kt < NKT; ++kt) {
             f32x4 sa = {0.f, 0.f, 0.f, 0.f}, da = {0.f, 0.f, 0.f, 0.f};
             if (kt < nkt) {
 #pragma unroll
@@ -150,7 +199,7 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
         m = fmaxf(m, __shfl_xor(m, 32, WAVE));
         float sum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) { s[kt][e] = __expf(s[kt][e] - m); sum += s[kt][e]; }
         sum += __shfl_xor(sum, 16, WAVE);
@@ -158,14 +207,14 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
         const float inv = 1.0f / sum;
         float dsum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) { s[kt][e] *= inv; dsum += s[kt][e] * dp[kt][e]; }      // s = P from here on
         dsum += __shfl_xor(dsum, 16, WAVE);
         dsum += __shfl_xor(dsum, 32, WAVE);
-        s16x4 dsf[kMaxKT];
+        s16x4 dsf[NKT];
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt) {
+        for (int kt = 0; kt < NKT; ++kt) {
             uint32_t pw[2], dw[2];
 #pragma unroll
             for (int e = 0; e < 4; e += 2) {
@@ -180,23 +229,19 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
             }
         }
         // dQ^T = K^T dS^T: A = K^T (transpose load, contraction over keys), B = dS^T from registers
-        const int qrow = qt * 16 + r16;
+        uint2 dqv[FT];
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) {
             f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kt = 0; kt < kMaxKT; ++kt)
+            for (int kt = 0; kt < NKT; ++kt)
                 if (kt < nkt) o = DT::mfma16(tr16(Ks, DHP, kt * 16, ft * 16, lane), dsf[kt], o);
-            if (qrow < TQ) {
-                uint2 ov;
-                ov.x = (uint32_t)DT::from_f(o[0] * a.scale) | ((uint32_t)DT::from_f(o[1] * a.scale) << 16);
-                ov.y = (uint32_t)DT::from_f(o[2] * a.scale) | ((uint32_t)DT::from_f(o[3] * a.scale) << 16);
-                *reinterpret_cast<uint2*>(dqp + (int64_t)qrow * a.dq_rs + ft * 16 + 4 * g) = ov;
-            }
+            dqv[ft].x = (uint32_t)DT::from_f(o[0] * a.scale) | ((uint32_t)DT::from_f(o[1] * a.scale) << 16);
+            dqv[ft].y = (uint32_t)DT::from_f(o[2] * a.scale) | ((uint32_t)DT::from_f(o[3] * a.scale) << 16);
         }
         // dV^T += dO^T P, dK^T += Q^T dS: contraction over this tile's 16 queries, both operands transposed
 #pragma unroll
-        for (int kt = 0; kt < kMaxKT; ++kt) {
+        for (int kt = 0; kt < NKT; ++kt) {
             if (kt < nkt) {
                 const s16x4 pb = tr16(Ps, PP, 0, kt * 16, lane), db = tr16(dSs, PP, 0, kt * 16, lane);
 #pragma unroll
@@ -206,13 +251,14 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
                 }
             }
         }
-    }
-    u16* dkp = static_cast<u16*>(a.dk) + b * a.dk_bs + h * DH;
-    u16* dvp = static_cast<u16*>(a.dv) + b * a.dv_bs + h * DH;
+        // this tile's q rows have had their last read: dQ takes their place until the rows leave
 #pragma unroll
-    for (int kt = 0; kt < kMaxKT; ++kt) {
-        const int key = kt * 16 + r16;
-        if (kt < nkt && key < T) {
+        for (int ft = 0; ft < FT; ++ft) *reinterpret_cast<uint2*>(Qs + (qt * 16 + r16) * DHP + ft * 16 + 4 * g) = dqv[ft];
+    }
+    // dK and dV take the place of k and v (every read of them is behind this wave), then the rows leave together
+#pragma unroll
+    for (int kt = 0; kt < NKT; ++kt) {
+        if (kt < nkt) {
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 uint2 kv, vv;
@@ -220,11 +266,35 @@ __global__ __launch_bounds__(128) void attn_bwd_mfma_kernel(AttnBwdArgs a) {
                 kv.y = (uint32_t)DT::from_f(dkt[ft][kt][2] * a.scale) | ((uint32_t)DT::from_f(dkt[ft][kt][3] * a.scale) << 16);
                 vv.x = (uint32_t)DT::from_f(dvt[ft][kt][0]) | ((uint32_t)DT::from_f(dvt[ft][kt][1]) << 16);
                 vv.y = (uint32_t)DT::from_f(dvt[ft][kt][2]) | ((uint32_t)DT::from_f(dvt[ft][kt][3]) << 16);
-                *reinterpret_cast<uint2*>(dkp + (int64_t)key * a.dk_rs + ft * 16 + 4 * g) = kv;
-                *reinterpret_cast<uint2*>(dvp + (int64_t)key * a.dv_rs + ft * 16 + 4 * g) = vv;
+                *reinterpret_cast<uint2*>(Ks + (kt * 16 + r16) * DHP + ft * 16 + 4 * g) = kv;
+                *reinterpret_cast<uint2*>(Vs + (kt * 16 + r16) * DHP + ft * 16 + 4 * g) = vv;
             }
         }
     }
+    if (COOP) __syncthreads();
+    u16* outs[3] = {static_cast<u16*>(a.dq) + b * a.dq_bs + h0 * DH, static_cast<u16*>(a.dk) + b * a.dk_bs + h0 * DH,
+                    static_cast<u16*>(a.dv) + b * a.dv_bs + h0 * DH};
+    const int64_t ors[3] = {a.dq_rs, a.dk_rs, a.dv_rs};
+    const int orows[3] = {TQ, T, T}, ooffs[3] = {offs[0], offs[2], offs[3]};
+#pragma unroll
+    for (int mtx = 0; mtx < 3; ++mtx) {
+        int row = row_first, cp = cp_first;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            if (row < orows[mtx]) {
+                const uint4 v = *reinterpret_cast<const uint4*>(tile_of(cp / PPR) + ooffs[mtx] + row * DHP + (cp % PPR) * 8);
+                u16* dst = outs[mtx] + (int64_t)row * ors[mtx] + (cp / PPR) * DH + (cp % PPR) * 8;
+                if (a.out16) *reinterpret_cast<uint4*>(dst) = v;
+                else { *reinterpret_cast<uint2*>(dst) = make_uint2(v.x, v.y); *reinterpret_cast<uint2*>(dst + 4) = make_uint2(v.z, v.w); }
+            }
+            row += row_step; cp += cp_step;
+            if (cp >= rp) { cp -= rp; ++row; }
+        }
+    }
+    if (!more) break;
+    __syncthreads();                               // every thread is done reading the gradient tiles
+    b = b_next;
+  }
 }
 
 // fp32: one wave per (env, head); tiles in LDS, thread-per-element loops.  dh <= 48, T <= 48.
@@ -305,7 +375,7 @@ extern "C" int bsrl_attn_bwd(const void* q, int64_t q_bs, int64_t q_rs, const vo
     if (B * H > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_attn_bwd: too many (env, head) pairs");
     const double scale = 1.0 / sqrt((double)dh);
     AttnBwdArgs a{q, k, v, dout, q_bs, q_rs, k_bs, k_rs, v_bs, v_rs, do_bs, do_rs, key_bias, n_valid, dq, dk, dv,
-                  dq_bs, dq_rs, dk_bs, dk_rs, dv_bs, dv_rs, B, (int)T, (int)TQ, (int)H, (float)scale, 0};
+                  dq_bs, dq_rs, dk_bs, dk_rs, dv_bs, dv_rs, B, (int)T, (int)TQ, (int)H, (float)scale, 0, 0};
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (dtype == BSRL_F32) {
         if (dh > 48) return BSRL_UNSUPPORTED;
@@ -323,12 +393,32 @@ extern "C" int bsrl_attn_bwd(const void* q, int64_t q_bs, int64_t q_rs, const vo
         const int tp = (int)((T + 15) / 16) * 16, tqp = (int)((TQ + 15) / 16) * 16;
         a.wave_elems = (2 * tqp + 2 * tp) * dhp + 2 * 16 * (tp + 8);
         a.wave_elems = (a.wave_elems + 7) & ~7;                          // keep each wave's region 16-byte aligned
-        const size_t lds = (size_t)2 * a.wave_elems * sizeof(u16);        // <= 50 KB
-        const dim3 grid((unsigned)((B * H + 1) / 2)), block(128);
-#define AB_GO(DT, DH) hipLaunchKernelGGL((attn_bwd_mfma_kernel<DT, DH>), grid, block, lds, st, a)
-        if (dtype == BSRL_F16) { if (dh == 32) AB_GO(F16, 32); else AB_GO(F16, 48); }
-        else { if (dh == 32) AB_GO(BF16, 32); else AB_GO(BF16, 48); }
-#undef AB_GO
+        a.out16 = 1;
+        for (int64_t s : out_s) if (s % 8 != 0) a.out16 = 0;
+        if (!bsrl_aligned(dq, 16) || !bsrl_aligned(dk, 16) || !bsrl_aligned(dv, 16)) a.out16 = 0;
+        // one workgroup per env (wave = head) when the H heads' tiles fit twice into a CU's LDS
+        const size_t wave_bytes = (size_t)a.wave_elems * sizeof(u16);
+        // (T <= 32: with three key tiles the prefetched rows no longer fit the register file)
+        const bool coop = H <= 8 && T <= 32 && (size_t)H * wave_bytes <= 80 * 1024;
+        const size_t lds = (coop ? (size_t)H : 2) * wave_bytes;
+        // COOP workgroups are persistent (two resident per CU by LDS) and prefetch their next env
+        int cus = 256, dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+        const int64_t resident = (int64_t)cus * 2;
+        const dim3 grid(coop ? (unsigned)(B < resident ? B : resident) : (unsigned)((B * H + 1) / 2)), block(coop ? (unsigned)(64 * H) : 128u);
+#define AB_COOP(DT, DH) do { \
+            auto kern = attn_bwd_mfma_kernel<DT, DH, true, 2>; \
+            if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
+                (void)hipGetLastError(); return BSRL_UNSUPPORTED; } \
+            hipLaunchKernelGGL(kern, grid, block, lds, st, a); } while (0)
+#define AB_T(DT, DH) do { \
+            if (coop) AB_COOP(DT, DH); \
+            else if (T <= 32) hipLaunchKernelGGL((attn_bwd_mfma_kernel<DT, DH, false, 2>), grid, block, lds, st, a); \
+            else hipLaunchKernelGGL((attn_bwd_mfma_kernel<DT, DH, false, 3>), grid, block, lds, st, a); } while (0)
+        if (dtype == BSRL_F16) { if (dh == 32) AB_T(F16, 32); else AB_T(F16, 48); }
+        else { if (dh == 32) AB_T(BF16, 32); else AB_T(BF16, 48); }
+#undef AB_T
+#undef AB_COOP
     }
     BSRL_CHECK_LAUNCH("bsrl_attn_bwd");
     return BSRL_OK;

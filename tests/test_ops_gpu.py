@@ -525,6 +525,24 @@ def test_attention_backward(dtype, T, TQ, H, dh, mask):
     assert torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
 
 
+@pytest.mark.parametrize("TQ", [29, 5])
+def test_attention_backward_persistent_workgroups_walk_many_envs(TQ):
+    """More envs than resident workgroups: every workgroup of the one-workgroup-per-env form processes several envs
+    with the next one's rows prefetched.  An env's gradients depend on nothing but that env: the big batch must give the
+    bits of the same envs run in small batches."""
+    B, T, H, dh = 1500, 29, 4, 48
+    d = H * dh
+    qkv = _rand(B, T, 3 * d, dtype=torch.float16, seed=3)
+    dout = _rand(B, TQ, d, dtype=torch.float16, seed=4)
+    bias = (((torch.rand(B, T, generator=torch.Generator().manual_seed(6)) < 0.7).float() - 1.0) * 16384.0).half().to(DEV)
+    bias[:, :5] = 0
+    q, k, v = qkv[:, :TQ, :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+    dq, dk, dv = ops.attn_bwd(q, k, v, dout, H, key_bias=bias)
+    for lo, hi in ((0, 3), (510, 515), (1022, 1030), (1493, 1500)):
+        sq, sk, sv = ops.attn_bwd(q[lo:hi], k[lo:hi], v[lo:hi], dout[lo:hi], H, key_bias=bias[lo:hi])
+        assert torch.equal(sq, dq[lo:hi]) and torch.equal(sk, dk[lo:hi]) and torch.equal(sv, dv[lo:hi])
+
+
 # ---------------------------------------------------------------- weight-resident streaming linear
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rows,K,M", [(8192, 128, 128), (8200, 128, 384), (9001, 192, 192), (8193, 192, 576), (8192, 192, 776),
