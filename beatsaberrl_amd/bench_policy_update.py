@@ -50,10 +50,8 @@ def eager_update(policy, opt, obs, act, logp, adv, ret, scale=1.0, step=True):
     (loss * scale).backward()
     if not step:
         return loss.detach()
-    if scale != 1.0:
-        for p in policy.parameters():
-            if p.grad is not None:
-                p.grad.div_(scale)
+    if scale != 1.0:                  # unscale in one multi-tensor pass
+        torch._foreach_div_([p.grad for p in policy.parameters() if p.grad is not None], scale)
     nn.utils.clip_grad_norm_(policy.parameters(), MAX_GRAD_NORM)
     opt.step()
     _fl.bump_weights_version()
