@@ -525,6 +525,21 @@ def test_attention_backward(dtype, T, TQ, H, dh, mask):
     assert torch.equal(dq2, dq) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
 
 
+@pytest.mark.parametrize("TQ", [29, 5, 1])
+def test_attention_forward_persistent_workgroups_walk_many_envs(TQ):
+    """More envs than resident workgroups of the one-workgroup-per-env forward: an env's output must not depend on
+    which other envs share the launch."""
+    B, T, H, dh = 3300, 29, 4, 48
+    d = H * dh
+    qkv = _rand(B, T, 3 * d, dtype=torch.float16, seed=13)
+    bias = (((torch.rand(B, T, generator=torch.Generator().manual_seed(16)) < 0.7).float() - 1.0) * 16384.0).half().to(DEV)
+    bias[:, :5] = 0
+    q, k, v = qkv[:, :TQ, :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+    out = ops.attn_fwd(q, k, v, H, key_bias=bias)
+    for lo, hi in ((0, 3), (766, 771), (1534, 1540), (3293, 3300)):
+        assert torch.equal(ops.attn_fwd(q[lo:hi], k[lo:hi], v[lo:hi], H, key_bias=bias[lo:hi]), out[lo:hi])
+
+
 @pytest.mark.parametrize("TQ", [29, 5])
 def test_attention_backward_persistent_workgroups_walk_many_envs(TQ):
     """More envs than resident workgroups: every workgroup of the one-workgroup-per-env form processes several envs
