@@ -162,8 +162,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnArgs a) {
             for (int kt = 0; kt < kMaxKT; ++kt) if (kt < nkt) o = DT::mfma16(vf[kt][ft], pf[kt], o);
             if (qlive) {
                 uint2 ov;
-                ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
-                ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                ov.x = DT::pack2(o[0], o[1]);
+                ov.y = DT::pack2(o[2], o[3]);
                 *reinterpret_cast<uint2*>(op + (int64_t)qrow * (a.H * DH) + ft * 16 + g * 4) = ov;
             }
         }
@@ -200,7 +200,6 @@ __global__ __launch_bounds__(512) void attn_mfma_coop_kernel(AttnArgs a, int wav
     const int T = a.T, TQ = a.TQ, H = a.H;
     const int nkt = (T + 15) >> 4, nqt = (TQ + 15) >> 4;
     const int TP = nkt * 16, TQP = nqt * 16;
-    const int h = wave;
     u16* Qs = smem + (int64_t)wave * wave_elems;
     u16* Ks = Qs + TQP * DHP;
     u16* Vs = Ks + TP * DHP;
@@ -326,8 +325,8 @@ __global__ __launch_bounds__(512) void attn_mfma_coop_kernel(AttnArgs a, int wav
                 f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kt = 0; kt < NKT; ++kt) if (kt < nkt) o = DT::mfma16(vf[kt][ft], pf[kt], o);
-                ov[ft].x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
-                ov[ft].y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                ov[ft].x = DT::pack2(o[0], o[1]);
+                ov[ft].y = DT::pack2(o[2], o[3]);
             }
             // the query rows of this tile are in registers: the output takes their place until the rows leave
 #pragma unroll

@@ -40,7 +40,6 @@ struct AttnBwdArgs {
     int out16;                 // 16-bit path: gradient rows may leave as 16-byte pieces (else 8-byte)
 };
 
-constexpr int kMaxKT = 3;      // key tiles of 16 (T <= 48)
 typedef short s16x4v __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
 
@@ -219,8 +218,8 @@ __global__ __launch_bounds__(COOP ? 512 : 128) void attn_bwd_mfma_kernel(AttnBwd
 #pragma unroll
             for (int e = 0; e < 4; e += 2) {
                 const float d0 = s[kt][e] * (dp[kt][e] - dsum), d1 = s[kt][e + 1] * (dp[kt][e + 1] - dsum);
-                pw[e >> 1] = (uint32_t)DT::from_f(s[kt][e]) | ((uint32_t)DT::from_f(s[kt][e + 1]) << 16);
-                dw[e >> 1] = (uint32_t)DT::from_f(d0) | ((uint32_t)DT::from_f(d1) << 16);
+                pw[e >> 1] = DT::pack2(s[kt][e], s[kt][e + 1]);
+                dw[e >> 1] = DT::pack2(d0, d1);
             }
             dsf[kt] = __builtin_bit_cast(s16x4, make_uint2(dw[0], dw[1]));
             if (kt < nkt) {                     // row = the lane's query, 4 consecutive keys: one 8-byte LDS write each
@@ -236,8 +235,8 @@ __global__ __launch_bounds__(COOP ? 512 : 128) void attn_bwd_mfma_kernel(AttnBwd
 #pragma unroll
             for (int kt = 0; kt < NKT; ++kt)
                 if (kt < nkt) o = DT::mfma16(tr16(Ks, DHP, kt * 16, ft * 16, lane), dsf[kt], o);
-            dqv[ft].x = (uint32_t)DT::from_f(o[0] * a.scale) | ((uint32_t)DT::from_f(o[1] * a.scale) << 16);
-            dqv[ft].y = (uint32_t)DT::from_f(o[2] * a.scale) | ((uint32_t)DT::from_f(o[3] * a.scale) << 16);
+            dqv[ft].x = DT::pack2(o[0] * a.scale, o[1] * a.scale);
+            dqv[ft].y = DT::pack2(o[2] * a.scale, o[3] * a.scale);
         }
         // dV^T += dO^T P, dK^T += Q^T dS: contraction over this tile's 16 queries, both operands transposed
 #pragma unroll
@@ -262,10 +261,10 @@ __global__ __launch_bounds__(COOP ? 512 : 128) void attn_bwd_mfma_kernel(AttnBwd
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 uint2 kv, vv;
-                kv.x = (uint32_t)DT::from_f(dkt[ft][kt][0] * a.scale) | ((uint32_t)DT::from_f(dkt[ft][kt][1] * a.scale) << 16);
-                kv.y = (uint32_t)DT::from_f(dkt[ft][kt][2] * a.scale) | ((uint32_t)DT::from_f(dkt[ft][kt][3] * a.scale) << 16);
-                vv.x = (uint32_t)DT::from_f(dvt[ft][kt][0]) | ((uint32_t)DT::from_f(dvt[ft][kt][1]) << 16);
-                vv.y = (uint32_t)DT::from_f(dvt[ft][kt][2]) | ((uint32_t)DT::from_f(dvt[ft][kt][3]) << 16);
+                kv.x = DT::pack2(dkt[ft][kt][0] * a.scale, dkt[ft][kt][1] * a.scale);
+                kv.y = DT::pack2(dkt[ft][kt][2] * a.scale, dkt[ft][kt][3] * a.scale);
+                vv.x = DT::pack2(dvt[ft][kt][0], dvt[ft][kt][1]);
+                vv.y = DT::pack2(dvt[ft][kt][2], dvt[ft][kt][3]);
                 *reinterpret_cast<uint2*>(Ks + (kt * 16 + r16) * DHP + ft * 16 + 4 * g) = kv;
                 *reinterpret_cast<uint2*>(Vs + (kt * 16 + r16) * DHP + ft * 16 + 4 * g) = vv;
             }

@@ -45,7 +45,7 @@ struct BlkArgs {
 };
 
 template <typename DT> __device__ __forceinline__ uint32_t bpack2(float a, float b) {
-    return (uint32_t)DT::from_f(a) | ((uint32_t)DT::from_f(b) << 16);
+    return DT::pack2(a, b);
 }
 template <> __device__ __forceinline__ uint32_t bpack2<F16>(float a, float b) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));

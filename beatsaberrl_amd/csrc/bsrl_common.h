@@ -30,6 +30,13 @@ static inline bool bsrl_aligned(const void* p, size_t a) { return (reinterpret_c
 struct F16 {
     static __device__ __forceinline__ float to_f(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
     static __device__ __forceinline__ u16 from_f(float f) { return __builtin_bit_cast(u16, (_Float16)f); }
+    // two roundings in one instruction (v_cvt_pk_f16_f32, round to nearest even): a in the low half
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
     // D(16x16) += A(16x32) * B(32x16); lane l holds A[l%16][8*(l/16)..+7], B[8*(l/16)..+7][l%16],
     // D[4*(l/16)+i][l%16].
     static __device__ __forceinline__ f32x4 mfma32(s16x8 a, s16x8 b, f32x4 c) {
@@ -44,6 +51,12 @@ struct BF16 {
     static __device__ __forceinline__ float to_f(u16 v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
     // round to nearest even; gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32)
     static __device__ __forceinline__ u16 from_f(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {          // v_cvt_pk_bf16_f32
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    }
     static __device__ __forceinline__ f32x4 mfma32(s16x8 a, s16x8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
@@ -58,11 +71,15 @@ template <typename DT> __device__ __forceinline__ float io_load(const u16* p) { 
 template <typename DT> __device__ __forceinline__ void io_store(u16* p, float v) { *p = DT::from_f(v); }
 
 // ---- activations ---------------------------------------------------------------
+// max(x, 0) as ONE instruction (v_med3_f32 x, 0, +inf): fmaxf(x, 0) compiles to a canonicalising v_max_f32 x, x plus the
+// max itself, and the epilogues that apply it are bound by VALU issue.  Same value for every non-NaN x (-0 gives +0).
+__device__ __forceinline__ float relu1(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, __builtin_inff()); }
+
 __device__ __forceinline__ float gelu_exact(float x) {
     return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
 template <int ACT> __device__ __forceinline__ float apply_act(float x) {
-    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_RELU) return relu1(x);
     if (ACT == BSRL_ACT_GELU) return gelu_exact(x);
     return x;
 }
@@ -90,7 +107,7 @@ template <int ACT> __device__ __forceinline__ Act16Head act16_head(float x) {
     return h;
 }
 template <int ACT> __device__ __forceinline__ float act16_tail(float x, Act16Head h) {
-    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_RELU) return relu1(x);
     if (ACT == BSRL_ACT_GELU) {
         constexpr float L2E = 1.44269504088896340736f;
         constexpr float C0 = -1.59501576f * L2E, C1 = -7.40113019e-02f * L2E, C2 = 7.03035067e-04f * L2E;
@@ -109,7 +126,7 @@ __device__ __forceinline__ float keep_f32(float v) { asm("" : "+v"(v)); return v
 
 // activation for values about to be rounded to fp16 / bf16
 template <int ACT> __device__ __forceinline__ float apply_act16(float x) {
-    if (ACT == BSRL_ACT_RELU) return fmaxf(x, 0.0f);
+    if (ACT == BSRL_ACT_RELU) return relu1(x);
     if (ACT == BSRL_ACT_GELU) return gelu_fast(x);
     return x;
 }

@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void critic_pool_kernel(CpArgs a) {
                 for (int e = 0; e < 4; ++e) {
                     const float o0 = (v[8 * c + 2 * e] - mean) * rstd * wv[2 * e] + bv[2 * e];
                     const float o1 = (v[8 * c + 2 * e + 1] - mean) * rstd * wv[2 * e + 1] + bv[2 * e + 1];
-                    o[e] = (uint32_t)DT::from_f(o0) | ((uint32_t)DT::from_f(o1) << 16);
+                    o[e] = DT::pack2(o0, o1);
                 }
                 *reinterpret_cast<u32x4*>(rp + 8 * c) = o;
             }
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void critic_pool_kernel(CpArgs a) {
     const float inv = 1.0f / sum;
     u32x4 pf;                                               // B fragment of the pool: slot (g, j) = token 4 g + j | 16 + 4 g + (j - 4)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) pf[e] = (uint32_t)DT::from_f(p[2 * e] * inv) | ((uint32_t)DT::from_f(p[2 * e + 1] * inv) << 16);
+    for (int e = 0; e < 4; ++e) pf[e] = DT::pack2(p[2 * e] * inv, p[2 * e + 1] * inv);
     if (n16 >= H) pf = (u32x4){0u, 0u, 0u, 0u};
     // 4. pool: D[m = column 16 j + 4 g' + e][n = head]; A = hv^T through the transpose load, rows in the slot order above
     u16* out = a.pooled + (env * H + n16) * (int64_t)D;
@@ -178,8 +178,8 @@ __global__ __launch_bounds__(256) void critic_pool_kernel(CpArgs a) {
         const f32x4 o = DT::mfma32(af, __builtin_bit_cast(s16x8, pf), (f32x4){0.f, 0.f, 0.f, 0.f});
         if (n16 < H) {
             u32x2 ov;
-            ov[0] = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
-            ov[1] = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+            ov[0] = DT::pack2(o[0], o[1]);
+            ov[1] = DT::pack2(o[2], o[3]);
             *reinterpret_cast<u32x2*>(out + 16 * j + 4 * g) = ov;
         }
     }

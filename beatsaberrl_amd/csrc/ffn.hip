@@ -32,7 +32,7 @@ struct FfnArgs {
 };
 
 template <typename DT> __device__ __forceinline__ uint32_t pk2(float a, float b) {
-    return (uint32_t)DT::from_f(a) | ((uint32_t)DT::from_f(b) << 16);
+    return DT::pack2(a, b);
 }
 
 template <typename DT, int D, int RT, int ACT>

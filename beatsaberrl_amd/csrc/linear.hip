@@ -160,8 +160,8 @@ __global__ __launch_bounds__(256) void linear_mfma_vec_kernel(LinArgs a) {
                 *reinterpret_cast<float4*>(static_cast<float*>(a.y) + lin_yoff(a, row) + col) = make_float4(o[0], o[1], o[2], o[3]);
             } else {
                 uint2 ov;
-                ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
-                ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                ov.x = DT::pack2(o[0], o[1]);
+                ov.y = DT::pack2(o[2], o[3]);
                 *reinterpret_cast<uint2*>(static_cast<u16*>(a.y) + lin_yoff(a, row) + col) = ov;
             }
         }

@@ -61,9 +61,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // clobber: what orders these asynchronous LDS writes against the fragment reads is the vmcnt wait + barrier of the
 // stage loop (both compiler barriers), never program order - and with the clobber the compiler kept every fragment
 // read behind the load issued before it, one LDS latency per MFMA group.  volatile keeps the loads in order among
-// themselves and against the waits.
+// themselves and against the waits.  m0 is written without telling the compiler (it rejects reserved registers in a clobber
+// list): nothing else in this kernel uses it - no dynamically indexed register arrays, no LDS instruction that needs it.
 __device__ __forceinline__ void frag_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr));
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(256 * WC, (Geo<WC, BK, NS, CT>::WG_PER_CU)) void li
             if (col_ok && row < a.rows) {
                 u32x4 ov;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ov[e] = (uint32_t)DT::from_f(v[2 * e]) | ((uint32_t)DT::from_f(v[2 * e + 1]) << 16);
+                for (int e = 0; e < 4; ++e) ov[e] = DT::pack2(v[2 * e], v[2 * e + 1]);
                 *reinterpret_cast<u32x4*>(y + lin_yoff(a, row) + colw) = ov;
             }
         }

@@ -148,8 +148,8 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
                     if (!(DT::to_f((u16)(gv.y >> 16)) > 0.f)) o[3] = 0.f;
                 }
                 uint2 ov;
-                ov.x = (uint32_t)DT::from_f(o[0]) | ((uint32_t)DT::from_f(o[1]) << 16);
-                ov.y = (uint32_t)DT::from_f(o[2]) | ((uint32_t)DT::from_f(o[3]) << 16);
+                ov.x = DT::pack2(o[0], o[1]);
+                ov.y = DT::pack2(o[2], o[3]);
                 *reinterpret_cast<uint2*>(wt + r16 * TP + mt * 16 + 4 * g) = ov;
             }
             // the tile leaves row-major: 16-byte pieces, consecutive lanes on consecutive pieces of a row

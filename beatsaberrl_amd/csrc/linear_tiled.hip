@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256, 2) void linear_tiled_kernel(LinArgs a) {
                         if (!(DT::to_f((u16)(gv.y >> 16)) > 0.f)) v[3] = 0.f;
                     }
                     uint2 ov;
-                    ov.x = (uint32_t)DT::from_f(v[0]) | ((uint32_t)DT::from_f(v[1]) << 16);
-                    ov.y = (uint32_t)DT::from_f(v[2]) | ((uint32_t)DT::from_f(v[3]) << 16);
+                    ov.x = DT::pack2(v[0], v[1]);
+                    ov.y = DT::pack2(v[2], v[3]);
                     *reinterpret_cast<uint2*>(y + lin_yoff(a, row) + col) = ov;
                 }
             }
