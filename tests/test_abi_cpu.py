@@ -92,6 +92,12 @@ def test_new_entry_points_reject_bad_arguments_without_a_device(lib):
                                                       16, 96, 96, 16, 96, 96, 16, 96, 96, 4, T, TQ, 1, dh, dt, None)
     assert ab(29, 30, 32, _lib.F16) == -1 and ab(29, 29, 32, _lib.F16, q=None) == -1
     assert ab(49, 5, 32, _lib.F16) == 1 and ab(29, 5, 40, _lib.F16) == 1 and ab(29, 5, 64, _lib.F32) == 1      # unsupported shapes
+    # critic pool: null pointers, heads that do not divide d, shapes outside the MFMA form (reported as unsupported)
+    cp = lambda T, d, H, dt, x=16, B=4: lib.bsrl_critic_pool(x, 16, 16, C.c_float(1e-5), 16, None, 16, B, T, d, H, dt, None)
+    assert cp(29, 192, 4, _lib.F16, x=None) == -1 and b"null" in lib.bsrl_last_error()
+    assert cp(29, 192, 5, _lib.F16) == -1 and cp(0, 192, 4, _lib.F16) == -1 and cp(29, 192, 4, 9) == -1
+    assert cp(29, 192, 4, _lib.F32) == 1 and cp(33, 192, 4, _lib.F16) == 1 and cp(29, 96, 3, _lib.F16) == 1
+    assert cp(29, 192, 4, _lib.F16, B=0) == 0
     # grouped linear: the group must divide the rows, fit its stride and exclude a split output
     g = lambda rows, grp, gs, y2=None, split=0: lib.bsrl_linear_grouped(
         16, 8, 16, None, None, 0, 16, 8, y2, 8 if y2 else 0, split, rows, 8, 8, 0, _lib.F16, _lib.F16, grp, gs, None)
