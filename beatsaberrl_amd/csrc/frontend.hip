@@ -67,9 +67,37 @@ __global__ __launch_bounds__(256) void note_frontend_kernel(FrontArgs a) {
 
     for (int i = tid; i < 2 * SABER_FEAT; i += 256) s_sab[i] = a.saber_idx[i];
     for (int i = tid; i < TORSO_FEAT + 2 * LEG_FEAT; i += 256) s_body[i] = a.body_idx[i];
-    for (int i = tid; i < nenv * OBS_DIM; i += 256) {
-        const int e = i / OBS_DIM, c = i - e * OBS_DIM;
-        so[e][c] = io::round(load_obs(a.obs, (b0 + e) * a.obs_ld + c, a.obs_dtype));
+    // dense fp32 rows (the rollout's obs buffer): the workgroup's 8 rows are one contiguous, 16-byte aligned block -
+    // every 16-byte load of a thread is issued before the first LDS write.  The general loop below pays one memory
+    // round trip per element (the dtype switch keeps its loads apart): 20 of them per thread.
+    if (a.obs_dtype == BSRL_F32 && a.obs_ld == OBS_DIM && nenv == EPB && (reinterpret_cast<uintptr_t>(a.obs) & 15) == 0) {
+        constexpr int NP = EPB * OBS_DIM / 4, NITF = (NP + 255) / 256;
+        static_assert(EPB * OBS_DIM % 4 == 0, "a workgroup's obs block is a whole number of 16-byte pieces");
+        const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(a.obs) + b0 * OBS_DIM);
+        float4 v[NITF];
+#pragma unroll
+        for (int it = 0; it < NITF; ++it) {
+            const int p = it * 256 + tid;
+            v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p < NP) v[it] = src[p];
+        }
+#pragma unroll
+        for (int it = 0; it < NITF; ++it) {
+            const int p = it * 256 + tid;
+            if (p < NP) {
+                const float f[4] = {v[it].x, v[it].y, v[it].z, v[it].w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int i = 4 * p + k, e = i / OBS_DIM, c = i - e * OBS_DIM;
+                    so[e][c] = io::round(f[k]);
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < nenv * OBS_DIM; i += 256) {
+            const int e = i / OBS_DIM, c = i - e * OBS_DIM;
+            so[e][c] = io::round(load_obs(a.obs, (b0 + e) * a.obs_ld + c, a.obs_dtype));
+        }
     }
     __syncthreads();
 
