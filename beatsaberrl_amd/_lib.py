@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -65,6 +65,7 @@ SIGNATURES = {
     "bsrl_blocks_pack": (_i32, [C.POINTER(BlocksDesc), C.POINTER(BlocksParams), _p, _p]),
     "bsrl_blocks_forward": (_i32, [C.POINTER(BlocksDesc), _p, _p, _p, _p, _p, _i64, _p]),
     "bsrl_note_frontend": (_i32, [_p, _i64, _i32, _p, _p, _i32, _i32, _f, _p, _p, _p, _p, _p, _i64, _i32, _p]),
+    "bsrl_note_frontend_padded": (_i32, [_p, _i64, _i32, _p, _p, _i32, _i32, _f, _p, _p, _p, _p, _p, _i64, _i32, _p]),
     "bsrl_counter_add": (_i32, [_p, C.c_uint64, _p]),
     "bsrl_sample_heads": (_i32, [_p, _i64, _i64, _i64, _p, _p, C.c_uint64, C.c_uint64, _p, _p, _i32,
                                  _p, _p, _p, _p, _p, _p]),

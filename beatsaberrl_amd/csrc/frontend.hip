@@ -23,6 +23,7 @@ constexpr int SABER_FEAT = 47, TORSO_FEAT = 29, LEG_FEAT = 32, N_LEAD = 5, T_TOK
 constexpr int S_WPOS = 15, S_WVEL = 18, S_BLADE = 21, S_TIPV = 44;
 constexpr float X_NORM = 1.0f, Y_NORM = 0.75f, Z_SCALE = 8.0f, V_NORM = 6.0f, HANDLE_LEN = 0.16f;
 constexpr float MASK_BIAS = 16384.0f;
+constexpr int PITCH = 64;                      // row pitch of the padded encoder inputs
 
 struct FrontArgs {
     const void* obs; int64_t obs_ld; int obs_dtype;
@@ -55,7 +56,7 @@ struct V3 { float x, y, z; };
 __device__ __forceinline__ float dot3(V3 a, V3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
 __device__ __forceinline__ float norm3(V3 a) { return sqrtf(dot3(a, a)); }
 
-template <typename IO>
+template <typename IO, bool PAD>
 __global__ __launch_bounds__(256) void note_frontend_kernel(FrontArgs a) {
     typedef FIO<IO> io;
     __shared__ float so[EPB][OBS_DIM + 2];
@@ -150,26 +151,32 @@ __global__ __launch_bounds__(256) void note_frontend_kernel(FrontArgs a) {
     }
 
     // ---- stores: each output tensor is contiguous over the workgroup's envs ----
+    // PAD: every encoder-input row is PITCH elements long, zero past its natural width, so the first encoder
+    // Linear runs as a K = PITCH GEMM on the vector kernels (zeros add nothing to the fp32 accumulators)
     constexpr int SAB_W = SABER_FEAT + 2, LEG_W = LEG_FEAT + 2;
-    for (int i = tid; i < nenv * 2 * SAB_W; i += 256) {            // (B, 2, 49): 47 lanes + hand one-hot
-        const int e = i / (2 * SAB_W), r = i - e * 2 * SAB_W, hand = r / SAB_W, c = r - hand * SAB_W;
-        const float v = c < SABER_FEAT ? so[e][s_sab[hand * SABER_FEAT + c]] : (c - SABER_FEAT == hand ? 1.f : 0.f);
-        io::st(a.saber_in, b0 * 2 * SAB_W + i, v);
+    constexpr int SAB_P = PAD ? PITCH : SAB_W, TOR_P = PAD ? PITCH : TORSO_FEAT, LEG_P = PAD ? PITCH : LEG_W;
+    for (int i = tid; i < nenv * 2 * SAB_P; i += 256) {            // (B, 2, 49): 47 lanes + hand one-hot
+        const int e = i / (2 * SAB_P), r = i - e * 2 * SAB_P, hand = r / SAB_P, c = r - hand * SAB_P;
+        const float v = c < SABER_FEAT ? so[e][s_sab[hand * SABER_FEAT + c]]
+                                       : (c < SAB_W && c - SABER_FEAT == hand ? 1.f : 0.f);
+        io::st(a.saber_in, b0 * 2 * SAB_P + i, v);
     }
-    for (int i = tid; i < nenv * TORSO_FEAT; i += 256) {           // (B, 29)
-        const int e = i / TORSO_FEAT, c = i - e * TORSO_FEAT;
-        io::st(a.torso_in, b0 * TORSO_FEAT + i, so[e][s_body[c]]);
+    for (int i = tid; i < nenv * TOR_P; i += 256) {                // (B, 29)
+        const int e = i / TOR_P, c = i - e * TOR_P;
+        io::st(a.torso_in, b0 * TOR_P + i, c < TORSO_FEAT ? so[e][s_body[c]] : 0.f);
     }
-    for (int i = tid; i < nenv * 2 * LEG_W; i += 256) {            // (B, 2, 34): 32 lanes + side one-hot
-        const int e = i / (2 * LEG_W), r = i - e * 2 * LEG_W, side = r / LEG_W, c = r - side * LEG_W;
-        const float v = c < LEG_FEAT ? so[e][s_body[TORSO_FEAT + side * LEG_FEAT + c]] : (c - LEG_FEAT == side ? 1.f : 0.f);
-        io::st(a.leg_in, b0 * 2 * LEG_W + i, v);
+    for (int i = tid; i < nenv * 2 * LEG_P; i += 256) {            // (B, 2, 34): 32 lanes + side one-hot
+        const int e = i / (2 * LEG_P), r = i - e * 2 * LEG_P, side = r / LEG_P, c = r - side * LEG_P;
+        const float v = c < LEG_FEAT ? so[e][s_body[TORSO_FEAT + side * LEG_FEAT + c]]
+                                     : (c < LEG_W && c - LEG_FEAT == side ? 1.f : 0.f);
+        io::st(a.leg_in, b0 * 2 * LEG_P + i, v);
     }
     const int NW = NOTE_FEAT + (a.note_geo ? GEO_FEAT : 0);
-    for (int i = tid; i < nenv * N_SLOTS * NW; i += 256) {         // (B, 24, 18 | 40)
-        const int p = i / NW, c = i - p * NW, e = p / N_SLOTS, s = p - e * N_SLOTS;
-        const float v = c < NOTE_FEAT ? so[e][OFF_NOTES + s * NOTE_FEAT + c] : sgeo[e][s][c - NOTE_FEAT];
-        io::st(a.note_in, b0 * N_SLOTS * NW + i, v);
+    const int NP_ = PAD ? PITCH : NW;
+    for (int i = tid; i < nenv * N_SLOTS * NP_; i += 256) {        // (B, 24, 18 | 40)
+        const int p = i / NP_, c = i - p * NP_, e = p / N_SLOTS, s = p - e * N_SLOTS;
+        const float v = c < NOTE_FEAT ? so[e][OFF_NOTES + s * NOTE_FEAT + c] : (c < NW ? sgeo[e][s][c - NOTE_FEAT] : 0.f);
+        io::st(a.note_in, b0 * N_SLOTS * NP_ + i, v);
     }
     for (int i = tid; i < nenv * T_TOK; i += 256) {                // (B, 29): lead tokens always attendable
         const int e = i / T_TOK, t = i - e * T_TOK;
@@ -180,26 +187,53 @@ __global__ __launch_bounds__(256) void note_frontend_kernel(FrontArgs a) {
 
 }  // namespace
 
-extern "C" int bsrl_note_frontend(const void* obs, int64_t obs_ld, int obs_dtype,
-                                  const int32_t* saber_idx, const int32_t* body_idx,
-                                  int note_geo, int flux, float z_asinh,
-                                  void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
-                                  int64_t B, int dtype, bsrl_stream stream) {
+namespace {
+
+int frontend_launch(const char* who, bool pad, const void* obs, int64_t obs_ld, int obs_dtype,
+                    const int32_t* saber_idx, const int32_t* body_idx, int note_geo, int flux, float z_asinh,
+                    void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
+                    int64_t B, int dtype, bsrl_stream stream) {
     if (!obs || !saber_idx || !body_idx || !saber_in || !torso_in || !leg_in || !note_in || !key_bias)
-        BSRL_FAIL(BSRL_EINVAL, "bsrl_note_frontend: null pointer");
-    if (B < 0 || obs_ld < OBS_DIM) BSRL_FAIL(BSRL_EINVAL, "bsrl_note_frontend: B < 0 or obs_ld < %d", OBS_DIM);
-    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_note_frontend: bad dtype %d", dtype);
+        BSRL_FAIL(BSRL_EINVAL, "%s: null pointer", who);
+    if (B < 0 || obs_ld < OBS_DIM) BSRL_FAIL(BSRL_EINVAL, "%s: B < 0 or obs_ld < %d", who, OBS_DIM);
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "%s: bad dtype %d", who, dtype);
     if (obs_dtype != BSRL_F32 && obs_dtype != dtype)
-        BSRL_FAIL(BSRL_EINVAL, "bsrl_note_frontend: obs must be fp32 or already in the stream dtype");
-    if (!(z_asinh > 0.f)) BSRL_FAIL(BSRL_EINVAL, "bsrl_note_frontend: z_asinh must be > 0");
+        BSRL_FAIL(BSRL_EINVAL, "%s: obs must be fp32 or already in the stream dtype", who);
+    if (!(z_asinh > 0.f)) BSRL_FAIL(BSRL_EINVAL, "%s: z_asinh must be > 0", who);
     if (B == 0) return BSRL_OK;
     FrontArgs a{obs, obs_ld, obs_dtype, saber_idx, body_idx, note_geo != 0, flux != 0, z_asinh,
                 saber_in, torso_in, leg_in, note_in, key_bias, B};
     const dim3 grid((unsigned)((B + EPB - 1) / EPB)), block(256);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == BSRL_F32) hipLaunchKernelGGL(note_frontend_kernel<F32IO>, grid, block, 0, st, a);
-    else if (dtype == BSRL_F16) hipLaunchKernelGGL(note_frontend_kernel<F16>, grid, block, 0, st, a);
-    else hipLaunchKernelGGL(note_frontend_kernel<BF16>, grid, block, 0, st, a);
-    BSRL_CHECK_LAUNCH("bsrl_note_frontend");
+#define BSRL_FRONT(IO)                                                                   \
+    do {                                                                                 \
+        if (pad) hipLaunchKernelGGL((note_frontend_kernel<IO, true>), grid, block, 0, st, a);  \
+        else hipLaunchKernelGGL((note_frontend_kernel<IO, false>), grid, block, 0, st, a);     \
+    } while (0)
+    if (dtype == BSRL_F32) BSRL_FRONT(F32IO);
+    else if (dtype == BSRL_F16) BSRL_FRONT(F16);
+    else BSRL_FRONT(BF16);
+#undef BSRL_FRONT
+    BSRL_CHECK_LAUNCH(who);
     return BSRL_OK;
+}
+
+}  // namespace
+
+extern "C" int bsrl_note_frontend(const void* obs, int64_t obs_ld, int obs_dtype,
+                                  const int32_t* saber_idx, const int32_t* body_idx,
+                                  int note_geo, int flux, float z_asinh,
+                                  void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
+                                  int64_t B, int dtype, bsrl_stream stream) {
+    return frontend_launch("bsrl_note_frontend", false, obs, obs_ld, obs_dtype, saber_idx, body_idx, note_geo, flux,
+                           z_asinh, saber_in, torso_in, leg_in, note_in, key_bias, B, dtype, stream);
+}
+
+extern "C" int bsrl_note_frontend_padded(const void* obs, int64_t obs_ld, int obs_dtype,
+                                         const int32_t* saber_idx, const int32_t* body_idx,
+                                         int note_geo, int flux, float z_asinh,
+                                         void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
+                                         int64_t B, int dtype, bsrl_stream stream) {
+    return frontend_launch("bsrl_note_frontend_padded", true, obs, obs_ld, obs_dtype, saber_idx, body_idx, note_geo,
+                           flux, z_asinh, saber_in, torso_in, leg_in, note_in, key_bias, B, dtype, stream);
 }

@@ -106,6 +106,22 @@ def _replica(w: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return cache[1]
 
 
+def _replica_padded(w: torch.Tensor, dtype: torch.dtype, k_pad: int) -> torch.Tensor:
+    """_replica with the (M, K) weight's columns zero-padded to k_pad: the operand of a Linear whose input
+    rows arrive padded the same way.  Refreshed in place like _replica."""
+    M, K = w.shape
+    cache = getattr(w, "_bsrl_replica_padded", None)
+    if cache is None or cache[1].dtype is not dtype or cache[1].device != w.device or cache[1].shape[1] != k_pad:
+        wp = torch.zeros(M, k_pad, device=w.device, dtype=dtype)
+        wp[:, :K].copy_(w.detach())
+        cache = [_weights_version, wp]
+        w._bsrl_replica_padded = cache
+    elif cache[0] != _weights_version:
+        cache[1][:, :K].copy_(w.detach())
+        cache[0] = _weights_version
+    return cache[1]
+
+
 def packed_halves(ms, dtype=torch.float16):
     """(w_cat in `dtype`, b_cat fp32) for an ordered group of same-input Linears."""
     key = ms[0].weight

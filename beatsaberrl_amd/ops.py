@@ -394,10 +394,15 @@ def cfg_embed(obs, wp, bp, wo, bo, T, dtype):
     return tokens
 
 
-def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z_asinh=8.0):
+FRONT_PITCH = 64        # row pitch of note_frontend's padded encoder inputs
+
+
+def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z_asinh=8.0, padded=False):
     """obs (B, 630) fp32 or `dtype` -> (saber_in (B, 2, 49), torso_in (B, 29), leg_in (B, 2, 34),
     note_in (B, 24, 18 | 40), key_bias (B, 29)), all in `dtype`: the forward's preamble in one
-    kernel (obs rounding, lane gathers, note-geometry lanes, one-hots, key bias)."""
+    kernel (obs rounding, lane gathers, note-geometry lanes, one-hots, key bias).  padded=True: every
+    encoder-input row is 64 wide, zero past its natural width (for a first Linear whose weight columns
+    are padded the same way)."""
     _need_cuda(obs, saber_idx, body_idx)
     if obs.dim() != 2 or obs.shape[1] != 630 or obs.stride(1) != 1:
         raise RuntimeError(f"note_frontend: obs must be (B, 630) with unit last stride, got {tuple(obs.shape)}")
@@ -408,14 +413,20 @@ def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z
         raise TypeError("note_frontend: saber_idx (94) / body_idx (93) must be contiguous int32 tables")
     B = obs.shape[0]
     mk = lambda *s: torch.empty(*s, device=obs.device, dtype=dtype)
-    saber_in, torso_in, leg_in = mk(B, 2, 49), mk(B, 29), mk(B, 2, 34)
-    note_in, key_bias = mk(B, 24, 40 if note_geo else 18), mk(B, 29)
+    if padded:
+        saber_in, torso_in, leg_in, note_in = mk(B, 2, FRONT_PITCH), mk(B, FRONT_PITCH), mk(B, 2, FRONT_PITCH), mk(B, 24, FRONT_PITCH)
+    else:
+        saber_in, torso_in, leg_in = mk(B, 2, 49), mk(B, 29), mk(B, 2, 34)
+        note_in = mk(B, 24, 40 if note_geo else 18)
+    key_bias = mk(B, 29)
+    lib = _lib.load()
+    entry = lib.bsrl_note_frontend_padded if padded else lib.bsrl_note_frontend
     with torch.cuda.device(obs.device):
-        rc = _lib.load().bsrl_note_frontend(obs.data_ptr(), obs.stride(0), dt_code(obs.dtype), saber_idx.data_ptr(),
+        rc = entry(obs.data_ptr(), obs.stride(0), dt_code(obs.dtype), saber_idx.data_ptr(),
                                             body_idx.data_ptr(), int(bool(note_geo)), int(bool(flux)), float(z_asinh),
                                             saber_in.data_ptr(), torso_in.data_ptr(), leg_in.data_ptr(),
                                             note_in.data_ptr(), key_bias.data_ptr(), B, dt_code(dtype), _stream(obs))
-    _lib.check(rc, "bsrl_note_frontend")
+    _lib.check(rc, "bsrl_note_frontend_padded" if padded else "bsrl_note_frontend")
     return saber_in, torso_in, leg_in, note_in, key_bias
 
 

@@ -73,7 +73,8 @@ def _lin(m: nn.Linear, x, act=None, residual=None, out=None):
 def _seq(seq: nn.Sequential, x, out=None):
     """Linear (ReLU Linear)* with each ReLU in its producer's epilogue (reference
     python/policy.py:76-145, `_seq` / `_run`).  out: a (N, G, M) slice of the token stream that
-    receives the last Linear's rows directly."""
+    receives the last Linear's rows directly.  x may be wider than the first Linear's input (rows
+    zero-padded by the producer): the first weight's columns are then padded to match."""
     ms = list(seq)
     i = 0
     while i < len(ms):
@@ -82,7 +83,13 @@ def _seq(seq: nn.Sequential, x, out=None):
             raise RuntimeError(f"unsupported module in Sequential: {type(m).__name__}")
         relu = i + 1 < len(ms) and isinstance(ms[i + 1], nn.ReLU)
         last = i + (2 if relu else 1) >= len(ms)
-        x = _lin(m, x, act="relu" if relu else None, out=out if last else None)
+        if x.shape[-1] != m.in_features:
+            if i or x.shape[-1] < m.in_features or x.dtype is torch.float32:
+                raise RuntimeError(f"_seq: input has {x.shape[-1]} lanes, the Linear takes {m.in_features}")
+            x = ops.linear(x, _fl._replica_padded(m.weight, x.dtype, x.shape[-1]), _fl._bias32(m.bias),
+                           act="relu" if relu else None, out=out if last else None)
+        else:
+            x = _lin(m, x, act="relu" if relu else None, out=out if last else None)
         i += 2 if relu else 1
     return x
 
@@ -434,7 +441,8 @@ class NotePolicy(nn.Module):
     def refresh_fp16_caches(self):
         """Force every weight copy the kernels read up to date for the current weights version
         (python/policy.py:1448-1461): call after optimizer steps under a captured graph.  On the
-        16-bit stream these are the replicas and the fused block image; on the fp32 stream only
+        16-bit stream these are the replicas (the encoders' column-padded first-layer copies among
+        them) and the fused block image; on the fp32 stream only
         the concatenated q|k|v / k|v / head matrices (single Linears read the masters)."""
         dt = self.stream_dtype if self.fp16 else torch.float32
         if self.fused_blocks_ok(dt):
@@ -443,6 +451,8 @@ class NotePolicy(nn.Module):
             for m in self.modules():
                 if isinstance(m, nn.Linear):
                     _fl._replica(m.weight, dt)
+            for enc in (self.saber_mlp, self.torso_mlp, self.leg_mlp, self.note_mlp):   # padded first-layer copies
+                _fl._replica_padded(enc[0].weight, dt, ops.FRONT_PITCH)
         for blk in self.blocks:
             _fl.packed_halves([blk.q_proj, blk.k_proj, blk.v_proj], dt)
             _fl.packed_halves([blk.k_proj, blk.v_proj], dt)
@@ -492,7 +502,9 @@ class NotePolicy(nn.Module):
             obs = obs.contiguous()
         sab_in, torso_in, leg_in, note_in, attn_bias = ops.note_frontend(
             obs, self._saber_idx32, self._body_idx32, dt, note_geo=self.note_geo, flux=self.game == "flux",
-            z_asinh=self.z_asinh)
+            z_asinh=self.z_asinh, padded=dt is not torch.float32)
+        # 16-bit streams: the encoder inputs arrive 64 lanes wide (zero past 49 / 29 / 34 / 40), so each first
+        # Linear is a K = 64 GEMM on the vector kernels instead of an odd-K one on the element-wise path.
         # every encoder writes its tokens straight into their rows of the (B, 29, d) stream
         # [saber_L, saber_R, torso, leg_L, leg_R, notes...] (the reference concatenates, policy.py:1247-1249)
         x = torch.empty(B, self.n_lead + N_NOTE_SLOTS, d, device=obs.device, dtype=dt)

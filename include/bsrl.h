@@ -222,6 +222,18 @@ int bsrl_note_frontend(const void* obs, int64_t obs_ld, int obs_dtype,
                        void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
                        int64_t B, int dtype, bsrl_stream stream);
 
+/* The same pass with every encoder-input row written at a pitch of 64 elements,
+ * zero past its natural width: saber_in (B, 2, 64), torso_in (B, 64), leg_in
+ * (B, 2, 64), note_in (B, 24, 64).  The first Linear of each encoder MLP
+ * (python/policy.py:1231-1246) then runs as a K = 64 GEMM against a weight whose
+ * columns are zero-padded the same way; the zero lanes add nothing to the fp32
+ * accumulators, so the tokens are the ones the unpadded route produces. */
+int bsrl_note_frontend_padded(const void* obs, int64_t obs_ld, int obs_dtype,
+                              const int32_t* saber_idx, const int32_t* body_idx,
+                              int note_geo, int flux, float z_asinh,
+                              void* saber_in, void* torso_in, void* leg_in, void* note_in, void* key_bias,
+                              int64_t B, int dtype, bsrl_stream stream);
+
 /* ---- Action epilogue ---------------------------------------------------------
  * log-softmax + Gumbel-max sampling + summed log-probability + per-head entropy
  * on the fp32 logits (B, n_heads, K), K <= 8, n_heads <= 32.  Replaces the tail

@@ -50,16 +50,17 @@ def test_new_entry_points_reject_bad_arguments_without_a_device(lib):
     C = ctypes
     # front end: null pointers, short rows, obs dtype that is neither fp32 nor the stream dtype, bad z scale
     args = [16, 630, _lib.F32, 16, 16, 1, 0, C.c_float(8.0), 16, 16, 16, 16, 16, 4, _lib.F16, None]
-    bad = list(args); bad[0] = None
-    assert lib.bsrl_note_frontend(*bad) == -1 and b"null" in lib.bsrl_last_error()
-    bad = list(args); bad[1] = 629
-    assert lib.bsrl_note_frontend(*bad) == -1
-    bad = list(args); bad[2] = _lib.BF16
-    assert lib.bsrl_note_frontend(*bad) == -1 and b"stream dtype" in lib.bsrl_last_error()
-    bad = list(args); bad[7] = C.c_float(0.0)
-    assert lib.bsrl_note_frontend(*bad) == -1
-    ok = list(args); ok[13] = 0
-    assert lib.bsrl_note_frontend(*ok) == 0                     # B == 0: nothing to do
+    for entry in (lib.bsrl_note_frontend, lib.bsrl_note_frontend_padded):
+        bad = list(args); bad[0] = None
+        assert entry(*bad) == -1 and b"null" in lib.bsrl_last_error()
+        bad = list(args); bad[1] = 629
+        assert entry(*bad) == -1
+        bad = list(args); bad[2] = _lib.BF16
+        assert entry(*bad) == -1 and b"stream dtype" in lib.bsrl_last_error()
+        bad = list(args); bad[7] = C.c_float(0.0)
+        assert entry(*bad) == -1
+        ok = list(args); ok[13] = 0
+        assert entry(*ok) == 0                                  # B == 0: nothing to do
     # action epilogue: K and head-count limits, sampling without an output
     assert lib.bsrl_sample_heads(16, 4, 29, 9, None, None, 0, 0, None, None, 0, 16, 16, None, None, None, None) == -1
     assert lib.bsrl_sample_heads(16, 4, 33, 7, None, None, 0, 0, None, None, 0, 16, 16, None, None, None, None) == -1

@@ -66,6 +66,26 @@ def test_frontend_matches_oracle(dtype, geo, flux, B):
             assert (gg == wg).float().mean().item() >= 0.99
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("geo", [False, True])
+@pytest.mark.parametrize("B", [1, 13, 1000])
+def test_frontend_padded_rows_hold_the_same_lanes_and_zeros(dtype, geo, B):
+    """The 64-pitch outputs carry the unpadded outputs' bits in their leading lanes and zeros after them (the
+    buffers are poisoned first: every pad lane must be written)."""
+    obs = _obs(B, 300 + B).to(DEV)
+    sab, body = _tables()
+    want = ops.note_frontend(obs, sab, body, TDT[dtype], note_geo=geo, flux=geo)
+    junk = torch.full((B * 6 * 24 * 64,), float("nan"), device=DEV, dtype=TDT[dtype])
+    del junk                                                           # the allocator hands these bytes out next
+    got = ops.note_frontend(obs, sab, body, TDT[dtype], note_geo=geo, flux=geo, padded=True)
+    for name, g_, w_ in zip(("saber_in", "torso_in", "leg_in", "note_in"), got, want):
+        assert g_.shape == (*w_.shape[:-1], ops.FRONT_PITCH), name
+        k = w_.shape[-1]
+        assert torch.equal(g_[..., :k], w_), name
+        assert bool((g_[..., k:] == 0).all()), name
+    assert torch.equal(got[4], want[4])
+
+
 def test_frontend_prerounded_and_strided_obs():
     """fp32 obs and obs already in the stream dtype give the same bits (python/policy.py:1200-1209);
     a row stride larger than 630 is honoured."""

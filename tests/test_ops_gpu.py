@@ -143,7 +143,7 @@ def test_linear_strided_views_split_and_packing(dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rows,K,M", [(4096, 128, 128), (5000, 128, 384), (4097, 384, 1152), (8192, 1536, 384),
                                       (6000, 192, 576), (4100, 40, 192), (9000, 256, 1024), (4099, 128, 136),
-                                      (4200, 96, 1024), (4500, 512, 1280)])
+                                      (4200, 96, 1024), (4500, 512, 1280), (4300, 64, 192), (5000, 64, 256)])
 @pytest.mark.parametrize("act,use_res", [(None, False), ("gelu", False), ("relu", True), (None, True)])
 def test_linear_large_row_counts_take_the_tiled_kernel(dtype, rows, K, M, act, use_res):
     """rows >= 4096 with aligned shapes run the LDS kernels (K a multiple of 32: the ring-buffered kernel, 256- or
@@ -159,6 +159,22 @@ def test_linear_large_row_counts_take_the_tiled_kernel(dtype, rows, K, M, act, u
     for lo, hi in ((0, 300), (rows - 257, rows)):
         small = ops.linear(x[lo:hi], w, b, act=act, residual=None if res is None else res[lo:hi])
         assert torch.equal(small, y[lo:hi])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,K,M", [(50, 49, 192), (4096, 29, 192), (32768, 34, 192), (9001, 40, 192), (100000, 40, 192)])
+def test_linear_zero_padded_k_gives_the_unpadded_bits(dtype, rows, K, M):
+    """Input rows and weight columns zero-padded to K = 64 (the padded encoder inputs): the vector kernels then
+    produce the BITS of the odd-K call - the pad lanes add exact zeros to the fp32 accumulators."""
+    x = _rand(rows, K, dtype=dtype, seed=rows + K)
+    w = _rand(M, K, dtype=dtype, seed=K + M, scale=1 / math.sqrt(K))
+    b = _rand(M, seed=M)
+    xp = torch.zeros(rows, 64, device=x.device, dtype=dtype)
+    xp[:, :K] = x
+    wp = torch.zeros(M, 64, device=x.device, dtype=dtype)
+    wp[:, :K] = w
+    for act in (None, "relu"):
+        assert torch.equal(ops.linear(xp, wp, b, act=act), ops.linear(x, w, b, act=act))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
