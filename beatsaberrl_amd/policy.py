@@ -20,7 +20,9 @@ Grad mode selects the path, as in the reference: under torch.no_grad() (rollout,
 forward-only routes above run; with grad mode on (the update), `forward_stacked` /
 `get_action_and_value(obs, action)` run op for op the per-op route as autograd Functions over the
 backward kernels (autograd_ops.py: LayerNorm, Linear data / weight / bias gradients, attention),
-so parameters receive fp32 gradients and the update forward is bitwise the per-op rollout forward.
+so parameters receive fp32 gradients and the update forward is bitwise the per-op rollout forward
+(`fused_ffn` off; with it on, the block FFNs of the update run forward as the fused kernel and
+recompute their hidden in the backward - less activation memory, one more GEMM per block).
 
 Stream dtype: `policy.fp16 = True` runs the 16-bit stream (fp16; set `stream_dtype =
 torch.bfloat16` for bf16) exactly as the reference's switch does (python/policy.py:
@@ -40,7 +42,7 @@ import torch.nn.functional as F
 from . import fp16_linear as _fl
 from . import obs_layout as L
 from . import ops
-from .autograd_ops import AttnPackedFn, AttnQKVFn, ChainFn, LinearFn, LnResFn
+from .autograd_ops import AttnPackedFn, AttnQKVFn, ChainFn, FusedFfnFn, LinearFn, LnResFn
 from .fused_ln import FusedLayerNorm
 
 OBS_DIM = L.OBS_DIM
@@ -234,9 +236,11 @@ class Block(nn.Module):
         return r + (v,) if want_v else r
 
 
-def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False):
+def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False, fused_ffn=False):
     """Block.forward under autograd (update path): the same kernels in the same order as the per-op
-    rollout route without the fused FFN, each paired with its backward; returns x_out (, v)."""
+    rollout route without the fused FFN, each paired with its backward; returns x_out (, v).
+    fused_ffn: the FFN's forward as the fused kernel (reference python/fp16_linear.py:1197-1275; its
+    bits are the fused rollout route's, not the unfused chain's)."""
     d = self.d
     # each LayerNorm hands the stream back with it: the residual branch's gradient joins LN's inside ln_bwd
     x, h = LnResFn.apply(x.contiguous(), self.ln_attn.weight, self.ln_attn.bias, self.ln_attn.eps)
@@ -256,7 +260,10 @@ def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False):
         att = AttnPackedFn.apply(qkv, attn_bias, self.n_heads)
     x = _lin_t(self.out_proj, att, residual=x)
     x, h2 = LnResFn.apply(x, self.ln_ffn.weight, self.ln_ffn.bias, self.ln_ffn.eps)
-    x = _seq_t(self.ffn, h2, residual=x)
+    if fused_ffn:
+        x = FusedFfnFn.apply(x, h2, self.ffn[0].weight, self.ffn[0].bias, self.ffn[2].weight, self.ffn[2].bias)
+    else:
+        x = _seq_t(self.ffn, h2, residual=x)
     return (x, v) if want_v else x
 
 
@@ -542,8 +549,11 @@ class NotePolicy(nn.Module):
         return out.view(B, N_ACTION_HEADS, self.k_max), value
 
     def _forward_train(self, obs):
-        """The update-path forward: op for op the per-op rollout route (no fused FFN, no fused block
-        stack), so its outputs are that route's bits, with autograd Functions instead of bare kernels."""
+        """The update-path forward: op for op the per-op rollout route (no fused block stack), so its
+        outputs are that route's bits, with autograd Functions instead of bare kernels.  With
+        `fused_ffn` on (16-bit stream, a width the fused kernel takes) the block FFNs run forward as the
+        fused kernel, as in the reference (python/fp16_linear.py:1254-1275); the outputs then follow the
+        fused per-op rollout route to 16-bit rounding (that route also folds the next LayerNorm in)."""
         dt = self.stream_dtype if self.fp16 else torch.float32
         B, d = obs.shape[0], self.embed
         obs = obs.detach()
@@ -559,13 +569,16 @@ class NotePolicy(nn.Module):
         if self.emb_ln is not None:
             x = self.emb_ln(x)
         v0 = None
+        ffn = self.blocks[0].ffn
+        fuse = (self.fp16 and self.fused_ffn != "off" and isinstance(ffn[1], nn.ReLU)
+                and ops.ffn_fused_profitable(ffn[0].in_features, ffn[0].out_features, dt))
         for i, blk in enumerate(self.blocks[:-1]):
             if self.value_residual and i == 0:
-                x, v0 = blk.forward_train(x, attn_bias, want_v=True)
+                x, v0 = blk.forward_train(x, attn_bias, want_v=True, fused_ffn=fuse)
             else:
-                x = blk.forward_train(x, attn_bias, v0=v0)
+                x = blk.forward_train(x, attn_bias, v0=v0, fused_ffn=fuse)
         x_res = x
-        lead = self.blocks[-1].forward_train(x, attn_bias, n_queries=self.n_lead, v0=v0)
+        lead = self.blocks[-1].forward_train(x, attn_bias, n_queries=self.n_lead, v0=v0, fused_ffn=fuse)
         if self.final_ln is not None:
             lead = self.final_ln(lead)
         z = lead.reshape(B, self.n_lead * d)

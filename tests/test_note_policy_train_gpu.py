@@ -253,3 +253,61 @@ def test_functions_match_torch_autograd_on_the_same_forward(dtype):
     (xr2 * g1 + yr * g2).sum().backward()
     for got, want in ((am.grad, ar.grad), (bm.grad, br.grad), (ln.weight.grad, wl.grad), (ln.bias.grad, bl.grad), (bb.grad, bb2.grad)):
         assert _rel(got.float(), want) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,d,F", [(70, 128, 512), (4133, 192, 768)])
+def test_fused_ffn_function_matches_the_unfused_chain(dtype, rows, d, F):
+    """FusedFfnFn (fused forward kernel, chain backward over the recomputed hidden; reference
+    python/fp16_linear.py:1197-1251) against ChainFn on the same operands: outputs to 16-bit rounding of the
+    stream, every gradient to 2 % of its largest entry (the two forwards accumulate in different k orders, so a
+    hidden unit within a rounding of 0 may sit on the other side of the ReLU)."""
+    from beatsaberrl_amd.autograd_ops import ChainFn, FusedFfnFn
+    g = torch.Generator().manual_seed(rows)
+    mk = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).to(DEV)
+    w0, b0, w2, b2 = mk(F, d, sc=d ** -0.5), mk(F, sc=0.1), mk(d, F, sc=F ** -0.5), mk(d, sc=0.1)
+    x0, h0, go = mk(rows, d).to(dtype), mk(rows, d).to(dtype), mk(rows, d).to(dtype)
+    outs = []
+    for fn in ("fused", "chain"):
+        leaves = [t.clone().requires_grad_(True) for t in (x0, h0, w0, b0, w2, b2)]
+        x, h, a0, c0, a2, c2 = leaves
+        y = FusedFfnFn.apply(x, h, a0, c0, a2, c2) if fn == "fused" else ChainFn.apply(h, x, False, a0, c0, a2, c2)
+        y.backward(go)
+        outs.append((y.detach(), [t.grad for t in leaves]))
+    (yf, gf), (yc, gc) = outs
+    eps = 2.0 ** -10 if dtype is torch.float16 else 2.0 ** -7
+    assert (yf.float() - yc.float()).abs().max().item() <= 2 * eps * yc.float().abs().max().item()
+    for name, a, b in zip(("dx", "dh2", "dw0", "db0", "dw2", "db2"), gf, gc):
+        assert a.dtype == b.dtype and a.shape == b.shape, name
+        err = (a.float() - b.float()).abs().max().item()
+        assert err <= 2e-2 * b.float().abs().max().item(), (name, err)
+    assert torch.equal(gf[0], go)                               # the residual branch passes the gradient through
+
+
+def test_update_path_with_the_fused_ffn_follows_the_unfused_update():
+    """fused_ffn = "on": the update forward's block FFNs run as the fused kernel; logits, value and every
+    parameter gradient stay within the 16-bit class of the unfused update on the same weights and batch."""
+    kw = dict(embed=192, trunk_dim=384, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True)
+    m = _policy(5, **kw).to(DEV)
+    m.fp16 = True
+    B = 64
+    obs = _obs(B, 3).to(DEV)
+    g = torch.Generator().manual_seed(2)
+    action = (torch.rand(B, 29, generator=g) * 5).long().to(DEV)
+    adv, ret = torch.randn(B, generator=g).to(DEV), torch.randn(B, generator=g).to(DEV)
+    res = []
+    for mode in ("off", "on"):
+        m.fused_ffn = mode
+        m.zero_grad(set_to_none=True)
+        logits, value = m.forward_stacked(obs)
+        (_loss(logits, value, action, adv, ret) * 1024.0).backward()
+        res.append((logits.detach(), value.detach(), {n: p.grad.detach().clone() / 1024.0 for n, p in m.named_parameters()}))
+    (l0, v0, g0), (l1, v1, g1) = res
+    assert not torch.equal(l0, l1)                              # the fused kernel did run
+    assert (l0 - l1).abs().max().item() < 2e-2 and (v0 - v1).abs().max().item() < 2e-2
+    gmax = max(t.abs().max().item() for t in g0.values())
+    for n in g0:
+        den = g0[n].norm().item()
+        if g0[n].abs().max().item() < 1e-5 * gmax:
+            continue
+        assert (g1[n] - g0[n]).norm().item() <= 0.15 * den, (n, (g1[n] - g0[n]).norm().item() / den)
