@@ -346,11 +346,12 @@ def ffn_fused_supported(d, F, dtype) -> bool:
 
 
 def ffn_fused_profitable(d, F, dtype) -> bool:
-    """Is the fused FFN kernel the faster route?  Measured on MI355X (fp16, GELU, 0.26M-3.1M rows):
-    d = 128: 0.17 ms fused vs 0.28 ms for the two linears; d = 192: 0.76 vs 0.98; d = 256: 4.0 vs 2.7;
-    d = 384: 44 vs 16.5 - at d >= 256 the per-workgroup row tile that fits in registers is too small
-    for the weight stream, so the unfused pair (LDS-tiled linears, hidden through HBM) wins."""
-    return d <= 192 and ffn_fused_supported(d, F, dtype)
+    """Is the fused FFN kernel the faster route?  Measured on MI355X (fp16, 475k rows, FFN + next LayerNorm):
+    d = 128 (F = 512): 0.31 ms fused vs 0.31 + 0.06 ms for the two linears + LayerNorm; d = 192 (F = 768): 0.81 vs
+    0.54 + 0.09 (streaming / ring-buffered linears); d = 256: 4.0 vs 2.7 at 3.1M rows; d = 384: 44 vs 16.5 - past
+    d = 128 the per-workgroup row tile that fits in registers is too small for the weight stream, so the unfused
+    pair (hidden through HBM) wins."""
+    return d <= 128 and ffn_fused_supported(d, F, dtype)
 
 
 def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5):

@@ -551,8 +551,9 @@ class NotePolicy(nn.Module):
     def _forward_train(self, obs):
         """The update-path forward: op for op the per-op rollout route (no fused block stack), so its
         outputs are that route's bits, with autograd Functions instead of bare kernels.  With
-        `fused_ffn` on (16-bit stream, a width the fused kernel takes) the block FFNs run forward as the
-        fused kernel, as in the reference (python/fp16_linear.py:1254-1275); the outputs then follow the
+        `fused_ffn` on (16-bit stream, a width the fused kernel takes - here the switch buys activation
+        memory, so it applies wherever the kernel exists, not only where it is the faster forward) the
+        block FFNs run forward as the fused kernel, as in the reference (python/fp16_linear.py:1254-1275); the outputs then follow the
         fused per-op rollout route to 16-bit rounding (that route also folds the next LayerNorm in)."""
         dt = self.stream_dtype if self.fp16 else torch.float32
         B, d = obs.shape[0], self.embed
@@ -571,7 +572,7 @@ class NotePolicy(nn.Module):
         v0 = None
         ffn = self.blocks[0].ffn
         fuse = (self.fp16 and self.fused_ffn != "off" and isinstance(ffn[1], nn.ReLU)
-                and ops.ffn_fused_profitable(ffn[0].in_features, ffn[0].out_features, dt))
+                and ops.ffn_fused_supported(ffn[0].in_features, ffn[0].out_features, dt))
         for i, blk in enumerate(self.blocks[:-1]):
             if self.value_residual and i == 0:
                 x, v0 = blk.forward_train(x, attn_bias, want_v=True, fused_ffn=fuse)
