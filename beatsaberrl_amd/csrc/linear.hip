@@ -52,29 +52,35 @@ __device__ __forceinline__ void mfma_mainloop(const LinArgs& a, int64_t row0, in
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     const int nk = (a.K + 31) / 32;
-    s16x8 xf[4], wf[4];
+    // PF chunks of fragments in flight: a wave of this kernel has nothing else to hide the memory latency behind
+    // (with one chunk ahead every 16 MFMAs waited a full round trip: 2.4 us per chunk at 16k rows x K = 384).  The
+    // register sets rotate by full unrolling, never by a run-time index.
+    constexpr int PF = FAST ? 4 : 1;
+    s16x8 xf[PF][4], wf[PF][4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        xf[t] = load_frag<FAST>(x, a.ldx, xr[t], g * 8, a.K);
-        wf[t] = load_frag<FAST>(w, a.K, wr[t], g * 8, a.K);
-    }
-    for (int kc = 0; kc < nk; ++kc) {
-        s16x8 xn[4], wn[4];
-        const int k1 = (kc + 1) * 32 + g * 8;
-        if (kc + 1 < nk) {   // next fragments in flight while this chunk's 16 MFMAs issue
+    for (int s = 0; s < PF; ++s)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                xn[t] = load_frag<FAST>(x, a.ldx, xr[t], k1, a.K);
-                wn[t] = load_frag<FAST>(w, a.K, wr[t], k1, a.K);
-            }
+        for (int t = 0; t < 4; ++t) {
+            xf[s][t] = load_frag<FAST>(x, a.ldx, xr[t], s * 32 + g * 8, a.K);       // past K: zeros, no load
+            wf[s][t] = load_frag<FAST>(w, a.K, wr[t], s * 32 + g * 8, a.K);
         }
+    for (int kc0 = 0; kc0 < nk; kc0 += PF) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int s = 0; s < PF; ++s) {
+            if (kc0 + s < nk) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[i][j] = DT::mfma32(wf[i], xf[j], acc[i][j]);
-        if (kc + 1 < nk) {
+                for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) { xf[t] = xn[t]; wf[t] = wn[t]; }
+                    for (int j = 0; j < 4; ++j) acc[i][j] = DT::mfma32(wf[s][i], xf[s][j], acc[i][j]);
+                const int k1 = (kc0 + s + PF) * 32 + g * 8;
+                if (kc0 + s + PF < nk) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        xf[s][t] = load_frag<FAST>(x, a.ldx, xr[t], k1, a.K);
+                        wf[s][t] = load_frag<FAST>(w, a.K, wr[t], k1, a.K);
+                    }
+                }
+            }
         }
     }
 }

@@ -52,12 +52,22 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
     const int m0 = cb * MT * 16;
     const u16* w = static_cast<const u16*>(a.w);
     // resident weight block: fragment (mt, kc), lane l <- W[m0 + 16 mt + l % 16][32 kc + 8 (l / 16) .. + 7]
-    for (int i = tid; i < MT * KC * 64; i += ST_THREADS) {
+    // every load of the block is issued before the first LDS write: one memory round trip for the prologue, not one
+    // per pass (with few rows per workgroup the prologue is most of the kernel)
+    constexpr int WPASS = (MT * KC * 64 + ST_THREADS - 1) / ST_THREADS;
+    u32x4 wv[WPASS];
+#pragma unroll
+    for (int it = 0; it < WPASS; ++it) {
+        const int i = it * ST_THREADS + tid;
         const int l = i & 63, f = i >> 6, mt = f / KC, kc = f % KC;
         const int m = m0 + mt * 16 + (l & 15);
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (m < a.M) v = *reinterpret_cast<const uint4*>(w + (int64_t)m * KE + kc * 32 + 8 * (l >> 4));
-        wl[i] = v;
+        wv[it] = (u32x4){0u, 0u, 0u, 0u};
+        if (i < MT * KC * 64 && m < a.M) wv[it] = *reinterpret_cast<const u32x4*>(w + (int64_t)m * KE + kc * 32 + 8 * (l >> 4));
+    }
+#pragma unroll
+    for (int it = 0; it < WPASS; ++it) {
+        const int i = it * ST_THREADS + tid;
+        if (i < MT * KC * 64) wl[i] = __builtin_bit_cast(uint4, wv[it]);
     }
     float* bl = reinterpret_cast<float*>(wl + MT * KC * 64);
     u16* wt = reinterpret_cast<u16*>(bl + MT * 16) + wave * (16 * TP);   // this wave's 16-row tile: x on the way in, y on the way out
