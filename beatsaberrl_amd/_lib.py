@@ -8,7 +8,8 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
+CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -19,7 +20,7 @@ _p, _i64, _i32, _f = C.c_void_p, C.c_int64, C.c_int, C.c_float
 
 class CfgDesc(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d", "n_heads", "ffn", "T", "n_gears", "act", "final_ln",
-                                         "prop_dim", "obj_dim", "dtype", "reserved")]
+                                         "prop_dim", "obj_dim", "dtype", "flags")]
 
 
 class _Blk(C.Structure):

@@ -78,6 +78,8 @@ class ConfigPolicy(nn.Module):
         # final-block query pruning on the fused route (the reference's n_queries path,
         # python/policy.py:533-539): exact; False = one persistent kernel computing every token
         self.prune_final = True
+        # fused route, pruned form, key counts given: envs of at most 8 tokens share 16-row tiles two by two (same bits)
+        self.pack_short = True
         self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
                      "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}
 
@@ -121,7 +123,8 @@ class ConfigPolicy(nn.Module):
     def _desc(self, dt):
         return _lib.CfgDesc(self.n_layers, self.d, self.n_heads, self.ffn_dim, self.T, self.n_gears,
                             _lib.ACT_GELU if self.act == "gelu" else _lib.ACT_RELU,
-                            int(self.final_ln is not None), self.prop_dim, self.obj_dim, ops.dt_code(dt), 0)
+                            int(self.final_ln is not None), self.prop_dim, self.obj_dim, ops.dt_code(dt),
+                            0 if self.pack_short else _lib.CFG_NO_PACK)
 
     def fused_supported(self, dt=None) -> bool:
         dt = dt or _DTYPES[self.dtype]

@@ -58,6 +58,8 @@ struct FwdArgs {
     const int32_t* n_valid;
     float* logits; float* value;
     uint32_t* ws;
+    const int2* pairs;            // PACK: tile -> (env of rows 0.., env of rows 8.. or -1), written by cfg_pair_kernel
+    const int32_t* n_packed;      // PACK: number of tiles in `pairs`
     int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
 };
 
@@ -125,8 +127,13 @@ enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
 constexpr int TAIL_ENVS = 16;
 constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
 
-template <typename DT, int RT, int ACT, int MODE>
+// PACK (HEAD launch only): two envs of at most 8 tokens each share a 16-row tile, the second at rows 8..15, with a
+// block-diagonal key mask.  Every per-row computation (GEMMs, LayerNorm) is untouched by the row's position; the
+// softmax sums and the P.V contraction see an env's keys in lanes / k slots 8 further on, which moves whole
+// butterfly partners and whole k groups and adds exact zeros elsewhere: an env's bits stay what they are alone in a tile.
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
+    static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
     __shared__ uint4 lds[2][STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
@@ -135,7 +142,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
     constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? TAIL_ENVS : 1;     // envs per 16-row MFMA tile
     constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
-    const int64_t ntiles = (a.B + ENVS_PER_WG - 1) / ENVS_PER_WG;
+    const int64_t n_units = PACK ? (int64_t)*a.n_packed : a.B;           // 16-row tiles (PACK) or envs to cover
+    const int64_t ntiles = (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
     const uint4* img = a.frags;
     uint4 pr0a, pr0b, pr1a, pr1b;
@@ -526,12 +534,39 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
         if (MODE != MODE_TAIL) {
             // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
             Frag8 e[RT][KC];
+            // PACK: the env of this lane's row r16 and the row's token index inside it (otherwise a tile is one env and
+            // both follow from the tile index: nothing is kept in registers)
+            int64_t lenv[PACK ? RT : 1];
+            int ltok[PACK ? RT : 1];
+            auto env_at = [&](int rt) __attribute__((always_inline)) -> int64_t {
+                if (PACK) return lenv[PACK ? rt : 0];
+                const int64_t env = env0 + rt;
+                return env < a.B ? env : a.B - 1;
+            };
+            auto tok_at = [&](int rt) __attribute__((always_inline)) { return PACK ? ltok[PACK ? rt : 0] : r16; };
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
-                const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
+                if (PACK) {
+                    int64_t tix = env0 + rt; tix = tix < n_units ? tix : n_units - 1;
+                    const int2 pr = a.pairs[tix];
+                    const int ea = __builtin_amdgcn_readfirstlane(pr.x), eb = __builtin_amdgcn_readfirstlane(pr.y);
+                    const bool second = eb >= 0 && r16 >= 8;
+                    const int64_t le = second ? eb : ea;
+                    lenv[PACK ? rt : 0] = le;
+                    ltok[PACK ? rt : 0] = second ? r16 - 8 : r16;
+                    const int nvalid = a.n_valid[le];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = 4 * g + i;
+                        const bool khalf = eb >= 0 && key >= 8;
+                        kmask[rt][i] = (khalf == second && (khalf ? key - 8 : key) <= nvalid) ? 0.f : -INFINITY;
+                    }
+                } else {
+                    const int64_t env = env_at(rt);
+                    const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
+                }
             }
             if (a.tok_vec) {
                 // a lane's 8 k slots per chunk are two runs of 4 consecutive obs lanes: k0 = 32 c + 4 g + 16 jh.
@@ -542,16 +577,16 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 asm volatile("" : "+v"(tr), "+v"(tg));
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
-                    const float* orow = static_cast<const float*>(a.obs) + env * a.obs_ld;
+                    const float* orow = static_cast<const float*>(a.obs) + env_at(rt) * a.obs_ld;
+                    const int tk = PACK ? tok_at(rt) : tr;                         // the row's token index
 #pragma unroll
                     for (int c = 0; c < KC; ++c)
 #pragma unroll
                         for (int jh = 0; jh < 2; ++jh) {
                             const int k0 = 32 * c + 4 * tg + 16 * jh;
                             bool valid; int idx;
-                            if (c == 0 && jh == 0) { valid = tr >= 1; idx = a.prop_dim + (tr - 1) * 16 + k0; }
-                            else { valid = tr == 0 && (k0 - 16) < a.prop_dim; idx = k0 - 16; }
+                            if (c == 0 && jh == 0) { valid = tk >= 1; idx = a.prop_dim + (tk - 1) * 16 + k0; }
+                            else { valid = tk == 0 && (k0 - 16) < a.prop_dim; idx = k0 - 16; }
                             const float4 v = *reinterpret_cast<const float4*>(orow + (valid ? idx : 0));
                             const uint32_t lo = pack2<DT>(v.x, v.y), hi = pack2<DT>(v.z, v.w);
                             e[rt][c].w[2 * jh] = valid ? lo : 0u;
@@ -561,7 +596,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             } else {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    int64_t env = env0 + rt; env = env < a.B ? env : a.B - 1;
+                    const int64_t env = env_at(rt);
+                    const int tk = tok_at(rt);
                     float ev[KC][8];
 #pragma unroll
                     for (int c = 0; c < KC; ++c)
@@ -569,8 +605,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         for (int j = 0; j < 8; ++j) {
                             const int k = 32 * c + 4 * g + (j & 3) + (j >> 2) * 16;    // permuted k order
                             int idx; bool on;
-                            if (k < 16) { on = r16 >= 1 && k < a.obj_dim; idx = a.prop_dim + (r16 - 1) * a.obj_dim + k; }
-                            else { on = r16 == 0 && (k - 16) < a.prop_dim; idx = k - 16; }
+                            if (k < 16) { on = tk >= 1 && k < a.obj_dim; idx = a.prop_dim + (tk - 1) * a.obj_dim + k; }
+                            else { on = tk == 0 && (k - 16) < a.prop_dim; idx = k - 16; }
                             float v = 0.f;
                             if (on) {
                                 const int64_t off = env * a.obs_ld + idx;
@@ -588,9 +624,11 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 bp = *reinterpret_cast<const float4*>(vlds + V_BP + 16 * nt + 4 * g);
                 const float4 bo = *reinterpret_cast<const float4*>(vlds + V_BO + 16 * nt + 4 * g);
-                const float4 b = r16 == 0 ? bp : bo;
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) x[rt][nt] = (f32x4){b.x, b.y, b.z, b.w};
+                for (int rt = 0; rt < RT; ++rt) {
+                    const float4 b = tok_at(rt) == 0 ? bp : bo;
+                    x[rt][nt] = (f32x4){b.x, b.y, b.z, b.w};
+                }
             }
 #pragma unroll
             for (int st = 0; st < EMB_STAGES; ++st) {
@@ -613,11 +651,13 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             if (MODE == MODE_HEAD) {
                 // last block: attention only, then park token 0 (lanes r16 == 0) for the TAIL launch
                 attention(vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F));
-                if (r16 == 0) {
+                if (PACK ? (r16 & 7) == 0 : r16 == 0) {
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
-                        const int64_t env = env0 + rt;
-                        if (env < a.B) {
+                        // PACK: rows 0 and 8 of a pair tile are token 0 of its two envs; units past the end are
+                        // recomputed copies of the last tile and store nothing
+                        const int64_t env = PACK ? lenv[PACK ? rt : 0] : env0 + rt;
+                        if (PACK ? (ltok[PACK ? rt : 0] == 0 && env0 + rt < n_units) : env < a.B) {
                             uint4* dst = reinterpret_cast<uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
 #pragma unroll
                             for (int nt = 0; nt < NT; ++nt) dst[nt] = __builtin_bit_cast(uint4, x[rt][nt]);
@@ -763,10 +803,101 @@ bool shape_ok(const bsrl_cfg_desc* d) {
 }
 int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
 
-template <typename DT, int RT, int ACT, int MODE>
+// Tile table of the packed HEAD launch.  Envs of at most 8 tokens (n_valid <= 7) are "short"; the short list and the
+// long list keep env order (a stable split, so the table is a function of the batch alone).  Tiles: the pairs
+// (short[2 i], short[2 i + 1]), then a lone last short env if their count is odd, then one tile per long env.
+// pairs[t] = (env of rows 0.., env of rows 8.. or -1); *n_packed = the number of tiles.
+// Workgroup b owns the envs [b span, (b + 1) span), `per` consecutive ones per thread.  Every workgroup counts the short
+// envs of the WHOLE batch for itself (coalesced reads of <= 4 B per env out of L2: cheaper than a second launch or a
+// cross-workgroup hand-off), which gives it both the count before its span and the total.
+constexpr int PAIR_THREADS = 256;
+constexpr int PAIR_MAX_WGS = 256;
+constexpr int PAIR_OWN = 4;                                // own envs a thread keeps in registers
+constexpr int PAIR_CNT = 64;                               // key counts per thread and counting pass
+__device__ __forceinline__ bool env_is_short(int nv) { return nv >= 0 && nv <= 7; }
+__global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n_valid, int64_t B, int64_t span, int per,
+                                                                int2* pairs, int32_t* n_packed) {
+    __shared__ int red[3][PAIR_THREADS / WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t w0 = (int64_t)blockIdx.x * span;
+    // Every global load of the common case leaves in one batch (own envs first, then PAIR_CNT counts per thread per
+    // pass): a dependent round trip costs ~1.5 us on an otherwise idle chip, and this kernel is nothing but round trips.
+    const int64_t lo = w0 + (int64_t)tid * per < B ? w0 + (int64_t)tid * per : B;
+    const int64_t hi = lo + per < B ? lo + per : B;
+    int own[PAIR_OWN];
+#pragma unroll
+    for (int j = 0; j < PAIR_OWN; ++j) {       // clamped index, not a guarded load: a load under a branch is waited for at once
+        const int v = n_valid[lo + j < B ? lo + j : B - 1];
+        own[j] = lo + j < hi ? v : -1;
+    }
+    int before = 0, total = 0;
+    for (int64_t i0 = 0; i0 < B; i0 += PAIR_CNT * PAIR_THREADS) {
+        int nv[PAIR_CNT];
+#pragma unroll
+        for (int j = 0; j < PAIR_CNT; ++j) {
+            const int64_t i = i0 + j * PAIR_THREADS + tid;
+            const int v = n_valid[i < B ? i : B - 1];
+            nv[j] = i < B ? v : -1;
+        }
+#pragma unroll
+        for (int j = 0; j < PAIR_CNT; ++j) {
+            const int s = env_is_short(nv[j]) ? 1 : 0;
+            total += s;
+            before += (i0 + j * PAIR_THREADS + tid < w0) ? s : 0;
+        }
+    }
+    // the inclusive scan of this thread's short count over the workgroup
+    int cs = 0;
+    if (per <= PAIR_OWN) {
+#pragma unroll
+        for (int j = 0; j < PAIR_OWN; ++j) cs += env_is_short(own[j]) ? 1 : 0;
+    } else {
+        for (int64_t e = lo; e < hi; ++e) cs += env_is_short(n_valid[e]) ? 1 : 0;
+    }
+    int inc = cs;
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int v = __shfl_up(inc, d, WAVE);
+        if (lane >= d) inc += v;
+    }
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) { before += __shfl_xor(before, d, WAVE); total += __shfl_xor(total, d, WAVE); }
+    if (lane == WAVE - 1) red[0][wave] = inc;
+    if (lane == 0) { red[1][wave] = before; red[2][wave] = total; }
+    __syncthreads();
+    int base = 0; before = 0; total = 0;
+#pragma unroll
+    for (int w = 0; w < PAIR_THREADS / WAVE; ++w) {
+        if (w < wave) base += red[0][w];
+        before += red[1][w]; total += red[2][w];
+    }
+    int64_t rs = (int64_t)before + base + inc - cs;        // short envs before this thread's first env
+    int64_t rl = lo - rs;                                  // long envs before it
+    const int64_t first_long = ((int64_t)total + 1) / 2;
+    auto place = [&](int64_t e, int nv) __attribute__((always_inline)) {
+        if (env_is_short(nv)) {
+            int32_t* p = reinterpret_cast<int32_t*>(pairs + rs / 2);
+            p[rs & 1] = (int32_t)e;
+            if (rs == total - 1 && !(rs & 1)) p[1] = -1;   // odd count: the last short env sits alone
+            ++rs;
+        } else {
+            pairs[first_long + rl] = make_int2((int)e, -1);
+            ++rl;
+        }
+    };
+    if (per <= PAIR_OWN) {
+#pragma unroll
+        for (int j = 0; j < PAIR_OWN; ++j) if (lo + j < hi) place(lo + j, own[j]);
+    } else {
+        for (int64_t e = lo; e < hi; ++e) place(e, n_valid[e]);
+    }
+    if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - total));
+}
+
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
 int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
     const size_t dyn = (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
-    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE>;
+    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK>;
     if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
@@ -779,7 +910,7 @@ int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
 }
 
 template <typename DT, int ACT>
-int launch_all(FwdArgs a, bool pruned, int cus, hipStream_t st) {
+int launch_all(FwdArgs a, bool pruned, bool pack, int cus, hipStream_t st) {
     const int ls = layer_stages(a.F), total = total_stages(a.n_layers, a.F);
     if (!pruned) {
         a.s_begin = 0; a.s_end = total;
@@ -787,7 +918,21 @@ int launch_all(FwdArgs a, bool pruned, int cus, hipStream_t st) {
     }
     const int split = EMB_STAGES + (a.n_layers - 1) * ls + 3 * H;
     a.s_begin = 0; a.s_end = split;
-    int rc = launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
+    int rc;
+    if (pack) {
+        // the grid is sized for the unpacked tile count (the packed one is known on the device only); workgroups past
+        // the packed count leave after their prologue
+        int64_t wgs = (a.B + PAIR_THREADS - 1) / PAIR_THREADS;
+        if (wgs > PAIR_MAX_WGS) wgs = PAIR_MAX_WGS;
+        const int per = (int)(((a.B + wgs - 1) / wgs + PAIR_THREADS - 1) / PAIR_THREADS);      // envs per thread
+        const int64_t span = (int64_t)per * PAIR_THREADS;                                      // envs per workgroup
+        wgs = (a.B + span - 1) / span;
+        hipLaunchKernelGGL(cfg_pair_kernel, dim3((unsigned)wgs), dim3(PAIR_THREADS), 0, st, a.n_valid, a.B, span, per,
+                           const_cast<int2*>(a.pairs), const_cast<int32_t*>(a.n_packed));
+        rc = launch_one<DT, 2, ACT, MODE_HEAD, true>(a, cus, st);
+    } else {
+        rc = launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
+    }
     if (rc != BSRL_OK) return rc;
     a.s_begin = split; a.s_end = total;
     return launch_one<DT, 1, ACT, MODE_TAIL>(a, cus, st);
@@ -826,9 +971,15 @@ extern "C" int bsrl_cfg_pack(const bsrl_cfg_desc* d, const bsrl_cfg_params* p, v
     return BSRL_OK;
 }
 
+namespace {
+// workspace layout: token-0 rows (B x 768 B), then the packed launch's tile table (B int2) and its tile count
+int64_t ws_rows_bytes(int64_t B) { return B * 4 * WS_DWORDS * (int64_t)sizeof(uint32_t); }
+int64_t ws_pairs_bytes(int64_t B) { return (B * (int64_t)sizeof(int2) + 15) / 16 * 16 + 16; }
+}  // namespace
+
 extern "C" int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* d, int64_t B) {
     if (!shape_ok(d) || B <= 0) return 0;
-    return B * 4 * WS_DWORDS * (int64_t)sizeof(uint32_t);
+    return ws_rows_bytes(B) + ws_pairs_bytes(B);
 }
 
 extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
@@ -851,7 +1002,17 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
     a.ws = static_cast<uint32_t*>(workspace);
     // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
-    const bool pruned = workspace && workspace_bytes >= bsrl_cfg_workspace_size(d, B) && d->ffn % 64 == 0;
+    const bool pruned = workspace && workspace_bytes >= ws_rows_bytes(B) && d->ffn % 64 == 0;
+    // short envs share tiles when the caller gives key counts, the workspace holds the tile table and the descriptor
+    // does not switch it off; B < 2^31 - 1 keeps env ids in the table's int32
+    const bool pack = pruned && n_valid && !(d->flags & BSRL_CFG_NO_PACK) && B < (int64_t)0x7fffffff &&
+                      workspace_bytes >= ws_rows_bytes(B) + ws_pairs_bytes(B);
+    a.pairs = nullptr; a.n_packed = nullptr;
+    if (pack) {
+        char* tail = static_cast<char*>(workspace) + ws_rows_bytes(B);
+        a.pairs = reinterpret_cast<const int2*>(tail);
+        a.n_packed = reinterpret_cast<const int32_t*>(tail + ws_pairs_bytes(B) - 16);
+    }
     if (workspace && !bsrl_aligned(workspace, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: workspace must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
@@ -859,9 +1020,9 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
     int rc;
     if (d->dtype == BSRL_F16)
-        rc = d->act == BSRL_ACT_GELU ? launch_all<F16, BSRL_ACT_GELU>(a, pruned, cus, st) : launch_all<F16, BSRL_ACT_RELU>(a, pruned, cus, st);
+        rc = d->act == BSRL_ACT_GELU ? launch_all<F16, BSRL_ACT_GELU>(a, pruned, pack, cus, st) : launch_all<F16, BSRL_ACT_RELU>(a, pruned, pack, cus, st);
     else
-        rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, cus, st);
+        rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, pack, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, pack, cus, st);
     if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH("bsrl_cfg_forward");
     return BSRL_OK;

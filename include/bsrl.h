@@ -162,8 +162,10 @@ int bsrl_cfg_embed(const void* obs, int64_t obs_ld, int obs_dtype,
  * step, its address must not move while a captured graph replays. */
 typedef struct {
     int32_t n_layers, d, n_heads, ffn, T, n_gears, act, final_ln;
-    int32_t prop_dim, obj_dim, dtype, reserved;
+    int32_t prop_dim, obj_dim, dtype, flags;      /* flags: 0, or BSRL_CFG_NO_PACK */
 } bsrl_cfg_desc;
+/* bsrl_cfg_forward: keep every env in a tile of its own (see below). */
+#define BSRL_CFG_NO_PACK 1
 
 /* fp32 master parameter pointers of one transformer block, in the reference's
  * registration order (python/policy.py:492-522); device memory. */
@@ -187,7 +189,8 @@ int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* desc);
 int bsrl_cfg_pack(const bsrl_cfg_desc* desc, const bsrl_cfg_params* params,
                   void* packed, bsrl_stream stream);
 /* Bytes of scratch the pruned two-launch form of bsrl_cfg_forward needs for B envs
- * (768 B per env), or 0 if the shape is unsupported. */
+ * (768 B per env for the parked rows + 8 B per env + 32 B for the tile table of
+ * the packed launch), or 0 if the shape is unsupported. */
 int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
 /* obs (B, obs_ld) F32 or 16-bit; n_valid (B,) int32 or NULL (all valid).
  * workspace == NULL (or smaller than bsrl_cfg_workspace_size): ONE persistent
@@ -196,7 +199,14 @@ int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
  * :1302-1305; exact, masking is key-side only) - launch 1 runs the tokenizer,
  * blocks 0..L-2 and the last block's attention and parks each env's token-0
  * row in the workspace, launch 2 runs the last block's output projection +
- * FFN and the heads on those rows, 16 envs per MFMA tile. */
+ * FFN and the heads on those rows, 16 envs per MFMA tile.  With n_valid given
+ * and the full workspace, launch 1 also packs envs of at most 8 tokens
+ * (n_valid <= 7) two to a 16-row tile (rows 0.. and 8.., block-diagonal key
+ * mask; a one-workgroup kernel builds the tile table on the stream first):
+ * padded rows are what the reference computes and discards
+ * (python/policy.py:1257-1260 masks them key-side), and an env's output bits
+ * are the same packed or alone.  desc->flags = BSRL_CFG_NO_PACK keeps one env
+ * per tile; a workspace of only 768 B per env does too. */
 int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      const void* obs, int64_t obs_ld, int obs_dtype,
                      const int32_t* n_valid, float* logits, float* value,

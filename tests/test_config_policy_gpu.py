@@ -215,6 +215,58 @@ def test_fused_route_invariants(prune):
     assert (l6 - lg).abs().max().item() < 5e-3
 
 
+def test_fused_route_packed_tiles_at_a_batch_with_several_envs_per_pairing_thread():
+    """B > 65536: the tile-table kernel walks several envs per thread; same bits as one env per tile."""
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    _, m = _build(spec, c["w_seed"], "f16", "fused")
+    obs, k = cm.make_inputs(spec, 70001, 77, "uniform")
+    od, kd = obs.to(DEV), k.to(DEV)
+    lg1, v1 = m.forward_stacked(od, kd)
+    m.pack_short = False
+    lg0, v0 = m.forward_stacked(od, kd)
+    assert torch.equal(lg1, lg0) and torch.equal(v1, v0)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("case", ["uniform", "all_short", "all_long", "one_short", "odd_short", "alternating"])
+@pytest.mark.parametrize("B", [1, 9, 700, 4099])
+def test_fused_route_packed_tiles_give_the_unpacked_bits(dtype, case, B):
+    """`pack_short` (envs of at most 8 tokens two to a 16-row tile in the pruned form's first launch) against one env
+    per tile: logits and values are bitwise equal for every mix of short and long envs, and both match the oracle."""
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    p, m = _build(spec, c["w_seed"], dtype, "fused")
+    obs, k = cm.make_inputs(spec, B, 40 + B, "uniform")
+    if case == "all_short":
+        k = k % 8
+    elif case == "all_long":
+        k = 8 + k % 8
+    elif case == "one_short":
+        k = 8 + k % 8
+        k[B // 2] = 3
+    elif case == "odd_short":
+        k = 8 + k % 8
+        k[: min(B, 5)] = torch.tensor([0, 7, 2, 5, 1], dtype=torch.int32)[: min(B, 5)]
+    elif case == "alternating":
+        k = torch.where(torch.arange(B) % 2 == 0, k % 8, 8 + k % 8).to(torch.int32)
+    od, kd = obs.to(DEV), k.to(DEV)
+    m.pack_short = True
+    lg1, v1 = m.forward_stacked(od, kd)
+    m.pack_short = False
+    lg0, v0 = m.forward_stacked(od, kd)
+    assert torch.equal(lg1, lg0) and torch.equal(v1, v0)
+    if B == 700:                                  # the class bounds are max statistics: not for a handful of envs
+        _check16(lg1, v1, p, spec, obs, k, dtype, round_residual=False)
+    # junk in the masked slots of a packed env cannot leak into its tile partner
+    obs2 = obs.clone()
+    for e in range(B):
+        obs2[e, spec.prop_dim + int(k[e]) * spec.obj_dim:] = -77.0
+    m.pack_short = True
+    lg2, v2 = m.forward_stacked(obs2.to(DEV), kd)
+    assert torch.equal(lg2, lg1) and torch.equal(v2, v1)
+
+
 def test_fused_unsupported_shapes_fall_to_ops_route():
     for ci in (2, 3):
         spec = cm.CONFIGS[ci]["spec"]
