@@ -813,7 +813,7 @@ int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_l
 constexpr int PAIR_THREADS = 256;
 constexpr int PAIR_MAX_WGS = 256;
 constexpr int PAIR_OWN = 4;                                // own envs a thread keeps in registers
-constexpr int PAIR_CNT = 64;                               // key counts per thread and counting pass
+constexpr int PAIR_CNT = 16;                               // 16-byte loads (4 key counts each) per thread and counting pass
 __device__ __forceinline__ bool env_is_short(int nv) { return nv >= 0 && nv <= 7; }
 __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n_valid, int64_t B, int64_t span, int per,
                                                                 int2* pairs, int32_t* n_packed) {
@@ -830,21 +830,29 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
         const int v = n_valid[lo + j < B ? lo + j : B - 1];
         own[j] = lo + j < hi ? v : -1;
     }
+    // counts of the whole batch, four envs per load (n_valid is 16-byte aligned on this path, B < 2^31)
     int before = 0, total = 0;
-    for (int64_t i0 = 0; i0 < B; i0 += PAIR_CNT * PAIR_THREADS) {
-        int nv[PAIR_CNT];
+    const int nq = (int)(B >> 2), w0q = (int)(w0 >> 2);     // w0 is a multiple of PAIR_THREADS
+    const int4* nvq = reinterpret_cast<const int4*>(n_valid);
+    for (int q0 = 0; q0 < nq; q0 += PAIR_CNT * PAIR_THREADS) {
+        int4 v[PAIR_CNT];
+#pragma unroll
+        for (int j = 0; j < PAIR_CNT; ++j) { const int q = q0 + j * PAIR_THREADS + tid; v[j] = nvq[q < nq ? q : nq - 1]; }
 #pragma unroll
         for (int j = 0; j < PAIR_CNT; ++j) {
-            const int64_t i = i0 + j * PAIR_THREADS + tid;
-            const int v = n_valid[i < B ? i : B - 1];
-            nv[j] = i < B ? v : -1;
+            const int q = q0 + j * PAIR_THREADS + tid;
+            int sh = (env_is_short(v[j].x) ? 1 : 0) + (env_is_short(v[j].y) ? 1 : 0) + (env_is_short(v[j].z) ? 1 : 0) +
+                     (env_is_short(v[j].w) ? 1 : 0);
+            sh = q < nq ? sh : 0;
+            total += sh;
+            before += q < w0q ? sh : 0;
         }
-#pragma unroll
-        for (int j = 0; j < PAIR_CNT; ++j) {
-            const int s = env_is_short(nv[j]) ? 1 : 0;
-            total += s;
-            before += (i0 + j * PAIR_THREADS + tid < w0) ? s : 0;
-        }
+    }
+    if (tid < (int)(B & 3)) {                               // the last B % 4 envs
+        const int64_t e = (int64_t)nq * 4 + tid;
+        const int sh = env_is_short(n_valid[e]) ? 1 : 0;
+        total += sh;
+        before += e < w0 ? sh : 0;
     }
     // the inclusive scan of this thread's short count over the workgroup
     int cs = 0;
@@ -1004,8 +1012,9 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
     const bool pruned = workspace && workspace_bytes >= ws_rows_bytes(B) && d->ffn % 64 == 0;
     // short envs share tiles when the caller gives key counts, the workspace holds the tile table and the descriptor
-    // does not switch it off; B < 2^31 - 1 keeps env ids in the table's int32
-    const bool pack = pruned && n_valid && !(d->flags & BSRL_CFG_NO_PACK) && B < (int64_t)0x7fffffff &&
+    // does not switch it off (n_valid 16-byte aligned: the table kernel reads it four at a time); B < 2^31 - 1 keeps
+    // env ids in the table's int32
+    const bool pack = pruned && n_valid && bsrl_aligned(n_valid, 16) && !(d->flags & BSRL_CFG_NO_PACK) && B < (int64_t)0x7fffffff &&
                       workspace_bytes >= ws_rows_bytes(B) + ws_pairs_bytes(B);
     a.pairs = nullptr; a.n_packed = nullptr;
     if (pack) {

@@ -206,7 +206,8 @@ int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
  * padded rows are what the reference computes and discards
  * (python/policy.py:1257-1260 masks them key-side), and an env's output bits
  * are the same packed or alone.  desc->flags = BSRL_CFG_NO_PACK keeps one env
- * per tile; a workspace of only 768 B per env does too. */
+ * per tile; a workspace of only 768 B per env, or an n_valid that is not
+ * 16-byte aligned, does too. */
 int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      const void* obs, int64_t obs_ld, int obs_dtype,
                      const int32_t* n_valid, float* logits, float* value,
