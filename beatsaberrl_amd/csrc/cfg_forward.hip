@@ -58,7 +58,8 @@ struct FwdArgs {
     const int32_t* n_valid;
     float* logits; float* value;
     uint32_t* ws;
-    const int2* pairs;            // PACK: tile -> (env of rows 0.., env of rows 8.. or -1), written by cfg_pair_kernel
+    const int4* pairs;            // PACK: tile -> the env that starts at rows 0 / 4 / 8 / 12 (-1: the slot continues the env
+                                  // before it), written by cfg_pair_kernel
     const int32_t* n_packed;      // PACK: number of tiles in `pairs`
     int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
 };
@@ -127,10 +128,11 @@ enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
 constexpr int TAIL_ENVS = 16;
 constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
 
-// PACK (HEAD launch only): two envs of at most 8 tokens each share a 16-row tile, the second at rows 8..15, with a
-// block-diagonal key mask.  Every per-row computation (GEMMs, LayerNorm) is untouched by the row's position; the
-// softmax sums and the P.V contraction see an env's keys in lanes / k slots 8 further on, which moves whole
-// butterfly partners and whole k groups and adds exact zeros elsewhere: an env's bits stay what they are alone in a tile.
+// PACK (HEAD launch only): short envs share a 16-row tile under a block-diagonal key mask - two of at most 8 tokens
+// (rows 0.. and 8..) or four of at most 4 tokens (rows 0.., 4.., 8.., 12..).  Every per-row computation (GEMMs,
+// LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
+// multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
+// and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
 template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
@@ -548,19 +550,25 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             for (int rt = 0; rt < RT; ++rt) {
                 if (PACK) {
                     int64_t tix = env0 + rt; tix = tix < n_units ? tix : n_units - 1;
-                    const int2 pr = a.pairs[tix];
-                    const int ea = __builtin_amdgcn_readfirstlane(pr.x), eb = __builtin_amdgcn_readfirstlane(pr.y);
-                    const bool second = eb >= 0 && r16 >= 8;
-                    const int64_t le = second ? eb : ea;
+                    const int4 pr = a.pairs[tix];
+                    const int e0 = __builtin_amdgcn_readfirstlane(pr.x), e1 = __builtin_amdgcn_readfirstlane(pr.y);
+                    const int e2 = __builtin_amdgcn_readfirstlane(pr.z), e3 = __builtin_amdgcn_readfirstlane(pr.w);
+                    // the slot (rows 4 s .. 4 s + 3) an env starts in, for this lane's row and for its 4 keys (one slot)
+                    auto owner = [&](int sl) __attribute__((always_inline)) {
+                        int o = 0;
+                        o = (sl >= 1 && e1 >= 0) ? 1 : o;
+                        o = (sl >= 2 && e2 >= 0) ? 2 : o;
+                        o = (sl >= 3 && e3 >= 0) ? 3 : o;
+                        return o;
+                    };
+                    const int orow = owner(r16 >> 2), okey = owner(g);
+                    const int64_t le = orow == 0 ? e0 : orow == 1 ? e1 : orow == 2 ? e2 : e3;
                     lenv[PACK ? rt : 0] = le;
-                    ltok[PACK ? rt : 0] = second ? r16 - 8 : r16;
+                    ltok[PACK ? rt : 0] = r16 - 4 * orow;
                     const int nvalid = a.n_valid[le];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = 4 * g + i;
-                        const bool khalf = eb >= 0 && key >= 8;
-                        kmask[rt][i] = (khalf == second && (khalf ? key - 8 : key) <= nvalid) ? 0.f : -INFINITY;
-                    }
+                    for (int i = 0; i < 4; ++i)
+                        kmask[rt][i] = (okey == orow && 4 * g + i - 4 * okey <= nvalid) ? 0.f : -INFINITY;
                 } else {
                     const int64_t env = env_at(rt);
                     const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
@@ -651,10 +659,10 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             if (MODE == MODE_HEAD) {
                 // last block: attention only, then park token 0 (lanes r16 == 0) for the TAIL launch
                 attention(vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F));
-                if (PACK ? (r16 & 7) == 0 : r16 == 0) {
+                if (PACK ? (r16 & 3) == 0 : r16 == 0) {
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
-                        // PACK: rows 0 and 8 of a pair tile are token 0 of its two envs; units past the end are
+                        // PACK: the first row of every occupied slot is token 0 of an env; units past the end are
                         // recomputed copies of the last tile and store nothing
                         const int64_t env = PACK ? lenv[PACK ? rt : 0] : env0 + rt;
                         if (PACK ? (ltok[PACK ? rt : 0] == 0 && env0 + rt < n_units) : env < a.B) {
@@ -803,24 +811,28 @@ bool shape_ok(const bsrl_cfg_desc* d) {
 }
 int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
 
-// Tile table of the packed HEAD launch.  Envs of at most 8 tokens (n_valid <= 7) are "short"; the short list and the
-// long list keep env order (a stable split, so the table is a function of the batch alone).  Tiles: the pairs
-// (short[2 i], short[2 i + 1]), then a lone last short env if their count is odd, then one tile per long env.
-// pairs[t] = (env of rows 0.., env of rows 8.. or -1); *n_packed = the number of tiles.
-// Workgroup b owns the envs [b span, (b + 1) span), `per` consecutive ones per thread.  Every workgroup counts the short
-// envs of the WHOLE batch for itself (coalesced reads of <= 4 B per env out of L2: cheaper than a second launch or a
-// cross-workgroup hand-off), which gives it both the count before its span and the total.
+// Tile table of the packed HEAD launch.  Envs of at most 4 tokens (n_valid <= 3) are "tiny", of 5..8 tokens "mid",
+// the rest long; each class keeps env order (a stable split, so the table is a function of the batch alone).  Tiles:
+// the mid pairs (mid[2 i], mid[2 i + 1]) at rows 0 / 8 (a lone last one if their count is odd), then the tiny quads
+// (tiny[4 i .. 4 i + 3]) at rows 0 / 4 / 8 / 12 (the last tile may hold fewer), then one tile per long env.
+// pairs[t] = the env that starts in each 4-row slot, -1 where the slot continues the env before it (or is empty
+// after the last tiny env); *n_packed = the number of tiles.
+// Workgroup b owns the envs [b span, (b + 1) span), `per` consecutive ones per thread.  Every workgroup counts the
+// classes of the WHOLE batch for itself (coalesced 16-byte reads out of L2: cheaper than a second launch or a
+// cross-workgroup hand-off), which gives it both the counts before its span and the totals.
 constexpr int PAIR_THREADS = 256;
 constexpr int PAIR_MAX_WGS = 256;
 constexpr int PAIR_OWN = 4;                                // own envs a thread keeps in registers
 constexpr int PAIR_CNT = 16;                               // 16-byte loads (4 key counts each) per thread and counting pass
-__device__ __forceinline__ bool env_is_short(int nv) { return nv >= 0 && nv <= 7; }
+// class counts travel as one int: tiny in the low 16 bits is not enough for a batch, so two ints - [0] tiny, [1] mid
+__device__ __forceinline__ int env_tiny(int nv) { return nv >= 0 && nv <= 3 ? 1 : 0; }
+__device__ __forceinline__ int env_mid(int nv) { return nv >= 4 && nv <= 7 ? 1 : 0; }
 __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n_valid, int64_t B, int64_t span, int per,
-                                                                int2* pairs, int32_t* n_packed) {
-    __shared__ int red[3][PAIR_THREADS / WAVE];
+                                                                int4* pairs, int32_t* n_packed) {
+    __shared__ int red[6][PAIR_THREADS / WAVE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t w0 = (int64_t)blockIdx.x * span;
-    // Every global load of the common case leaves in one batch (own envs first, then PAIR_CNT counts per thread per
+    // Every global load of the common case leaves in one batch (own envs first, then PAIR_CNT loads per thread per
     // pass): a dependent round trip costs ~1.5 us on an otherwise idle chip, and this kernel is nothing but round trips.
     const int64_t lo = w0 + (int64_t)tid * per < B ? w0 + (int64_t)tid * per : B;
     const int64_t hi = lo + per < B ? lo + per : B;
@@ -830,8 +842,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
         const int v = n_valid[lo + j < B ? lo + j : B - 1];
         own[j] = lo + j < hi ? v : -1;
     }
-    // counts of the whole batch, four envs per load (n_valid is 16-byte aligned on this path, B < 2^31)
-    int before = 0, total = 0;
+    // class counts of the whole batch, four envs per load (n_valid is 16-byte aligned on this path, B < 2^31)
+    int bt = 0, bm = 0, tt = 0, tm = 0;                     // tiny / mid before this workgroup's span, and in total
     const int nq = (int)(B >> 2), w0q = (int)(w0 >> 2);     // w0 is a multiple of PAIR_THREADS
     const int4* nvq = reinterpret_cast<const int4*>(n_valid);
     for (int q0 = 0; q0 < nq; q0 += PAIR_CNT * PAIR_THREADS) {
@@ -841,65 +853,84 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
 #pragma unroll
         for (int j = 0; j < PAIR_CNT; ++j) {
             const int q = q0 + j * PAIR_THREADS + tid;
-            int sh = (env_is_short(v[j].x) ? 1 : 0) + (env_is_short(v[j].y) ? 1 : 0) + (env_is_short(v[j].z) ? 1 : 0) +
-                     (env_is_short(v[j].w) ? 1 : 0);
-            sh = q < nq ? sh : 0;
-            total += sh;
-            before += q < w0q ? sh : 0;
+            int ct = env_tiny(v[j].x) + env_tiny(v[j].y) + env_tiny(v[j].z) + env_tiny(v[j].w);
+            int cm = env_mid(v[j].x) + env_mid(v[j].y) + env_mid(v[j].z) + env_mid(v[j].w);
+            ct = q < nq ? ct : 0; cm = q < nq ? cm : 0;
+            tt += ct; tm += cm;
+            bt += q < w0q ? ct : 0; bm += q < w0q ? cm : 0;
         }
     }
     if (tid < (int)(B & 3)) {                               // the last B % 4 envs
         const int64_t e = (int64_t)nq * 4 + tid;
-        const int sh = env_is_short(n_valid[e]) ? 1 : 0;
-        total += sh;
-        before += e < w0 ? sh : 0;
+        const int nv = n_valid[e];
+        tt += env_tiny(nv); tm += env_mid(nv);
+        bt += e < w0 ? env_tiny(nv) : 0; bm += e < w0 ? env_mid(nv) : 0;
     }
-    // the inclusive scan of this thread's short count over the workgroup
-    int cs = 0;
+    // the inclusive scans of this thread's class counts over the workgroup
+    int ct = 0, cm = 0;
     if (per <= PAIR_OWN) {
 #pragma unroll
-        for (int j = 0; j < PAIR_OWN; ++j) cs += env_is_short(own[j]) ? 1 : 0;
+        for (int j = 0; j < PAIR_OWN; ++j) { ct += env_tiny(own[j]); cm += env_mid(own[j]); }
     } else {
-        for (int64_t e = lo; e < hi; ++e) cs += env_is_short(n_valid[e]) ? 1 : 0;
+        for (int64_t e = lo; e < hi; ++e) { const int nv = n_valid[e]; ct += env_tiny(nv); cm += env_mid(nv); }
     }
-    int inc = cs;
+    int it = ct, im = cm;
 #pragma unroll
     for (int d = 1; d < WAVE; d <<= 1) {
-        const int v = __shfl_up(inc, d, WAVE);
-        if (lane >= d) inc += v;
+        const int vt = __shfl_up(it, d, WAVE), vm = __shfl_up(im, d, WAVE);
+        if (lane >= d) { it += vt; im += vm; }
     }
 #pragma unroll
-    for (int d = 1; d < WAVE; d <<= 1) { before += __shfl_xor(before, d, WAVE); total += __shfl_xor(total, d, WAVE); }
-    if (lane == WAVE - 1) red[0][wave] = inc;
-    if (lane == 0) { red[1][wave] = before; red[2][wave] = total; }
+    for (int d = 1; d < WAVE; d <<= 1) {
+        bt += __shfl_xor(bt, d, WAVE); bm += __shfl_xor(bm, d, WAVE);
+        tt += __shfl_xor(tt, d, WAVE); tm += __shfl_xor(tm, d, WAVE);
+    }
+    if (lane == WAVE - 1) { red[0][wave] = it; red[1][wave] = im; }
+    if (lane == 0) { red[2][wave] = bt; red[3][wave] = bm; red[4][wave] = tt; red[5][wave] = tm; }
     __syncthreads();
-    int base = 0; before = 0; total = 0;
+    int baset = 0, basem = 0; bt = 0; bm = 0; tt = 0; tm = 0;
 #pragma unroll
     for (int w = 0; w < PAIR_THREADS / WAVE; ++w) {
-        if (w < wave) base += red[0][w];
-        before += red[1][w]; total += red[2][w];
+        if (w < wave) { baset += red[0][w]; basem += red[1][w]; }
+        bt += red[2][w]; bm += red[3][w]; tt += red[4][w]; tm += red[5][w];
     }
-    int64_t rs = (int64_t)before + base + inc - cs;        // short envs before this thread's first env
-    int64_t rl = lo - rs;                                  // long envs before it
-    const int64_t first_long = ((int64_t)total + 1) / 2;
-    auto place = [&](int64_t e, int nv) __attribute__((always_inline)) {
-        if (env_is_short(nv)) {
-            int32_t* p = reinterpret_cast<int32_t*>(pairs + rs / 2);
-            p[rs & 1] = (int32_t)e;
-            if (rs == total - 1 && !(rs & 1)) p[1] = -1;   // odd count: the last short env sits alone
-            ++rs;
-        } else {
-            pairs[first_long + rl] = make_int2((int)e, -1);
-            ++rl;
-        }
-    };
+    int64_t rt_ = (int64_t)bt + baset + it - ct;           // tiny envs before this thread's first env
+    int64_t rm = (int64_t)bm + basem + im - cm;            // mid envs before it
+    int64_t rl = lo - rt_ - rm;                            // long envs before it
+    const int64_t first_tiny = ((int64_t)tm + 1) / 2;
+    const int64_t first_long = first_tiny + ((int64_t)tt + 3) / 4;
+    // every slot of every tile is written exactly once: an env writes the slot it starts in and the -1 of the slots
+    // that can only continue it; the last mid / tiny env also closes the rest of its tile
+    // (a macro, not a lambda: with the counters captured by reference the closure went through scratch memory, and a
+    // kernel with a private segment pays for it at every dispatch)
+#define PAIR_PLACE(E, NV)                                                                          \
+    do {                                                                                           \
+        const int64_t e_ = (E);                                                                    \
+        const int nv_ = (NV);                                                                      \
+        if (env_mid(nv_)) {                                                                        \
+            int32_t* p = reinterpret_cast<int32_t*>(pairs + rm / 2) + 2 * (rm & 1);               \
+            p[0] = (int32_t)e_; p[1] = -1;                                                         \
+            if (rm == tm - 1 && !(rm & 1)) { p[2] = -1; p[3] = -1; }                               \
+            ++rm;                                                                                  \
+        } else if (env_tiny(nv_)) {                                                                \
+            int32_t* p = reinterpret_cast<int32_t*>(pairs + first_tiny + rt_ / 4);                \
+            const int sl = (int)(rt_ & 3);                                                         \
+            p[sl] = (int32_t)e_;                                                                   \
+            if (rt_ == tt - 1) { if (sl < 1) p[1] = -1; if (sl < 2) p[2] = -1; if (sl < 3) p[3] = -1; } \
+            ++rt_;                                                                                 \
+        } else {                                                                                   \
+            pairs[first_long + rl] = make_int4((int)e_, -1, -1, -1);                               \
+            ++rl;                                                                                  \
+        }                                                                                          \
+    } while (0)
     if (per <= PAIR_OWN) {
 #pragma unroll
-        for (int j = 0; j < PAIR_OWN; ++j) if (lo + j < hi) place(lo + j, own[j]);
+        for (int j = 0; j < PAIR_OWN; ++j) if (lo + j < hi) PAIR_PLACE(lo + j, own[j]);
     } else {
-        for (int64_t e = lo; e < hi; ++e) place(e, n_valid[e]);
+        for (int64_t e = lo; e < hi; ++e) PAIR_PLACE(e, n_valid[e]);
     }
-    if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - total));
+#undef PAIR_PLACE
+    if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - tt - tm));
 }
 
 template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
@@ -936,7 +967,7 @@ int launch_all(FwdArgs a, bool pruned, bool pack, int cus, hipStream_t st) {
         const int64_t span = (int64_t)per * PAIR_THREADS;                                      // envs per workgroup
         wgs = (a.B + span - 1) / span;
         hipLaunchKernelGGL(cfg_pair_kernel, dim3((unsigned)wgs), dim3(PAIR_THREADS), 0, st, a.n_valid, a.B, span, per,
-                           const_cast<int2*>(a.pairs), const_cast<int32_t*>(a.n_packed));
+                           const_cast<int4*>(a.pairs), const_cast<int32_t*>(a.n_packed));
         rc = launch_one<DT, 2, ACT, MODE_HEAD, true>(a, cus, st);
     } else {
         rc = launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
@@ -980,9 +1011,9 @@ extern "C" int bsrl_cfg_pack(const bsrl_cfg_desc* d, const bsrl_cfg_params* p, v
 }
 
 namespace {
-// workspace layout: token-0 rows (B x 768 B), then the packed launch's tile table (B int2) and its tile count
+// workspace layout: token-0 rows (B x 768 B), then the packed launch's tile table (B int4) and its tile count
 int64_t ws_rows_bytes(int64_t B) { return B * 4 * WS_DWORDS * (int64_t)sizeof(uint32_t); }
-int64_t ws_pairs_bytes(int64_t B) { return (B * (int64_t)sizeof(int2) + 15) / 16 * 16 + 16; }
+int64_t ws_pairs_bytes(int64_t B) { return B * (int64_t)sizeof(int4) + 16; }
 }  // namespace
 
 extern "C" int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* d, int64_t B) {
@@ -1019,7 +1050,7 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.pairs = nullptr; a.n_packed = nullptr;
     if (pack) {
         char* tail = static_cast<char*>(workspace) + ws_rows_bytes(B);
-        a.pairs = reinterpret_cast<const int2*>(tail);
+        a.pairs = reinterpret_cast<const int4*>(tail);
         a.n_packed = reinterpret_cast<const int32_t*>(tail + ws_pairs_bytes(B) - 16);
     }
     if (workspace && !bsrl_aligned(workspace, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: workspace must be 16-byte aligned");

@@ -189,7 +189,7 @@ int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* desc);
 int bsrl_cfg_pack(const bsrl_cfg_desc* desc, const bsrl_cfg_params* params,
                   void* packed, bsrl_stream stream);
 /* Bytes of scratch the pruned two-launch form of bsrl_cfg_forward needs for B envs
- * (768 B per env for the parked rows + 8 B per env + 32 B for the tile table of
+ * (768 B per env for the parked rows + 16 B per env + 16 B for the tile table of
  * the packed launch), or 0 if the shape is unsupported. */
 int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
 /* obs (B, obs_ld) F32 or 16-bit; n_valid (B,) int32 or NULL (all valid).
@@ -200,9 +200,10 @@ int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
  * blocks 0..L-2 and the last block's attention and parks each env's token-0
  * row in the workspace, launch 2 runs the last block's output projection +
  * FFN and the heads on those rows, 16 envs per MFMA tile.  With n_valid given
- * and the full workspace, launch 1 also packs envs of at most 8 tokens
- * (n_valid <= 7) two to a 16-row tile (rows 0.. and 8.., block-diagonal key
- * mask; a one-workgroup kernel builds the tile table on the stream first):
+ * and the full workspace, launch 1 also packs short envs into shared 16-row
+ * tiles under a block-diagonal key mask: two of 5..8 tokens (n_valid 4..7) at
+ * rows 0 / 8, four of at most 4 tokens (n_valid <= 3) at rows 0 / 4 / 8 / 12
+ * (a small kernel builds the tile table on the stream first):
  * padded rows are what the reference computes and discards
  * (python/policy.py:1257-1260 masks them key-side), and an env's output bits
  * are the same packed or alone.  desc->flags = BSRL_CFG_NO_PACK keeps one env
