@@ -20,12 +20,13 @@ if ROOT not in sys.path:
 
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 # HBM bytes per forward of the headline workload (config[1], B = 16384, fp16, fused route with the final
-# block pruned: the HEAD + TAIL launch pair), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per
-# dispatch) scaled by what the same counters read for a plain 256 MiB device copy (--calib-copy 256):
-# FETCH_SIZE reads 131080 for 262144 KiB fetched (factor 2.000), WRITE_SIZE reads 262140 (factor 1.000).
-#   fetched: HEAD 13373 x 2.000 + TAIL 7784 x 2.000 KiB; written: HEAD 12288 + TAIL 13486 KiB
-# (profiles/cfg_forward_config1_b16384_f16.txt).  Other workloads report null.
-TRAFFIC_BYTES_CFG1_FUSED_PRUNED = int(((13373 + 7784) * 2.000 + 12288 + 13486) * 1024)
+# block pruned and short envs sharing tiles: tile-table kernel + HEAD + TAIL launches), from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain 256 MiB device
+# copy (--calib-copy 256): FETCH_SIZE reads 131085 for 262144 KiB fetched (factor 2.000), WRITE_SIZE reads 262144
+# (factor 1.000).
+#   fetched: (table 329 + HEAD 11614 + TAIL 7787) x 2.000 KiB; written: table 181 + HEAD 12288 + TAIL 13547 KiB
+# (profiles/cfg_forward_config1_b16384_f16.txt).  Other workloads, and --no-pack, report null.
+TRAFFIC_BYTES_CFG1_FUSED_PRUNED = int(((329 + 11614 + 7787) * 2.000 + 181 + 12288 + 13547) * 1024)
 HBM_PEAK_GBS = 8000.0
 
 
@@ -72,6 +73,7 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="override B (0 = the config's B)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-eager", action="store_true", help="skip the torch-ROCm eager leg")
+    ap.add_argument("--no-pack", action="store_true", help="fused route: one env per 16-row tile (no sharing of tiles by short envs)")
     ap.add_argument("--no-prune", action="store_true",
                     help="fused route: one persistent kernel computing every token of the last block")
     ap.add_argument("--calib-copy", type=int, default=0, metavar="MIB",
@@ -109,6 +111,7 @@ def main():
     m.load_state_dict(p)
     m = m.to(dev)
     m.prune_final = not args.no_prune
+    m.pack_short = not args.no_pack
     obs, k = obs_cpu.to(dev), k_cpu.to(dev)
     route = args.route
     if route == "auto":
@@ -139,9 +142,11 @@ def main():
     dev_ms_avg = sum(dev_ms) / len(dev_ms)
     value = B / (ms_per_step * 1e-3)
 
-    # FLOPs per forward: the dense algorithmic figure (every token of every block), and the
-    # EXECUTED figure when the fused route prunes the final block to token 0 (the reference's
-    # own n_queries path): the roofline fraction is quoted on executed work only.
+    # FLOPs per forward: the dense figure (every token of every block), and the ALGORITHMIC figure of the path as
+    # the reference runs it - the final block pruned to token 0 (its own n_queries path), every env's 16 token rows
+    # (padding rows included: the reference computes and masks them).  The roofline fraction is quoted on the
+    # algorithmic figure; what the matrix pipe is really issued (fewer tiles when short envs share them) is
+    # reported beside it as issued_frac.
     dense_flops = cm.flops_per_env(spec) * B
     pruned = (route == "fused" and m.prune_final) or route == "blocks"
     exec_flops = dense_flops
@@ -149,18 +154,37 @@ def main():
         d_, T_, F_ = spec.d, spec.T, spec.ffn
         saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the 15 unread tokens
         exec_flops = dense_flops - 2 * saved * B
+    # ... and, on the fused route, the 16-row tiles the first launch really runs: envs of 5..8 tokens go two to a
+    # tile, of at most 4 tokens four to a tile (same output bits), so the per-tile work is counted per tile
+    tiles, issued_flops = None, None
+    if route == "fused" and m.prune_final and m.pack_short and c["mask"] != "none" and spec.T == 16:
+        tiny, mid = int((k_cpu <= 3).sum()), int(((k_cpu >= 4) & (k_cpu <= 7)).sum())
+        tiles = (mid + 1) // 2 + (tiny + 3) // 4 + (B - tiny - mid)
+        d_, T_, F_, L_ = spec.d, spec.T, spec.ffn, spec.n_layers
+        e_ = spec.prop_dim * d_ + (T_ - 1) * spec.obj_dim * d_
+        per_layer = 3 * T_ * d_ * d_ + 2 * T_ * T_ * d_ + T_ * d_ * d_ + 2 * T_ * d_ * F_
+        head_tile = 2 * (e_ + (L_ - 1) * per_layer + 3 * T_ * d_ * d_ + 2 * T_ * T_ * d_)
+        tail_env = 2 * (d_ * d_ + 2 * d_ * F_ + d_ * spec.n_out)
+        assert head_tile + tail_env == exec_flops // B
+        issued_flops = tiles * head_tile + B * tail_env
     achieved = exec_flops / (dev_ms_avg * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[dtype]
-    kname = ("cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
+    kname = ("cfg_pair_kernel + cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0, short envs share tiles)"
+             if tiles is not None else
+             "cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
              "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else
              "cfg_embed_kernel + blocks_kernel (final block pruned to token 0) + heads" if route == "blocks" else
              "launch train (per-op route)")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(achieved / peak, 4),
-                "traffic": TRAFFIC_BYTES_CFG1_FUSED_PRUNED if (pruned and args.config == 1 and B == 16384) else None,
+                "traffic": TRAFFIC_BYTES_CFG1_FUSED_PRUNED if (tiles is not None and args.config == 1 and B == 16384) else None,
                 "kernel": kname,
                 "launch_ms_avg": round(dev_ms_avg, 4), "launch_ms_p50": round(dev_ms[len(dev_ms) // 2], 4),
                 "flop_per_launch": exec_flops, "dense_flop_per_forward": dense_flops,
+                # MFMA work really issued when short envs share tiles (the algorithmic figure above counts every env's
+                # 16 token rows, as the reference computes them)
+                "tiles_per_forward": tiles, "issued_flop_per_launch": issued_flops,
+                "issued_frac": None if issued_flops is None else round(issued_flops / (dev_ms_avg * 1e-3) / 1e12 / peak, 4),
                 "dense_equivalent_frac": round(dense_flops / (dev_ms_avg * 1e-3) / 1e12 / peak, 4)}
 
     out = {"metric": "policy fwd env-samples/sec at B=16384 fp16 (1 GPU); % of MFMA roofline",
