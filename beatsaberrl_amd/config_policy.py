@@ -78,7 +78,7 @@ class ConfigPolicy(nn.Module):
         # final-block query pruning on the fused route (the reference's n_queries path,
         # python/policy.py:533-539): exact; False = one persistent kernel computing every token
         self.prune_final = True
-        # fused route, pruned form, key counts given: envs of at most 8 / 4 tokens share 16-row tiles two / four at a time (same bits)
+        # fused route, pruned form, key counts given: envs of at most 8 tokens share 16-row tiles in twos, of at most 4 tokens ride behind a 9..12-token env or in fours (same bits)
         self.pack_short = True
         self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
                      "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}

@@ -129,7 +129,8 @@ constexpr int TAIL_ENVS = 16;
 constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
 
 // PACK (HEAD launch only): short envs share a 16-row tile under a block-diagonal key mask - two of at most 8 tokens
-// (rows 0.. and 8..) or four of at most 4 tokens (rows 0.., 4.., 8.., 12..).  Every per-row computation (GEMMs,
+// (rows 0.. and 8..), four of at most 4 tokens (rows 0.., 4.., 8.., 12..), or one of at most 12 tokens with one of
+// at most 4 behind it (rows 12..).  Every per-row computation (GEMMs,
 // LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
 // multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
 // and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
@@ -811,12 +812,13 @@ bool shape_ok(const bsrl_cfg_desc* d) {
 }
 int64_t frag_bytes(const bsrl_cfg_desc* d) { return (int64_t)total_stages(d->n_layers, d->ffn) * STAGE_U4 * 16; }
 
-// Tile table of the packed HEAD launch.  Envs of at most 4 tokens (n_valid <= 3) are "tiny", of 5..8 tokens "mid",
-// the rest long; each class keeps env order (a stable split, so the table is a function of the batch alone).  Tiles:
-// the mid pairs (mid[2 i], mid[2 i + 1]) at rows 0 / 8 (a lone last one if their count is odd), then the tiny quads
-// (tiny[4 i .. 4 i + 3]) at rows 0 / 4 / 8 / 12 (the last tile may hold fewer), then one tile per long env.
-// pairs[t] = the env that starts in each 4-row slot, -1 where the slot continues the env before it (or is empty
-// after the last tiny env); *n_packed = the number of tiles.
+// Tile table of the packed HEAD launch.  Classes by token count (1 + n_valid): tiny <= 4, mid 5..8, host 9..12, long
+// the rest; each class keeps env order (a stable split, so the table is a function of the batch alone).  Tiles, in
+// this order: the mid pairs (mid[2 i], mid[2 i + 1]) at rows 0 / 8 (a lone last one if their count is odd); the quads
+// of the tiny envs that found no host, at rows 0 / 4 / 8 / 12 (the last tile may hold fewer); one tile per host env,
+// host[i] at rows 0..11 with tiny[i] at rows 12..15 while tiny envs last; one tile per long env.
+// pairs[t] = the env that starts in each 4-row slot, -1 where the slot continues the env before it (or is empty);
+// *n_packed = the number of tiles.
 // Workgroup b owns the envs [b span, (b + 1) span), `per` consecutive ones per thread.  Every workgroup counts the
 // classes of the WHOLE batch for itself (coalesced 16-byte reads out of L2: cheaper than a second launch or a
 // cross-workgroup hand-off), which gives it both the counts before its span and the totals.
@@ -824,12 +826,12 @@ constexpr int PAIR_THREADS = 256;
 constexpr int PAIR_MAX_WGS = 256;
 constexpr int PAIR_OWN = 4;                                // own envs a thread keeps in registers
 constexpr int PAIR_CNT = 16;                               // 16-byte loads (4 key counts each) per thread and counting pass
-// class counts travel as one int: tiny in the low 16 bits is not enough for a batch, so two ints - [0] tiny, [1] mid
 __device__ __forceinline__ int env_tiny(int nv) { return nv >= 0 && nv <= 3 ? 1 : 0; }
 __device__ __forceinline__ int env_mid(int nv) { return nv >= 4 && nv <= 7 ? 1 : 0; }
+__device__ __forceinline__ int env_host(int nv) { return nv >= 8 && nv <= 11 ? 1 : 0; }
 __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n_valid, int64_t B, int64_t span, int per,
                                                                 int4* pairs, int32_t* n_packed) {
-    __shared__ int red[6][PAIR_THREADS / WAVE];
+    __shared__ int red[9][PAIR_THREADS / WAVE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t w0 = (int64_t)blockIdx.x * span;
     // Every global load of the common case leaves in one batch (own envs first, then PAIR_CNT loads per thread per
@@ -842,8 +844,9 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
         const int v = n_valid[lo + j < B ? lo + j : B - 1];
         own[j] = lo + j < hi ? v : -1;
     }
-    // class counts of the whole batch, four envs per load (n_valid is 16-byte aligned on this path, B < 2^31)
-    int bt = 0, bm = 0, tt = 0, tm = 0;                     // tiny / mid before this workgroup's span, and in total
+    // class counts of the whole batch, four envs per load (n_valid is 16-byte aligned on this path, B < 2^31):
+    // [0] tiny, [1] mid, [2] host; b* = before this workgroup's span, t* = in total
+    int bt = 0, bm = 0, bh = 0, tt = 0, tm = 0, th = 0;
     const int nq = (int)(B >> 2), w0q = (int)(w0 >> 2);     // w0 is a multiple of PAIR_THREADS
     const int4* nvq = reinterpret_cast<const int4*>(n_valid);
     for (int q0 = 0; q0 < nq; q0 += PAIR_CNT * PAIR_THREADS) {
@@ -853,54 +856,63 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
 #pragma unroll
         for (int j = 0; j < PAIR_CNT; ++j) {
             const int q = q0 + j * PAIR_THREADS + tid;
-            int ct = env_tiny(v[j].x) + env_tiny(v[j].y) + env_tiny(v[j].z) + env_tiny(v[j].w);
-            int cm = env_mid(v[j].x) + env_mid(v[j].y) + env_mid(v[j].z) + env_mid(v[j].w);
-            ct = q < nq ? ct : 0; cm = q < nq ? cm : 0;
-            tt += ct; tm += cm;
-            bt += q < w0q ? ct : 0; bm += q < w0q ? cm : 0;
+            int c0 = env_tiny(v[j].x) + env_tiny(v[j].y) + env_tiny(v[j].z) + env_tiny(v[j].w);
+            int c1 = env_mid(v[j].x) + env_mid(v[j].y) + env_mid(v[j].z) + env_mid(v[j].w);
+            int c2 = env_host(v[j].x) + env_host(v[j].y) + env_host(v[j].z) + env_host(v[j].w);
+            c0 = q < nq ? c0 : 0; c1 = q < nq ? c1 : 0; c2 = q < nq ? c2 : 0;
+            tt += c0; tm += c1; th += c2;
+            bt += q < w0q ? c0 : 0; bm += q < w0q ? c1 : 0; bh += q < w0q ? c2 : 0;
         }
     }
     if (tid < (int)(B & 3)) {                               // the last B % 4 envs
         const int64_t e = (int64_t)nq * 4 + tid;
         const int nv = n_valid[e];
-        tt += env_tiny(nv); tm += env_mid(nv);
-        bt += e < w0 ? env_tiny(nv) : 0; bm += e < w0 ? env_mid(nv) : 0;
+        tt += env_tiny(nv); tm += env_mid(nv); th += env_host(nv);
+        if (e < w0) { bt += env_tiny(nv); bm += env_mid(nv); bh += env_host(nv); }
     }
     // the inclusive scans of this thread's class counts over the workgroup
-    int ct = 0, cm = 0;
+    int ct = 0, cm = 0, ch = 0;
     if (per <= PAIR_OWN) {
 #pragma unroll
-        for (int j = 0; j < PAIR_OWN; ++j) { ct += env_tiny(own[j]); cm += env_mid(own[j]); }
+        for (int j = 0; j < PAIR_OWN; ++j) { ct += env_tiny(own[j]); cm += env_mid(own[j]); ch += env_host(own[j]); }
     } else {
-        for (int64_t e = lo; e < hi; ++e) { const int nv = n_valid[e]; ct += env_tiny(nv); cm += env_mid(nv); }
+        for (int64_t e = lo; e < hi; ++e) { const int nv = n_valid[e]; ct += env_tiny(nv); cm += env_mid(nv); ch += env_host(nv); }
     }
-    int it = ct, im = cm;
+    int it = ct, im = cm, ih = ch;
 #pragma unroll
     for (int d = 1; d < WAVE; d <<= 1) {
-        const int vt = __shfl_up(it, d, WAVE), vm = __shfl_up(im, d, WAVE);
-        if (lane >= d) { it += vt; im += vm; }
+        const int vt = __shfl_up(it, d, WAVE), vm = __shfl_up(im, d, WAVE), vh = __shfl_up(ih, d, WAVE);
+        if (lane >= d) { it += vt; im += vm; ih += vh; }
     }
 #pragma unroll
     for (int d = 1; d < WAVE; d <<= 1) {
-        bt += __shfl_xor(bt, d, WAVE); bm += __shfl_xor(bm, d, WAVE);
-        tt += __shfl_xor(tt, d, WAVE); tm += __shfl_xor(tm, d, WAVE);
+        bt += __shfl_xor(bt, d, WAVE); bm += __shfl_xor(bm, d, WAVE); bh += __shfl_xor(bh, d, WAVE);
+        tt += __shfl_xor(tt, d, WAVE); tm += __shfl_xor(tm, d, WAVE); th += __shfl_xor(th, d, WAVE);
     }
-    if (lane == WAVE - 1) { red[0][wave] = it; red[1][wave] = im; }
-    if (lane == 0) { red[2][wave] = bt; red[3][wave] = bm; red[4][wave] = tt; red[5][wave] = tm; }
+    if (lane == WAVE - 1) { red[0][wave] = it; red[1][wave] = im; red[2][wave] = ih; }
+    if (lane == 0) {
+        red[3][wave] = bt; red[4][wave] = bm; red[5][wave] = bh;
+        red[6][wave] = tt; red[7][wave] = tm; red[8][wave] = th;
+    }
     __syncthreads();
-    int baset = 0, basem = 0; bt = 0; bm = 0; tt = 0; tm = 0;
+    int baset = 0, basem = 0, baseh = 0; bt = 0; bm = 0; bh = 0; tt = 0; tm = 0; th = 0;
 #pragma unroll
     for (int w = 0; w < PAIR_THREADS / WAVE; ++w) {
-        if (w < wave) { baset += red[0][w]; basem += red[1][w]; }
-        bt += red[2][w]; bm += red[3][w]; tt += red[4][w]; tm += red[5][w];
+        if (w < wave) { baset += red[0][w]; basem += red[1][w]; baseh += red[2][w]; }
+        bt += red[3][w]; bm += red[4][w]; bh += red[5][w];
+        tt += red[6][w]; tm += red[7][w]; th += red[8][w];
     }
     int64_t rt_ = (int64_t)bt + baset + it - ct;           // tiny envs before this thread's first env
     int64_t rm = (int64_t)bm + basem + im - cm;            // mid envs before it
-    int64_t rl = lo - rt_ - rm;                            // long envs before it
-    const int64_t first_tiny = ((int64_t)tm + 1) / 2;
-    const int64_t first_long = first_tiny + ((int64_t)tt + 3) / 4;
+    int64_t rh = (int64_t)bh + baseh + ih - ch;            // host envs before it
+    int64_t rl = lo - rt_ - rm - rh;                       // long envs before it
+    const int64_t loose = tt > th ? tt - th : 0;           // tiny envs without a host
+    const int64_t first_quad = ((int64_t)tm + 1) / 2;
+    const int64_t first_host = first_quad + (loose + 3) / 4;
+    const int64_t first_long = first_host + th;
     // every slot of every tile is written exactly once: an env writes the slot it starts in and the -1 of the slots
-    // that can only continue it; the last mid / tiny env also closes the rest of its tile
+    // that can only continue it; the last mid / loose tiny env also closes the rest of its tile, a host without a
+    // tiny env its own last slot
     // (a macro, not a lambda: with the counters captured by reference the closure went through scratch memory, and a
     // kernel with a private segment pays for it at every dispatch)
 #define PAIR_PLACE(E, NV)                                                                          \
@@ -913,11 +925,21 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
             if (rm == tm - 1 && !(rm & 1)) { p[2] = -1; p[3] = -1; }                               \
             ++rm;                                                                                  \
         } else if (env_tiny(nv_)) {                                                                \
-            int32_t* p = reinterpret_cast<int32_t*>(pairs + first_tiny + rt_ / 4);                \
-            const int sl = (int)(rt_ & 3);                                                         \
-            p[sl] = (int32_t)e_;                                                                   \
-            if (rt_ == tt - 1) { if (sl < 1) p[1] = -1; if (sl < 2) p[2] = -1; if (sl < 3) p[3] = -1; } \
+            if (rt_ < th) {                                                                        \
+                reinterpret_cast<int32_t*>(pairs + first_host + rt_)[3] = (int32_t)e_;            \
+            } else {                                                                               \
+                const int64_t q_ = rt_ - th;                                                       \
+                int32_t* p = reinterpret_cast<int32_t*>(pairs + first_quad + q_ / 4);             \
+                const int sl = (int)(q_ & 3);                                                      \
+                p[sl] = (int32_t)e_;                                                               \
+                if (rt_ == tt - 1) { if (sl < 1) p[1] = -1; if (sl < 2) p[2] = -1; if (sl < 3) p[3] = -1; } \
+            }                                                                                      \
             ++rt_;                                                                                 \
+        } else if (env_host(nv_)) {                                                                \
+            int32_t* p = reinterpret_cast<int32_t*>(pairs + first_host + rh);                     \
+            p[0] = (int32_t)e_; p[1] = -1; p[2] = -1;                                              \
+            if (rh >= tt) p[3] = -1;                                                               \
+            ++rh;                                                                                  \
         } else {                                                                                   \
             pairs[first_long + rl] = make_int4((int)e_, -1, -1, -1);                               \
             ++rl;                                                                                  \
@@ -930,7 +952,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
         for (int64_t e = lo; e < hi; ++e) PAIR_PLACE(e, n_valid[e]);
     }
 #undef PAIR_PLACE
-    if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - tt - tm));
+    if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - tt - tm - th));
 }
 
 template <typename DT, int RT, int ACT, int MODE, bool PACK = false>

@@ -155,11 +155,13 @@ def main():
         saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the 15 unread tokens
         exec_flops = dense_flops - 2 * saved * B
     # ... and, on the fused route, the 16-row tiles the first launch really runs: envs of 5..8 tokens go two to a
-    # tile, of at most 4 tokens four to a tile (same output bits), so the per-tile work is counted per tile
+    # tile, of at most 4 tokens behind an env of 9..12 tokens or four to a tile (same output bits), so the per-tile
+    # work is counted per tile
     tiles, issued_flops = None, None
     if route == "fused" and m.prune_final and m.pack_short and c["mask"] != "none" and spec.T == 16:
         tiny, mid = int((k_cpu <= 3).sum()), int(((k_cpu >= 4) & (k_cpu <= 7)).sum())
-        tiles = (mid + 1) // 2 + (tiny + 3) // 4 + (B - tiny - mid)
+        host = int(((k_cpu >= 8) & (k_cpu <= 11)).sum())                   # 9..12 tokens: a tiny env rides in rows 12..15
+        tiles = (mid + 1) // 2 + (max(tiny - host, 0) + 3) // 4 + (B - tiny - mid)
         d_, T_, F_, L_ = spec.d, spec.T, spec.ffn, spec.n_layers
         e_ = spec.prop_dim * d_ + (T_ - 1) * spec.obj_dim * d_
         per_layer = 3 * T_ * d_ * d_ + 2 * T_ * T_ * d_ + T_ * d_ * d_ + 2 * T_ * d_ * F_

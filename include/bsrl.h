@@ -202,8 +202,9 @@ int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
  * FFN and the heads on those rows, 16 envs per MFMA tile.  With n_valid given
  * and the full workspace, launch 1 also packs short envs into shared 16-row
  * tiles under a block-diagonal key mask: two of 5..8 tokens (n_valid 4..7) at
- * rows 0 / 8, four of at most 4 tokens (n_valid <= 3) at rows 0 / 4 / 8 / 12
- * (a small kernel builds the tile table on the stream first):
+ * rows 0 / 8; one of at most 4 tokens (n_valid <= 3) at rows 12.. behind one of
+ * 9..12 tokens, or four of them at rows 0 / 4 / 8 / 12 (a small kernel builds
+ * the tile table on the stream first):
  * padded rows are what the reference computes and discards
  * (python/policy.py:1257-1260 masks them key-side), and an env's output bits
  * are the same packed or alone.  desc->flags = BSRL_CFG_NO_PACK keeps one env

@@ -230,11 +230,11 @@ def test_fused_route_packed_tiles_at_a_batch_with_several_envs_per_pairing_threa
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("case", ["uniform", "all_short", "all_long", "one_short", "odd_short", "alternating", "all_tiny",
-                                  "all_mid", "five_tiny"])
+                                  "all_mid", "five_tiny", "host_tiny", "few_hosts", "many_hosts"])
 @pytest.mark.parametrize("B", [1, 9, 700, 4099])
 def test_fused_route_packed_tiles_give_the_unpacked_bits(dtype, case, B):
-    """`pack_short` (envs of 5..8 tokens two to a 16-row tile, of at most 4 tokens four to a tile, in the pruned form's
-    first launch) against one env per tile: logits and values are bitwise equal for every mix of short and long envs, and both match the oracle."""
+    """`pack_short` (envs of 5..8 tokens two to a 16-row tile, of at most 4 tokens behind an env of 9..12 tokens or four
+    to a tile, in the pruned form's first launch) against one env per tile: logits and values are bitwise equal for every mix of short and long envs, and both match the oracle."""
     c = cm.CONFIGS[1]
     spec = c["spec"]
     p, m = _build(spec, c["w_seed"], dtype, "fused")
@@ -256,6 +256,14 @@ def test_fused_route_packed_tiles_give_the_unpacked_bits(dtype, case, B):
     elif case == "five_tiny":
         k = 8 + k % 8
         k[: min(B, 5)] = torch.tensor([0, 3, 2, 1, 3], dtype=torch.int32)[: min(B, 5)]
+    elif case == "host_tiny":                     # every tiny env finds a 9..12-token host
+        k = torch.where(torch.arange(B) % 2 == 0, 8 + k % 4, k % 4).to(torch.int32)
+    elif case == "few_hosts":                     # more tiny envs than hosts: the rest go four to a tile
+        k = k % 4
+        k[::7] = 9
+    elif case == "many_hosts":                    # more hosts than tiny envs
+        k = 8 + k % 4
+        k[::5] = 2
     elif case == "alternating":
         k = torch.where(torch.arange(B) % 2 == 0, k % 8, 8 + k % 8).to(torch.int32)
     od, kd = obs.to(DEV), k.to(DEV)
