@@ -215,12 +215,14 @@ def test_fused_route_invariants(prune):
     assert (l6 - lg).abs().max().item() < 5e-3
 
 
-def test_fused_route_packed_tiles_at_a_batch_with_several_envs_per_pairing_thread():
-    """B > 65536: the tile-table kernel walks several envs per thread; same bits as one env per tile."""
+@pytest.mark.parametrize("B", [70001, 270003])
+def test_fused_route_packed_tiles_at_a_batch_with_several_envs_per_pairing_thread(B):
+    """B > 65536: the tile-table kernel walks several envs per thread (kept in registers up to 4, re-read from memory
+    beyond: B > 262144); same bits as one env per tile."""
     c = cm.CONFIGS[1]
     spec = c["spec"]
     _, m = _build(spec, c["w_seed"], "f16", "fused")
-    obs, k = cm.make_inputs(spec, 70001, 77, "uniform")
+    obs, k = cm.make_inputs(spec, B, 77, "uniform")
     od, kd = obs.to(DEV), k.to(DEV)
     lg1, v1 = m.forward_stacked(od, kd)
     m.pack_short = False
