@@ -285,6 +285,32 @@ def test_fused_route_packed_tiles_give_the_unpacked_bits(dtype, case, B):
     assert torch.equal(lg2, lg1) and torch.equal(v2, v1)
 
 
+def test_fused_route_packed_forward_replays_in_a_graph_with_new_key_counts():
+    """The packed forward is capturable: the tile table is rebuilt on the device by every replay (its grid does not
+    depend on the key counts), so a replay with new obs AND new key counts in the static buffers returns the eager bits."""
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    _, m = _build(spec, c["w_seed"], "f16", "fused")
+    B = 3000
+    obs0, k0 = cm.make_inputs(spec, B, 1, "uniform")
+    s_obs, s_k = obs0.to(DEV), k0.to(DEV)
+    m.forward_stacked(s_obs, s_k)                                  # warm-up: image, workspace
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        g_lg, g_v = m.forward_stacked(s_obs, s_k)
+    for seed, mask in ((5, "uniform"), (6, "quarter_empty"), (7, "none"), (8, "uniform")):
+        obs, k = cm.make_inputs(spec, B, seed, mask)
+        s_obs.copy_(obs.to(DEV))
+        s_k.copy_(k.to(DEV))
+        g.replay()
+        got_lg, got_v = g_lg.clone(), g_v.clone()
+        x = torch.randn(300, 300, device=DEV)
+        (x @ x).sum().item()                                       # unrelated eager work and a sync between replays
+        lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+        assert torch.equal(got_lg, lg) and torch.equal(got_v, v), seed
+
+
 def test_fused_unsupported_shapes_fall_to_ops_route():
     for ci in (2, 3):
         spec = cm.CONFIGS[ci]["spec"]
