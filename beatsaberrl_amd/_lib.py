@@ -8,8 +8,9 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
+CFG_STATIC_MAX_ENVS = 16384     # BSRL_CFG_STATIC_MAX_ENVS: batch limit of bsrl_cfg_forward_static
 
 F32, F16, BF16 = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
@@ -62,6 +63,7 @@ SIGNATURES = {
     "bsrl_cfg_pack": (_i32, [C.POINTER(CfgDesc), C.POINTER(CfgParams), _p, _p]),
     "bsrl_cfg_workspace_size": (_i64, [C.POINTER(CfgDesc), _i64]),
     "bsrl_cfg_forward": (_i32, [C.POINTER(CfgDesc), _p, _p, _i64, _i32, _p, _p, _p, _i64, _p, _i64, _p]),
+    "bsrl_cfg_forward_static": (_i32, [C.POINTER(CfgDesc), _p, _p, _i64, _i32, _p, _p, _p, _i64, _p]),
     "bsrl_blocks_pack_size": (_i64, [C.POINTER(BlocksDesc)]),
     "bsrl_blocks_pack": (_i32, [C.POINTER(BlocksDesc), C.POINTER(BlocksParams), _p, _p]),
     "bsrl_blocks_forward": (_i32, [C.POINTER(BlocksDesc), _p, _p, _p, _p, _p, _i64, _p]),

@@ -26,6 +26,7 @@
 // benchmark-config model; the weight image is the analogue of the reference's
 // flat fp16 replica buffer (python/fp16_linear.py:249-346).
 #include "bsrl_common.h"
+#include <mutex>
 
 namespace {
 
@@ -1043,15 +1044,19 @@ extern "C" int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* d, int64_t B) {
     return ws_rows_bytes(B) + ws_pairs_bytes(B);
 }
 
-extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
-                                int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
-                                void* workspace, int64_t workspace_bytes, bsrl_stream stream) {
-    if (!d || !packed || !obs || !logits || !value) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: null pointer");
+namespace {
+// Shared body of the two forward entry points.  `rows` = the parked token-0 rows (768 B per env) or null (one-launch
+// form); `table` = the packed launch's tile table (B int4 + 16 B for the tile count) or null (one env per tile).
+int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
+                     int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
+                     void* rows, void* table, hipStream_t st) {
+    if (!d || !packed || !obs || !logits || !value) BSRL_FAIL(BSRL_EINVAL, "%s: null pointer", who);
     if (!shape_ok(d)) return BSRL_UNSUPPORTED;
-    if (B < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: negative batch");
-    if (obs_dtype != BSRL_F32 && obs_dtype != d->dtype) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: obs must be F32 or the stream dtype");
-    if (obs_ld < d->prop_dim + (d->T - 1) * d->obj_dim) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: obs_ld smaller than an obs row");
-    if (!bsrl_aligned(packed, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: image must be 16-byte aligned");
+    if (B < 0) BSRL_FAIL(BSRL_EINVAL, "%s: negative batch", who);
+    if (obs_dtype != BSRL_F32 && obs_dtype != d->dtype) BSRL_FAIL(BSRL_EINVAL, "%s: obs must be F32 or the stream dtype", who);
+    if (obs_ld < d->prop_dim + (d->T - 1) * d->obj_dim) BSRL_FAIL(BSRL_EINVAL, "%s: obs_ld smaller than an obs row", who);
+    if (!bsrl_aligned(packed, 16)) BSRL_FAIL(BSRL_EINVAL, "%s: image must be 16-byte aligned", who);
+    if (rows && !bsrl_aligned(rows, 16)) BSRL_FAIL(BSRL_EINVAL, "%s: workspace must be 16-byte aligned", who);
     if (B == 0) return BSRL_OK;
     FwdArgs a;
     a.frags = static_cast<const uint4*>(packed);
@@ -1061,22 +1066,19 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     a.n_valid = n_valid; a.logits = logits; a.value = value; a.B = B;
     a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
-    a.ws = static_cast<uint32_t*>(workspace);
+    a.ws = static_cast<uint32_t*>(rows);
     // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
-    const bool pruned = workspace && workspace_bytes >= ws_rows_bytes(B) && d->ffn % 64 == 0;
-    // short envs share tiles when the caller gives key counts, the workspace holds the tile table and the descriptor
+    const bool pruned = rows && d->ffn % 64 == 0;
+    // short envs share tiles when the caller gives key counts, there is room for the tile table and the descriptor
     // does not switch it off (n_valid 16-byte aligned: the table kernel reads it four at a time); B < 2^31 - 1 keeps
     // env ids in the table's int32
-    const bool pack = pruned && n_valid && bsrl_aligned(n_valid, 16) && !(d->flags & BSRL_CFG_NO_PACK) && B < (int64_t)0x7fffffff &&
-                      workspace_bytes >= ws_rows_bytes(B) + ws_pairs_bytes(B);
+    const bool pack = pruned && table && n_valid && bsrl_aligned(n_valid, 16) && !(d->flags & BSRL_CFG_NO_PACK) &&
+                      B < (int64_t)0x7fffffff;
     a.pairs = nullptr; a.n_packed = nullptr;
     if (pack) {
-        char* tail = static_cast<char*>(workspace) + ws_rows_bytes(B);
-        a.pairs = reinterpret_cast<const int4*>(tail);
-        a.n_packed = reinterpret_cast<const int32_t*>(tail + ws_pairs_bytes(B) - 16);
+        a.pairs = static_cast<const int4*>(table);
+        a.n_packed = reinterpret_cast<const int32_t*>(static_cast<const char*>(table) + ws_pairs_bytes(B) - 16);
     }
-    if (workspace && !bsrl_aligned(workspace, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward: workspace must be 16-byte aligned");
-    hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
@@ -1086,6 +1088,69 @@ extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, cons
     else
         rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, pack, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, pack, cus, st);
     if (rc != BSRL_OK) return rc;
-    BSRL_CHECK_LAUNCH("bsrl_cfg_forward");
+    BSRL_CHECK_LAUNCH(who);
     return BSRL_OK;
+}
+}  // namespace
+
+extern "C" int bsrl_cfg_forward(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
+                                int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
+                                void* workspace, int64_t workspace_bytes, bsrl_stream stream) {
+    void* rows = nullptr;
+    void* table = nullptr;
+    if (workspace && B > 0 && workspace_bytes >= ws_rows_bytes(B)) {
+        rows = workspace;
+        if (workspace_bytes >= ws_rows_bytes(B) + ws_pairs_bytes(B)) table = static_cast<char*>(workspace) + ws_rows_bytes(B);
+    }
+    return cfg_forward_impl("bsrl_cfg_forward", d, packed, obs, obs_ld, obs_dtype, n_valid, logits, value, B, rows, table,
+                            static_cast<hipStream_t>(stream));
+}
+
+// ---- the same forward for callers that cannot allocate ---------------------------------------------------------
+// The parked rows and the tile table live in a file-scope device array instead of a caller workspace.  Every GPU the
+// library runs on holds its own copy of the array, at its own address, until the process ends.
+namespace {
+constexpr int64_t STATIC_MAX_ENVS = BSRL_CFG_STATIC_MAX_ENVS;
+constexpr int64_t STATIC_ROWS_BYTES = STATIC_MAX_ENVS * 4 * WS_DWORDS * (int64_t)sizeof(uint32_t);
+constexpr int64_t STATIC_TABLE_BYTES = STATIC_MAX_ENVS * (int64_t)sizeof(int4) + 16;
+static __device__ __align__(256) unsigned char scratch[STATIC_ROWS_BYTES + STATIC_TABLE_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[MAX_DEVICES] = {};       // device address of `scratch` on each device, taken once per device
+
+// `scratch` in host code is only a handle for the runtime: the array's device address on the current device comes from
+// hipGetSymbolAddress, and that address is what kernels and copies get.
+int scratch_on_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) BSRL_FAIL(BSRL_ELAUNCH, "bsrl_cfg_forward_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            BSRL_FAIL(BSRL_ELAUNCH, "bsrl_cfg_forward_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return BSRL_OK;
+}
+}  // namespace
+
+extern "C" int bsrl_cfg_forward_static(const bsrl_cfg_desc* d, const void* packed, const void* obs, int64_t obs_ld,
+                                       int obs_dtype, const int32_t* n_valid, float* logits, float* value, int64_t B,
+                                       bsrl_stream stream) {
+    if (B > STATIC_MAX_ENVS)
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_cfg_forward_static: B = %lld exceeds the built-in scratch (%lld envs); "
+                  "use bsrl_cfg_forward with a workspace", (long long)B, (long long)STATIC_MAX_ENVS);
+    if (d && shape_ok(d) && d->ffn % 64 != 0) return BSRL_UNSUPPORTED;    // the two-launch form needs it (see above)
+    void* base = nullptr;
+    const int rc = scratch_on_current_device(&base);
+    if (rc != BSRL_OK) return rc;
+    // fixed split of the array, whatever B: rows first, table behind the rows of the largest batch.  Nothing in either
+    // part has to start at zero: the first launch writes the row of every env and every table slot the second reads.
+    return cfg_forward_impl("bsrl_cfg_forward_static", d, packed, obs, obs_ld, obs_dtype, n_valid, logits, value, B,
+                            base, static_cast<char*>(base) + STATIC_ROWS_BYTES, static_cast<hipStream_t>(stream));
 }

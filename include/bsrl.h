@@ -216,6 +216,26 @@ int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      int64_t B, void* workspace, int64_t workspace_bytes,
                      bsrl_stream stream);
 
+/* bsrl_cfg_forward for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference (whose ops allocate their outputs,
+ * layer_norm.cu:545-547).  Same arguments and results as bsrl_cfg_forward in its
+ * two-launch form with short envs sharing tiles, bit for bit, but the parked
+ * rows and the tile table live in a device array built into the library
+ * (BSRL_CFG_STATIC_MAX_ENVS * 784 + 16 bytes, held on every GPU the library is
+ * used on until the process ends) instead of a caller workspace; the call
+ * allocates and frees nothing.  B > BSRL_CFG_STATIC_MAX_ENVS is an error
+ * (BSRL_EINVAL); ffn not a multiple of 64 returns BSRL_UNSUPPORTED.  Every call
+ * on one GPU shares that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race - serialise them or use bsrl_cfg_forward
+ * with one workspace per stream.  Nothing in the array has to be cleared
+ * between calls. */
+#define BSRL_CFG_STATIC_MAX_ENVS 16384
+int bsrl_cfg_forward_static(const bsrl_cfg_desc* desc, const void* packed,
+                            const void* obs, int64_t obs_ld, int obs_dtype,
+                            const int32_t* n_valid, float* logits, float* value,
+                            int64_t B, bsrl_stream stream);
+
 /* ---- NotePolicy front end --------------------------------------------------
  * One pass over the (B, 630) observation that writes every encoder input and
  * the additive key bias.  Replaces the preamble of the reference forward
