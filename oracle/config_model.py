@@ -36,7 +36,11 @@ invariants "masked slots cannot change outputs", "full mask == no mask" and
 `forward(..., emulate=...)` additionally restates the rounding points of the
 16-bit stream (weights and every GEMM operand rounded to fp16/bf16, fp32
 accumulate, fp32 LayerNorm/softmax statistics) so a 16-bit kernel can be
-compared against its own precision class as well as against fp32.
+compared against its own precision class as well as against fp32.  That branch is
+pinned too (tests/test_oracle_emulate.py): the casts on hand-picked ties and against
+an independent bit-pattern rounding; a float64 restatement with an explicit cast at
+each rounding point, matched on the median env (single-ulp flips aside) while every
+one-rounding-point mutant of it is rejected; torch's own CPU 16-bit kernels per op.
 """
 
 from __future__ import annotations

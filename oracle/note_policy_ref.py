@@ -26,7 +26,13 @@ by the reference's own properties (python/tests/test_arch_ab_options.py:131-139,
 
 `forward(..., emulate="f16")` restates the rounding points of the 16-bit stream (obs,
 weights and every GEMM operand rounded, fp32 accumulate, fp32 LayerNorm / softmax /
-geometry) for comparing a 16-bit kernel path against its own precision class.
+geometry) for comparing a 16-bit kernel path against its own precision class.  Pinned by
+tests/test_oracle_emulate.py: every cast the branch performs is recorded and a float64
+restatement with explicit casts is walked along that record (same rounding points in the same
+places, same arithmetic between them to fp32-accumulate precision); an oracle that forgets
+any single rounding fails the walk.  The value-residual / SimBaV2 options' emulate branches
+are outside that walk: parity unpinned for those two options on 16-bit streams (their fp32
+path is pinned by the notepolicy_vres_v2 vector).
 """
 from __future__ import annotations
 
