@@ -30,9 +30,7 @@ geometry) for comparing a 16-bit kernel path against its own precision class.  P
 tests/test_oracle_emulate.py: every cast the branch performs is recorded and a float64
 restatement with explicit casts is walked along that record (same rounding points in the same
 places, same arithmetic between them to fp32-accumulate precision); an oracle that forgets
-any single rounding fails the walk.  The value-residual / SimBaV2 options' emulate branches
-are outside that walk: parity unpinned for those two options on 16-bit streams (their fp32
-path is pinned by the notepolicy_vres_v2 vector).
+any single rounding fails the walk; the value-residual and SimBaV2 options are walked too.
 """
 from __future__ import annotations
 

@@ -300,12 +300,16 @@ def _blocks_walk(P, arch, x, bias, r, round_residual=True):
         w = r(w / w.sum(-1, keepdims=True), what + " probabilities")
         return np.einsum("bhqk,bkhd->bqhd", w, v.reshape(B, T, H, dh)).reshape(B, Tq, d)
 
-    x_res = None
+    x_res, v0, vres = None, None, bool(arch.get("value_residual", False))
     for i in range(L):
         p = f"blocks.{i}."
         h = r(ln(p + "ln_attn", x), p + "ln_attn")
         k = r(lin(p + "k_proj", h), p + "k")
         v = r(lin(p + "v_proj", h), p + "v")
+        if vres and i == 0:
+            v0 = v                              # block 0 hands its values to every later block
+        elif vres:
+            v = r(v * P[p + "vres_a"] + v0 * P[p + "vres_b"], p + "value-residual mix")
         if i == L - 1:
             x_res = x
             x, h = x[:, :nr.N_LEAD], h[:, :nr.N_LEAD]
@@ -354,10 +358,23 @@ def _np_walk(sd, arch, obs, tape):
     lead, x_res, attend = _blocks_walk(P, arch, x, bias, r)
     if arch.get("final_ln", False):
         lead = r(ln("final_ln", lead), "final_ln")
-    t = r(lin("trunk_proj", lead.reshape(B, -1)), "trunk_proj")
-    u = r(ln("trunk_ln1", t), "trunk_ln1")
-    dlt = lin("trunk_fc2", r(np.maximum(lin("trunk_fc1", u), 0.0), "trunk hidden"))
-    hfeat = r(ln("trunk_ln2", r(t + dlt, "trunk sum")), "trunk_ln2")
+    if arch.get("trunk_arch", "simba") == "simbav2":
+        # SimBaV2 (python/policy.py:1140-1155): GEMM results and GEMM inputs are stored 16-bit; scalers, ReLU, the
+        # row normalisations and the LERP are fp32 in between; one rounding of the feature row at the end
+        l2n = lambda v: v / np.maximum(np.sqrt((v * v).sum(-1, keepdims=True)), 1e-6)
+        D = arch["trunk_dim"]
+        xx = l2n(r(lin("trunk_in", lead.reshape(B, -1)), "trunk_in") * P["trunk_s_in"])
+        xr = r(xx, "trunk_w1 input")
+        uu = np.maximum(r(lin("trunk_w1", xr), "trunk_w1") * P["trunk_s_1"], 0.0)
+        ur = r(uu, "trunk_w2 input")
+        yy = l2n(r(lin("trunk_w2", ur), "trunk_w2"))
+        xx = l2n(xx + P["trunk_alpha"] * (0.5 * math.sqrt(D)) * (yy - xx))
+        hfeat = r(xx * math.sqrt(D), "trunk feature")
+    else:
+        t = r(lin("trunk_proj", lead.reshape(B, -1)), "trunk_proj")
+        u = r(ln("trunk_ln1", t), "trunk_ln1")
+        dlt = lin("trunk_fc2", r(np.maximum(lin("trunk_fc1", u), 0.0), "trunk hidden"))
+        hfeat = r(ln("trunk_ln2", r(t + dlt, "trunk sum")), "trunk_ln2")
     wh = r(np.concatenate([P[f"heads.{j}.weight"] for j in range(nr.N_HEADS_OUT)]), "packed head weights")
     flat = hfeat @ wh.T + np.concatenate([P[f"heads.{j}.bias"] for j in range(nr.N_HEADS_OUT)])
     hv = r(ln("critic_ln", x_res), "critic_ln")
@@ -393,11 +410,10 @@ def _np_taped_oracle(sd, arch, obs, dtype, skip_call=None):
 def _fixture(name):
     import os
     arch, sd, obs, _, _ = nr.load_fixture(os.path.join(os.path.dirname(__file__), "golden", name + ".npz"))
-    assert arch.get("trunk_arch", "simba") == "simba" and not arch.get("value_residual", False)
     return arch, sd, obs[:3]
 
 
-@pytest.mark.parametrize("fixture", ["notepolicy_geo", "notepolicy_ragged_ln", "notepolicy_flux"])
+@pytest.mark.parametrize("fixture", ["notepolicy_geo", "notepolicy_ragged_ln", "notepolicy_flux", "notepolicy_vres_v2"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_notepolicy_emulate_walks_the_float64_restatement(dtype, fixture):
     arch, sd, obs = _fixture(fixture)
