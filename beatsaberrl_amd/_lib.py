@@ -97,6 +97,10 @@ def load():
         raise RuntimeError(
             f"{LIB_PATH} not found: the HIP kernels are not built. Run `python -m beatsaberrl_amd.build` "
             "(there is no CPU or torch fallback for the kernel path).")
+    # torch first: it ships its own HIP runtime, and the library must bind to THAT copy (the one that owns torch's
+    # device memory and streams).  Loaded the other way round, the system runtime comes in with the library, torch
+    # brings a second one, and launches fail with "no ROCm-capable device is detected".
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)        # AttributeError here = a symbol the header declares is missing

@@ -66,7 +66,7 @@ def build_policy(args, device):
         ckpt = torch.load(args.ckpt, map_location="cpu", weights_only=True)
         policy = load_policy(ckpt)
         print(f"weights: {args.ckpt}")
-    except (FileNotFoundError, SystemExit):
+    except FileNotFoundError:              # an incompatible checkpoint is an error, not a reason to time random weights
         torch.manual_seed(0)
         if args.legacy_arch:
             policy = NotePolicy(n_gears=5)
@@ -91,12 +91,18 @@ def main(argv=None):
     p.add_argument("--fp16-accum", default=None, choices=_fl.ACCUM_MODES, help="recorded only: accumulate is fp32")
     p.add_argument("--fused-ffn", nargs="+", default=None, choices=_fl.FFN_MODES)
     p.add_argument("--legacy-arch", action="store_true", help="ctor defaults (128 / 256 / 3 blocks) instead of the recipe")
+    p.add_argument("--fused-forward", default="auto", choices=("auto", "off"),
+                   help="auto: the block stack as one persistent kernel and the pooled critic where the shape has them "
+                        "(16-bit stream); off: the per-op launch train with the reference's critic op order, whose "
+                        "outputs are the update forward's bits")
     args = p.parse_args(argv)
     device = torch.device("cuda")
     policy = build_policy(args, device)
+    policy.fused_blocks = args.fused_forward
+    policy.critic_pool = args.fused_forward == "auto"
     if args.fp16_accum is not None:
         policy.fp16_accum = policy.arch["fp16_accum"] = args.fp16_accum
-    print(f"gpu: {torch.cuda.get_device_name(0)}  torch {torch.__version__}")
+    print(f"gpu: {torch.cuda.get_device_name(0)}  torch {torch.__version__}  fused-forward {args.fused_forward}")
     print(f"best of {args.reps} x {args.iters} iters, us/forward\n")
     hdr = f"{'ffn':<6}{'op':<8}{'N':>6}{'eager':>10}{'graphed':>10}{'vs eager':>10}{'env-samples/s':>16}"
     print(hdr)

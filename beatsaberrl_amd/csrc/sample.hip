@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void sample_heads_kernel(SampleArgs a) {
         if (a.action_in) {
             act = a.action_in_u8 ? (int)static_cast<const uint8_t*>(a.action_in)[row]
                                  : (int)static_cast<const int64_t*>(a.action_in)[row];
-            act = act < 0 ? 0 : (act >= K ? K - 1 : act);               // host validates; never index out of the row
+            act = act < 0 ? 0 : (act >= K ? K - 1 : act);               // out-of-range actions are clamped into the row (documented in bsrl.h): never index out of it
         } else {
             const int nvalid = a.head_sizes ? a.head_sizes[h] : K;
             uint32_t r[8];

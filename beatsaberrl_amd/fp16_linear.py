@@ -123,18 +123,25 @@ def _replica_padded(w: torch.Tensor, dtype: torch.dtype, k_pad: int) -> torch.Te
 
 
 def packed_halves(ms, dtype=torch.float16):
-    """(w_cat in `dtype`, b_cat fp32) for an ordered group of same-input Linears."""
+    """(w_cat in `dtype`, b_cat fp32) for an ordered group of same-input Linears.  16-bit copies are refreshed per
+    weights version (bump_weights_version), like every replica.  The fp32 "copy" is a plain concatenation of the
+    masters: the reference's fp32 forward reads the masters themselves (python/policy.py:1371-1376), so it is also
+    rebuilt whenever torch's own in-place counters of the members move (any in-place edit, with or without a bump)."""
     key = ms[0].weight
-    cache = getattr(key, "_bsrl_packed", None)
-    stale = cache is None or cache[1].dtype is not dtype or cache[1].device != key.device or cache[3] != len(ms)
-    if stale:
+    ident = tuple(id(m) for m in ms)                      # the members, not just the first one and the count
+    table = getattr(key, "_bsrl_packed", None)
+    if table is None:
+        table = key._bsrl_packed = {}
+    cache = table.get((ident, dtype))
+    tv = tuple((m.weight._version, m.bias._version) for m in ms) if dtype is torch.float32 else None
+    if cache is None or cache[1].device != key.device:
         cache = [_weights_version, torch.cat([m.weight.detach() for m in ms]).to(dtype).contiguous(),
-                 torch.cat([m.bias.detach() for m in ms]).float().contiguous(), len(ms)]
-        key._bsrl_packed = cache
-    elif cache[0] != _weights_version:
+                 torch.cat([m.bias.detach() for m in ms]).float().contiguous(), tv]
+        table[(ident, dtype)] = cache
+    elif cache[0] != _weights_version or cache[3] != tv:
         cache[1].copy_(torch.cat([m.weight.detach() for m in ms]))
         cache[2].copy_(torch.cat([m.bias.detach() for m in ms]))
-        cache[0] = _weights_version
+        cache[0], cache[3] = _weights_version, tv
     return cache[1], cache[2]
 
 

@@ -57,6 +57,8 @@ def ln_fwd(x, weight, bias, eps=1e-5, want_stats=False):
     d = x.shape[-1]
     if not x.is_contiguous():
         raise RuntimeError("ln_fwd: x must be contiguous")
+    if weight.numel() != d or bias.numel() != d:
+        raise RuntimeError(f"ln_fwd: weight / bias must have {d} elements")
     rows = x.numel() // d
     y = torch.empty_like(x)
     mean = rstd = None
@@ -78,6 +80,8 @@ def ln_fwd_add(a, b, weight, bias, eps=1e-5, b_bias=None, want_stats=False):
     if a.shape != b.shape or a.dtype is not b.dtype or not (a.is_contiguous() and b.is_contiguous()):
         raise RuntimeError("ln_fwd_add: a and b must be contiguous with equal shape and dtype")
     d = a.shape[-1]
+    if weight.numel() != d or bias.numel() != d or (b_bias is not None and b_bias.numel() != d):
+        raise RuntimeError(f"ln_fwd_add: weight / bias / b_bias must have {d} elements")
     rows = a.numel() // d
     x = torch.empty_like(a)
     y = torch.empty_like(a)
@@ -362,6 +366,12 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5)
     Fh = w0.shape[0]
     if not (x.is_contiguous() and h2.is_contiguous() and w0.is_contiguous() and w2.is_contiguous()):
         raise RuntimeError("ffn_fused: contiguous tensors required")
+    if h2.shape != x.shape or not (h2.dtype is x.dtype and w0.dtype is x.dtype and w2.dtype is x.dtype):
+        raise RuntimeError("ffn_fused: h2 must have x's shape, and h2 / w0 / w2 x's dtype")
+    if tuple(w0.shape) != (Fh, d) or tuple(w2.shape) != (d, Fh) or b0.numel() != Fh or b2.numel() != d:
+        raise RuntimeError(f"ffn_fused: expected w0 ({Fh}, {d}), w2 ({d}, {Fh}), b0 ({Fh},), b2 ({d},)")
+    if (ln_w is None) != (ln_b is None) or (ln_w is not None and (ln_w.numel() != d or ln_b.numel() != d)):
+        raise RuntimeError(f"ffn_fused: ln_w and ln_b come together, {d} elements each")
     rows = x.numel() // d
     xo = torch.empty_like(x)
     ho = torch.empty_like(x) if ln_w is not None else None
@@ -432,7 +442,7 @@ def note_frontend(obs, saber_idx, body_idx, dtype, note_geo=False, flux=False, z
 
 
 def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, action=None,
-                 need_entropy=True, want_ent_h=False, want_noise=False, counter=None):
+                 need_entropy=True, want_ent_h=False, want_noise=False, counter=None, validate_action=False):
     """Action epilogue on fp32 logits (B, n_heads, K).  action=None samples (Gumbel-max with the
     caller's Exp(1) draws `exp_noise`, or the kernel's Philox stream keyed by (seed, offset));
     otherwise evaluates the given (B, n_heads) int64 / uint8 actions.  counter: a one-element
@@ -454,6 +464,10 @@ def sample_heads(logits, head_sizes=None, exp_noise=None, seed=0, offset=0, acti
         if action.shape != (B, NH) or action.dtype not in (torch.int64, torch.uint8) or not action.is_contiguous():
             raise TypeError("sample_heads: action must be a contiguous (B, n_heads) int64 or uint8 tensor")
         u8 = int(action.dtype is torch.uint8)
+        if validate_action:             # a host round trip (synchronises): off on the rollout / captured paths
+            lo, hi = int(action.min()), int(action.max())
+            if lo < 0 or hi >= K:
+                raise IndexError(f"sample_heads: action values in [{lo}, {hi}] outside [0, {K}) (the kernel would clamp them)")
     if counter is not None and (counter.dtype is not torch.int64 or counter.numel() != 1 or not counter.is_cuda):
         raise TypeError("sample_heads: counter must be a one-element int64 device tensor")
     dev = logits.device

@@ -393,6 +393,13 @@ class NotePolicy(nn.Module):
         # around it (no (B T, 2d) keys / values); False: the reference's op order
         self.critic_pool = True
         self._critic_pool_cache = None
+        # The reference keeps the grad-free rollout forward and the grad-mode update forward bit-identical
+        # (python/tests/test_fp16_accum.py:146-160): PPO's first-epoch ratio is then exactly 1.  The two fast rollout
+        # routes above (fused block stack: fp32 residual in registers; pooled critic: k / v never rounded) differ from
+        # the update forward, which is the per-op route, by 16-bit rounding (log-prob of a 29-head action to ~1e-2,
+        # value to ~2e-4 at the recipe shape).  True: the rollout takes the per-op route and the reference's critic op
+        # order whatever the two switches say - same bits as the update forward, at the per-op route's speed.
+        self.rollout_matches_update = False
         # sampling-call counter of the in-kernel Philox stream; on the device so that a captured
         # get_action_and_value draws fresh noise on every replay
         self.register_buffer("_sample_ctr", torch.zeros(1, dtype=torch.int64), persistent=False)
@@ -419,7 +426,7 @@ class NotePolicy(nn.Module):
 
     def fused_blocks_ok(self, dt) -> bool:
         """True when the block stack of this architecture has a fused kernel in dtype dt."""
-        if self.fused_blocks == "off" or dt is torch.float32 or self.value_residual:
+        if self.fused_blocks == "off" or self.rollout_matches_update or dt is torch.float32 or self.value_residual:
             return False                    # the value-residual mix has no place in the fused stack
         if self.fused_blocks != "auto":
             raise ValueError(f"fused_blocks must be 'auto' or 'off', got {self.fused_blocks!r}")
@@ -674,7 +681,7 @@ class NotePolicy(nn.Module):
         packed k|v -> 1-query attention pool -> out -> MLP -> HL-Gauss expectation."""
         B, T, d = x_res.shape
         H = self.n_heads
-        if self.critic_pool and ops.critic_pool_supported(T, d, H, x_res.dtype):
+        if self.critic_pool and not self.rollout_matches_update and ops.critic_pool_supported(T, d, H, x_res.dtype):
             # one query per env: the k | v projections commute with the pool, so keys and values are never formed
             wqk, wvo, bvo = self._critic_pool_weights(x_res.dtype)
             q = _lin(self.critic_q, self.critic_ln(x_res[:, 2].contiguous()))          # (B, d), the torso token's query
@@ -716,8 +723,11 @@ class NotePolicy(nn.Module):
             logprob = logsm.gather(-1, action.long().unsqueeze(-1)).squeeze(-1).sum(-1)
             entropy = None
             if need_entropy:
-                self._ent_h = -(logsm.exp() * logsm).sum(-1)
-                entropy = self._ent_h.sum(-1)
+                ent_h = -(logsm.exp() * logsm).sum(-1)
+                # detached (a view, no copy): the stash outlives the backward and must not pin the micro-batch's
+                # autograd graph (reference python/policy.py:1509-1515)
+                self._ent_h = ent_h.detach()
+                entropy = ent_h.sum(-1)
             return action, logprob, entropy, value
         with torch.no_grad():
             return self._act_rollout(obs, action, need_entropy)

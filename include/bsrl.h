@@ -283,7 +283,9 @@ int bsrl_note_frontend_padded(const void* obs, int64_t obs_ld, int obs_dtype,
  * the stream (the part torch's graph-registered generator offset plays in the
  * reference's captured rollout, python/rollout_graph.py:43-78).  noise_out, if
  * not NULL, receives the E used.  Evaluation (action_in != NULL, int64 or uint8 when action_in_u8):
- * no sampling; action_out may be NULL.
+ * no sampling; action_out may be NULL.  A given action outside [0, K) is clamped into the row (the
+ * reference's torch.gather would raise): validate on the host where that matters - no entry point
+ * synchronises, so the kernel cannot report it.
  * Outputs: action_out (B, n_heads) int64; logprob (B); entropy (B) or NULL;
  * ent_h (B, n_heads) or NULL. */
 int bsrl_sample_heads(const float* logits, int64_t B, int64_t n_heads, int64_t K,

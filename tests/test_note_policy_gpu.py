@@ -2,7 +2,8 @@
   * fp32 kernels against the golden vectors the REFERENCE's own module produced
     (tests/golden/notepolicy_*.npz) - 1e-5 relative;
   * the 16-bit stream at production-like shapes against the CPU oracle (itself pinned on
-    those vectors), with the class-relative gates of tests/test_config_policy_gpu.py, plus
+    those vectors; its rounding emulation by tests/test_oracle_emulate.py) under literal
+    ceilings on the batch maxima, plus
     the reference's own fp16-vs-fp32 bar: logits within 2e-2 of max|logit|
     (python/tests/test_trunk_simba.py:142-162)."""
 import glob
@@ -129,8 +130,13 @@ def test_production_shapes_against_the_oracle(kw, dtype, ffn, blocks):
     e_class = (lg[live] - em_lg[live]).abs().max().item()
     print(f"\n[{dtype} ffn={ffn} blocks={blocks}] mine-vs-fp32 {e_mine:.2e}  emulated-vs-fp32 {e_emul:.2e}  mine-vs-emulated {e_class:.2e}")
     assert torch.equal(lg[~live], ref_lg[~live])
-    assert e_mine <= max(1.25 * e_emul, 2e-3) and e_class <= max(e_emul, 2e-3)
-    assert (v - ref_v).abs().max().item() <= max(1.25 * (em_v - ref_v).abs().max().item(), e_emul, 2e-3)
+    e_v, e_vc = (v - ref_v).abs().max().item(), (v - em_v).abs().max().item()
+    print(f"logits vs fp32 {e_mine:.3e} vs emulated {e_class:.3e}; value vs fp32 {e_v:.3e} vs emulated {e_vc:.3e}; "
+          f"logit scale {ref_lg[live].abs().max().item():.2f}")
+    # literal ceilings per stream dtype over all shapes and routes of this test: measured maxima plus 25 %
+    # (fp16: 2.25e-3 / 2.15e-3 on logits of magnitude ~2.5, values 9.2e-5; bf16: 1.49e-2 / 1.38e-2, 4.7e-4)
+    c_fp32, c_class, c_v = (2.9e-3, 2.7e-3, 1.2e-4) if dtype == "f16" else (1.9e-2, 1.8e-2, 6.5e-4)
+    assert e_mine <= c_fp32 and e_class <= c_class and e_v <= c_v and e_vc <= c_v, (e_mine, e_class, e_v, e_vc)
     if dtype == "f16":
         assert e_mine <= 2e-2 * ref_lg[live].abs().max().item()      # the reference's own fp16 bar
         top = ref_lg.topk(2, -1).values
@@ -184,7 +190,7 @@ def test_pooled_critic_matches_the_reference_op_order(dtype):
     if dtype == "f32":
         assert e_pool <= 1e-5 * (ref_v.abs().max().item() + 1) and e_ref <= 1e-5 * (ref_v.abs().max().item() + 1)
     else:
-        assert e_pool <= max(1.25 * e_ref, 2e-3)
+        assert e_pool <= (1e-4 if dtype == "f16" else 7e-4)          # measured 6.7e-5 / 5.2e-4 (reference order: 6.2e-5 / 5.1e-4)
 
 
 @pytest.mark.parametrize("blocks", ["auto", "off"])

@@ -4,12 +4,12 @@ the CPU oracle on the same weights and inputs.
 
   * fp32: every parameter's gradient within 2e-4 of the oracle's (relative to that gradient's largest
     entry), outputs within the forward's 1e-5;
-  * 16-bit stream: per-parameter relative Frobenius error against the fp32 oracle no worse than
-    the rounding-emulating oracle's own (x 2) or 0.15 - the reference's "no worse than the replaced
-    path" idiom (python/tests/test_fused_ffn.py:295-306).  The floor is that wide because a ReLU unit whose
-    pre-activation sits within a rounding of 0 may flip between two 16-bit forwards, and at this batch size
-    ONE flipped unit of the critic MLP (1 of 4608 at B = 48) moves that path's gradients by 5 % (measured; the
-    reference's tests note the same effect, python/tests/test_fused_ffn.py:220-224);
+  * 16-bit stream: per-parameter relative Frobenius error against the fp32 oracle under literal ceilings per
+    parameter group (`_GRAD_CEIL`), plus the gradient's direction (cosine >= 0.99 fp16 / 0.97 bf16 against the
+    oracle's: a flipped sign or a dropped term fails whatever the group's ceiling).  The ceilings are wide for the
+    critic because a ReLU unit whose pre-activation sits within a rounding of 0 may flip between two 16-bit
+    forwards, and at this batch size ONE flipped unit of the critic MLP (1 of 4608 at B = 48) moves that path's
+    gradients by 5 % (measured; the reference's tests note the same effect, python/tests/test_fused_ffn.py:220-224);
   * each Function against torch autograd on the SAME rounded forward (identical masks): 5e-3 (fp16);
   * the update forward is bitwise the per-op rollout forward (the reference's rollout == update contract,
     python/train_batch.py:2364-2372)."""
@@ -119,10 +119,71 @@ def test_gradients_match_the_oracle(kw, dtype):
             continue
         den = want.norm().item() + 1e-12
         e_mine, e_emul = (got - want).norm().item() / den, (emu - want).norm().item() / den
-        worst.append((e_mine / max(e_emul, 1e-9), n, e_mine, e_emul))
-        assert e_mine <= max(2.0 * e_emul, 0.15), (n, e_mine, e_emul)
+        cos = float((got * want).sum() / (got.norm() * want.norm() + 1e-30))
+        grp = _group(n)
+        worst.append((e_mine / _GRAD_CEIL[dtype][grp], n, e_mine, e_emul, cos))
+        assert e_mine <= _GRAD_CEIL[dtype][grp], (n, e_mine, _GRAD_CEIL[dtype][grp], e_emul)
+        # direction: a flipped sign gives -1, a dropped term of comparable size ~0.7
+        assert cos >= (0.99 if dtype == "f16" else 0.97), (n, cos)
     w = max(worst)
-    print(f"\n[{dtype}] worst gradient vs emulated class: {w[1]} mine {w[2]:.2e} emulated {w[3]:.2e}")
+    print(f"\n[{dtype}] gradient closest to its ceiling: {w[1]} error {w[2]:.2e} ({w[0]:.2f} of the ceiling; emulated oracle "
+          f"{w[3]:.2e}), cosine {w[4]:.4f}")
+
+
+# Literal ceilings on the relative Frobenius error of each parameter's gradient against the fp32 oracle's, per stream
+# dtype and parameter group: the maxima measured over the three architectures of this test plus 30 %.  The critic's
+# gradients are 1e-3 .. 1e-5 of the model's largest (a value loss against a unit-variance target) and carry the
+# class's rounding noise at that relative size; vres_a / vres_b are single scalars.
+_GRAD_CEIL = {
+    "f16": {"heads": 2.2e-3, "trunk": 2.7e-2, "encoder": 5.2e-2, "blocks": 3.1e-2, "vres": 9.0e-2, "critic": 1.3e-1, "ln": 1.0e-2},
+    "bf16": {"heads": 1.6e-2, "trunk": 1.05e-1, "encoder": 1.15e-1, "blocks": 1.3e-1, "vres": 2.9e-1, "critic": 1.9e-1, "ln": 4.4e-2},
+}
+
+
+def _group(name):
+    if name.startswith("heads"):
+        return "heads"
+    if name.startswith("trunk"):
+        return "trunk"
+    if name.startswith("critic"):
+        return "critic"
+    if name.startswith(("emb_ln", "final_ln")):
+        return "ln"
+    if name.startswith("blocks"):
+        return "vres" if "vres" in name else "blocks"
+    assert name.split(".")[0] in ("saber_mlp", "torso_mlp", "leg_mlp", "note_mlp"), name
+    return "encoder"
+
+
+def test_rollout_update_gap_on_the_default_routes_is_bounded_and_the_switch_closes_it():
+    """The reference holds rollout == update bitwise (python/tests/test_fp16_accum.py:146-160).  Here the DEFAULT
+    rollout (fused block stack + pooled critic) and the update forward differ by 16-bit rounding; this test bounds the
+    gap at the recipe shape with literal ceilings (measured at B = 4096: log-prob of the 29-head action 8.9e-3, i.e.
+    a first-epoch PPO ratio within 0.9 % of 1; logits 2.5e-3; value 1.5e-4), and shows that
+    `rollout_matches_update = True` restores the reference's contract: identical logits and value bits."""
+    torch.manual_seed(0)
+    m = NotePolicy(embed=192, trunk_dim=384, n_blocks=6, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True).to(DEV)
+    m.fp16 = True
+    assert m.fused_blocks == "auto" and m.critic_pool and not m.rollout_matches_update
+    od = _obs(4096, 0).to(DEV)
+    with torch.no_grad():
+        assert m.fused_blocks_ok(torch.float16)
+        act, logp_r, _, v_r = m.get_action_and_value(od)
+        lg_r, _ = m.forward_stacked(od)
+    _, logp_u, _, v_u = m.get_action_and_value(od, action=act)
+    lg_u, _ = m.forward_stacked(od)
+    logp_u, v_u, lg_u = logp_u.detach(), v_u.detach(), lg_u.detach()
+    g_logp, g_lg, g_v = (logp_r - logp_u).abs().max().item(), (lg_r - lg_u).abs().max().item(), (v_r - v_u).abs().max().item()
+    print(f"\nrollout(default routes) vs update: |dlogp| {g_logp:.3e} (ratio off 1 by {(torch.exp(logp_u - logp_r) - 1).abs().max().item():.3e}), "
+          f"|dlogit| {g_lg:.3e}, |dvalue| {g_v:.3e}")
+    assert 0 < g_logp <= 1.2e-2 and g_lg <= 3.5e-3 and g_v <= 3e-4
+    m.rollout_matches_update = True
+    with torch.no_grad():
+        assert not m.fused_blocks_ok(torch.float16)
+        lg_s, v_s = m.forward_stacked(od)
+        _, logp_s, _, _ = m.get_action_and_value(od, action=act)
+    assert torch.equal(lg_s, lg_u) and torch.equal(v_s, v_u)
+    assert (logp_s - logp_u).abs().max().item() <= 5e-5        # same logits; kernel vs torch log-softmax summation
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
@@ -310,4 +371,4 @@ def test_update_path_with_the_fused_ffn_follows_the_unfused_update():
         den = g0[n].norm().item()
         if g0[n].abs().max().item() < 1e-5 * gmax:
             continue
-        assert (g1[n] - g0[n]).norm().item() <= 0.15 * den, (n, (g1[n] - g0[n]).norm().item() / den)
+        assert (g1[n] - g0[n]).norm().item() <= 6e-2 * den, (n, (g1[n] - g0[n]).norm().item() / den)     # measured maximum 4.4e-2 (critic_q.weight)
