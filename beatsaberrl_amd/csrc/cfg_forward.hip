@@ -84,6 +84,27 @@ template <> __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
 union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
 union Frag4 { s16x4 v; uint32_t w[2]; };
 
+// gfx950's lane-row exchanges, as plain VALU instructions (no LDS round trip, no lgkmcnt wait behind the weight
+// fragment reads).  A wave is four rows of 16 lanes.  v_permlane16_swap_b32 a, b: rows 1 and 3 of a change places
+// with rows 0 and 2 of b; v_permlane32_swap_b32 a, b: rows 2..3 of a with rows 0..1 of b.  Written as asm because
+// the compiler builtin returns the first result twice in this toolchain; the s_nop is the two wait states the
+// instruction needs after a VALU write of either operand (the compiler does not look inside an asm statement).
+__device__ __forceinline__ void row_swap16(float& a, float& b) { asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void row_swap32(float& a, float& b) { asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+// The lane-row butterfly (combine with lane ^ 16, then with lane ^ 32) of TWO values at once: on return every lane
+// holds the combination of its column over the four rows, for both values, associated (r0 . r1) . (r2 . r3) exactly
+// as the two-step shuffle butterfly associates it.  8 VALU ops for the pair.
+template <typename OP> __device__ __forceinline__ void rows_reduce2(float& s, float& q, OP op) {
+    row_swap16(s, q);                   // s = {s0, q0, s2, q2}, q = {s1, q1, s3, q3} (by row)
+    float z = op(s, q), w = z;          // {s0.s1, q0.q1, s2.s3, q2.q3}
+    row_swap32(z, w);                   // z = {z0, z1, z0, z1}, w = {z2, z3, z2, z3}
+    float t = op(z, w), u = t;          // {S, Q, S, Q}
+    row_swap16(t, u);                   // t = {S, S, S, S}, u = {Q, Q, Q, Q}
+    s = t; q = u;
+}
+struct OpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were issued 3
@@ -138,6 +159,7 @@ constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 
 template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
+    static_assert(RT == 1 || RT == 2, "the softmax butterflies pair the row tiles");
     __shared__ uint4 lds[2][STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
@@ -206,8 +228,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) { s += x[rt][nt][i]; q = fmaf(x[rt][nt][i], x[rt][nt][i], q); }
-                    s += __shfl_xor(s, 16, WAVE); q += __shfl_xor(q, 16, WAVE);
-                    s += __shfl_xor(s, 32, WAVE); q += __shfl_xor(q, 32, WAVE);
+                    rows_reduce2(s, q, OpAdd());
                     mean = s * (1.0f / D);
                     rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q * (1.0f / D)), 0.f) + 1e-5f);
                 }
@@ -277,24 +298,33 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 // scores^T = K Q^T (lane: query r16, keys 4g..4g+3), softmax over keys, O = P V (+ b_v)
                 const float4 bv0 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 4 * g);
                 const float4 bv1 = *reinterpret_cast<const float4*>(lv + LV_BV + 32 * hd + 16 + 4 * g);
+                // both row tiles side by side: their max / sum butterflies share the row exchanges
+                float sv[RT][4], mx[2], sm[2];
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    f32x4 sc = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                    const f32x4 sc = DT::mfma32(kf[rt].v, qf[rt].v, (f32x4){0.f, 0.f, 0.f, 0.f});
                     // raw scores + additive key mask (0 / -inf); softmax of (scale * s) = exp2((s - max) * scale*log2e)
-                    float sv[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) sv[i] = sc[i] + kmask[rt][i];
-                    float m = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-                    m = fmaxf(m, __shfl_xor(m, 16, WAVE)); m = fmaxf(m, __shfl_xor(m, 32, WAVE));
-                    const float ms = -m * scale_l2e;
-                    float sum = 0.f;
+                    for (int i = 0; i < 4; ++i) sv[rt][i] = sc[i] + kmask[rt][i];
+                    mx[rt] = fmaxf(fmaxf(sv[rt][0], sv[rt][1]), fmaxf(sv[rt][2], sv[rt][3]));
+                }
+                if (RT == 1) mx[1] = mx[0];
+                rows_reduce2(mx[0], mx[1], OpMax());
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) { sv[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_l2e, ms)); sum += sv[i]; }
-                    sum += __shfl_xor(sum, 16, WAVE); sum += __shfl_xor(sum, 32, WAVE);
-                    const float inv = __builtin_amdgcn_rcpf(sum);
+                for (int rt = 0; rt < RT; ++rt) {
+                    const float ms = -mx[rt] * scale_l2e;
+                    sm[rt] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[rt][i] = __builtin_amdgcn_exp2f(fmaf(sv[rt][i], scale_l2e, ms)); sm[rt] += sv[rt][i]; }
+                }
+                if (RT == 1) sm[1] = sm[0];
+                rows_reduce2(sm[0], sm[1], OpAdd());
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    const float inv = __builtin_amdgcn_rcpf(sm[rt]);
                     Frag4 pf;
-                    pf.w[0] = pack2<DT>(sv[0] * inv, sv[1] * inv);
-                    pf.w[1] = pack2<DT>(sv[2] * inv, sv[3] * inv);
+                    pf.w[0] = pack2<DT>(sv[rt][0] * inv, sv[rt][1] * inv);
+                    pf.w[1] = pack2<DT>(sv[rt][2] * inv, sv[rt][3] * inv);
                     const f32x4 o0 = DT::mfma16(vt[rt][0].v, pf.v, (f32x4){bv0.x, bv0.y, bv0.z, bv0.w});
                     const f32x4 o1 = DT::mfma16(vt[rt][1].v, pf.v, (f32x4){bv1.x, bv1.y, bv1.z, bv1.w});
                     of[rt][hd].w[0] = pack2<DT>(o0[0], o0[1]); of[rt][hd].w[1] = pack2<DT>(o0[2], o0[3]);
@@ -344,48 +374,45 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 dst.w[ntl * 2 + 1] = pack2<DT>(apply_act16<ACT>(v[2]), apply_act16<ACT>(v[3]));
             };
             if (RT == 1) {
-                // single row tile (TAIL launch): plain chunk loop, no split
-                // stage indices count from the TAIL launch's first stage: 4 output-projection stages precede,
-                // chunk ch's stages are W1(ch+1) = 5 + 2 ch and W2(ch) = 6 + 2 ch (the last chunk: W2 = 3 + 2 nch);
-                // the hidden width is a multiple of 64 here, so two chunks advance the index by 4
-                {
-                    ADV(4);
-                    LOAD_STAGE(0, w1);
-                    up_init(0, accA);
+                // Single row tile (TAIL launch): plain chunk loop, no split.  Stage indices count from the TAIL launch's
+                // first stage: 0..3 the output projection, 4 = W1(0), then W1(ch+1) = 5 + 2 ch and W2(ch) = 6 + 2 ch, the
+                // last W2 = 3 + 2 nch.  The hidden width is a multiple of 64 (nch even), and a loop trip advances two
+                // chunks = four stages, so every stage keeps its place in the rotation of the four prefetch register sets.
+                // The loop body is branch-free on purpose: with the last chunk's stage under a condition inside it, the
+                // compiler could no longer count the loads in flight at the loop head and drained the whole prefetch queue
+                // (s_waitcnt vmcnt(0)) before every stage - one L2 round trip per stage, 32 times per tile.
+                auto up = [&](int ch, int slot) __attribute__((always_inline)) {
+                    s16x8 w1[STAGE_FRAGS];
+#pragma unroll
+                    for (int f = 0; f < STAGE_FRAGS; ++f) w1[f] = slot ? WFRAG(1, f) : WFRAG(0, f);
+                    up_init(ch, accA);
 #pragma unroll
                     for (int c = 0; c < KC; ++c)
 #pragma unroll
                         for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
+                };
+                auto down = [&](int slot) __attribute__((always_inline)) {
+                    s16x8 w2[STAGE_FRAGS];
+#pragma unroll
+                    for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = slot ? WFRAG(1, f) : WFRAG(0, f);
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
+                };
+                auto activate = [&]() __attribute__((always_inline)) { act4(accA[0][0], hidA[0], 0); act4(accA[1][0], hidA[0], 1); };
+                ADV(4); up(0, 0);
+                for (int ch2 = 0; ch2 < nch - 2; ch2 += 2) {
+                    activate();                              // chunk ch2
+                    ADV(5); up(ch2 + 1, 1);
+                    ADV(6); down(0);
+                    activate();                              // chunk ch2 + 1
+                    ADV(7); up(ch2 + 2, 1);
+                    ADV(8); down(0);
                 }
-                for (int ch2 = 0; ch2 < nch; ch2 += 2) {
-#pragma unroll
-                    for (int o = 0; o < 2; ++o) {
-                        const int ch = ch2 + o;
-                        act4(accA[0][0], hidA[0], 0); act4(accA[1][0], hidA[0], 1);
-                        if (ch + 1 < nch) {
-                            ADV(5 + 2 * o);
-                            LOAD_STAGE(1, w1);
-                            up_init(ch + 1, accA);
-#pragma unroll
-                            for (int c = 0; c < KC; ++c)
-#pragma unroll
-                                for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
-                            ADV(6 + 2 * o);
-                        } else {
-                            ADV(3);             // o == 1: the last chunk's down-projection stage, index 3 + 2 nch
-                        }
-                        s16x8 w2[STAGE_FRAGS];
-                        if (ch + 1 < nch) {
-#pragma unroll
-                            for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(0, f);
-                        } else {
-#pragma unroll
-                            for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = WFRAG(1, f);
-                        }
-#pragma unroll
-                        for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
-                    }
-                }
+                activate();                                  // chunk nch - 2
+                ADV(5); up(nch - 1, 1);
+                ADV(6); down(0);
+                activate();                                  // chunk nch - 1
+                ADV(7); down(1);                             // stage 3 + 2 nch
             } else {
                 {   // prologue: up-projection of chunk 0, activation of its lower row tiles
                     ADVANCE(0);
