@@ -10,6 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
 ABI_VERSION = 10
 CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
+CFG_NO_LATENCY = 2              # bsrl_cfg_desc.flags: small batches take the throughput forms too
 CFG_STATIC_MAX_ENVS = 16384     # BSRL_CFG_STATIC_MAX_ENVS: batch limit of bsrl_cfg_forward_static
 
 F32, F16, BF16 = 0, 1, 2

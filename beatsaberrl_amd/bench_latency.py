@@ -1,6 +1,7 @@
 """Small-batch latency of the benchmark-config policy forward (config[4]): p50 microseconds per
-forward at B in {1, 8, 64}, the whole forward as ONE persistent kernel against the per-op
-(multi-kernel) route, eager launches and a captured HIP graph.
+forward at B in {1, 8, 64}, the whole forward as ONE persistent kernel (in its latency form: one env
+per wave, weights through a deep direct-to-LDS ring; and in the throughput form) against the two-launch
+pruned form and the per-op (multi-kernel) route, eager launches and a captured HIP graph.
 
     python -m beatsaberrl_amd.bench_latency [--batches 1 8 64] [--iters 300]
 
@@ -55,18 +56,20 @@ def main(argv=None):
     for B in args.batches:
         obs = torch.randn(B, m.obs_dim, device=dev)
         variants = {
+            "persistent kernel, latency form (1 launch)": dict(route="fused", prune=False, latency=True),
             "persistent kernel (1 launch)": dict(route="fused", prune=False),
             "fused, final block pruned (2 launches)": dict(route="fused", prune=True),
             "per-op route (multi-kernel)": dict(route="ops", prune=False),
         }
         for name, v in variants.items():
             m.prune_final = v["prune"]
+            m.latency_form = v.get("latency", False)      # False: the throughput forms (small batches default to the latency form)
             fn = lambda: m.forward_stacked(obs, None, route=v["route"])
             eager = p50_us(fn, args.iters)
             replay = graphed(fn)
             gr = p50_us(replay, args.iters)
             rows.append({"B": B, "variant": name, "p50_us_eager": round(eager, 1), "p50_us_graph": round(gr, 1)})
-            print(f"B={B:<3d} {name:<40s} eager {eager:8.1f} us   graph {gr:8.1f} us", flush=True)
+            print(f"B={B:<3d} {name:<44s} eager {eager:8.1f} us   graph {gr:8.1f} us", flush=True)
     print(json.dumps({"metric": "p50 forward latency, config[4] model fp16", "rows": rows}))
     return rows
 

@@ -75,6 +75,10 @@ class ConfigPolicy(nn.Module):
         self._replica = None          # (version, dtype, device) -> 16-bit weight copies
         self._packed = None           # (version, dtype, device) -> fused-kernel weight image
         self._workspace = None        # scratch of the pruned fused route (grown on demand, then reused)
+        # fused route, small batches (B <= 4 x CUs): one persistent launch, one env per wave, the weight image streamed
+        # straight into a deep LDS ring - the lowest latency per forward (B = 1: 33 us against 52); same output bits as
+        # the throughput forms, so it is on by default.  False: the throughput forms at every batch size
+        self.latency_form = True
         # final-block query pruning on the fused route (the reference's n_queries path,
         # python/policy.py:533-539): exact; False = one persistent kernel computing every token
         self.prune_final = True
@@ -124,7 +128,7 @@ class ConfigPolicy(nn.Module):
         return _lib.CfgDesc(self.n_layers, self.d, self.n_heads, self.ffn_dim, self.T, self.n_gears,
                             _lib.ACT_GELU if self.act == "gelu" else _lib.ACT_RELU,
                             int(self.final_ln is not None), self.prop_dim, self.obj_dim, ops.dt_code(dt),
-                            0 if self.pack_short else _lib.CFG_NO_PACK)
+                            (0 if self.pack_short else _lib.CFG_NO_PACK) | (0 if self.latency_form else _lib.CFG_NO_LATENCY))
 
     def fused_supported(self, dt=None) -> bool:
         dt = dt or _DTYPES[self.dtype]

@@ -63,6 +63,7 @@ struct FwdArgs {
                                   // before it), written by cfg_pair_kernel
     const int32_t* n_packed;      // PACK: number of tiles in `pairs`
     int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
+    int ring_epw;     // RING: envs per workgroup (1..4): one per wave, the other waves only feed the weight ring
 };
 
 // ---- helpers -------------------------------------------------------------------
@@ -105,6 +106,20 @@ template <typename OP> __device__ __forceinline__ void rows_reduce2(float& s, fl
 struct OpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
+// RING variant of the weight pipeline (the latency form): stages go global -> LDS directly (global_load_lds_dwordx4:
+// one wave instruction lands one 1 KB fragment, lane l's 16 bytes at slot l), RING_DEPTH stages ahead of the one being
+// consumed, into a ring of RING_DEPTH + 1 stage slots; no register staging, so the depth is bounded by LDS, not VGPRs.
+// A lone workgroup walking ~100 stages is bound by the L2 round trip divided by the stages in flight: 3 in the
+// register-staged pipeline, 13 here.
+constexpr int RING_DEPTH = 13, RING_SLOTS = RING_DEPTH + 1;
+// m0 (the LDS base of the transfer) is written without telling the compiler, which rejects reserved registers in a
+// clobber list: nothing else in these kernels uses it (no dynamically indexed register arrays, no instruction that
+// reads m0).  No "memory" clobber: what orders the asynchronous LDS writes against the fragment reads is the explicit
+// vmcnt wait + barrier of ring_advance.
+__device__ __forceinline__ void ring_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr));
+}
+
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Weight-stage pipeline: stage s lives in LDS slot s & 1; its global loads were issued 3
@@ -121,7 +136,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
         RB = src_[256]; \
         pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1; \
     } while (0)
-#define ADVANCE(par) do { if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
+// (RING: the advance happens inside the fragment fetch, one stage ahead - see ring_take)
+#define ADVANCE(par) do { if (RING) { } else if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
 // TAIL launch: a workgroup streams its 44 stages for ONE tile with little arithmetic per stage, so the
 // step time is the L2 latency of the weight stream divided by the stages in flight.  Four register
 // sets (q0..q3) keep four stages in flight instead of two: ADVANCE4(Q), Q = index of the stage about to
@@ -133,9 +149,11 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // ADV(sidx): sidx = stage index counted from the start of the block (HEAD / FULL: only its parity
 // matters) or from the start of the TAIL launch's own stage range (its value modulo 4 matters)
 #define ADV(sidx) do { if (MODE == MODE_TAIL) ADVANCE4((sidx) & 3); else ADVANCE((sidx) & 1); } while (0)
-#define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[par][(f) * 64 + lane]))
+#define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[RING ? 0 : (par)][RING ? 0 : (f) * 64 + lane]))
 // all 8 fragments of the current stage -> registers in one burst of LDS reads (one wait instead of 8)
-#define LOAD_STAGE(par, W) s16x8 W[STAGE_FRAGS]; _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = WFRAG(par, f_)
+#define LOAD_STAGE(par, W) s16x8 W[STAGE_FRAGS]; if (RING) ring_take(W); else _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = WFRAG(par, f_)
+// the same with the slot chosen at run time among the two (a wave-uniform value)
+#define LOAD_STAGE_SLOT(slot, W) s16x8 W[STAGE_FRAGS]; if (RING) ring_take(W); else _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = (slot) ? WFRAG(1, f_) : WFRAG(0, f_)
 
 // MODE_FULL: the whole forward, one launch, every token of the last block computed.
 // MODE_HEAD + MODE_TAIL: final-block query pruning (the reference's n_queries path,
@@ -156,26 +174,85 @@ constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 
 // LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
 // multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
 // and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
-template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
-__global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false>
+__global__ __launch_bounds__(256, (RT <= 2 && !RING) ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
+    static_assert(!RING || MODE == MODE_FULL, "the ring pipeline is the one-launch latency form");
     static_assert(RT == 1 || RT == 2, "the softmax butterflies pair the row tiles");
-    __shared__ uint4 lds[2][STAGE_U4];
+    __shared__ uint4 lds[RING ? 1 : 2][RING ? 64 : STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
+    // RING: the stage ring sits behind the vectors (1 KB aligned) in the dynamic region
+    const int ring_off_u4 = (vec_floats(a.n_layers, a.F) / 4 + 63) & ~63;
+    const uint4* ring = reinterpret_cast<const uint4*>(vlds4) + ring_off_u4;
+    int ring_cur = RING_SLOTS - 1;                    // slot of the stage last consumed (the first advance wraps to 0)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
     constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? TAIL_ENVS : 1;     // envs per 16-row MFMA tile
     constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
     const int64_t n_units = PACK ? (int64_t)*a.n_packed : a.B;           // 16-row tiles (PACK) or envs to cover
-    const int64_t ntiles = (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
+    const int64_t ntiles = RING ? (a.B + a.ring_epw - 1) / a.ring_epw : (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
     const uint4* img = a.frags;
+    const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
+    const int uwave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint4 pr0a, pr0b, pr1a, pr1b;
     uint4 q0a, q0b, q1a, q1b, q2a, q2b, q3a, q3b;       // TAIL launch only
     int pnext;
-    {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
+    // RING: this wave's two fragments of stage `stage` -> ring slot `slot` (every wave loads, working or not: leaving the
+    // loads to the waves without an env - 3 + 3 + 2 fragments - measured slower, 36 against 33 us per forward)
+    auto ring_issue = [&](int stage, int slot) __attribute__((always_inline)) {
+        const char* sb = reinterpret_cast<const char*>(img) + (int64_t)stage * (STAGE_U4 * 16) + uwave * 2048;
+        const uint32_t dst = ring_base + slot * (STAGE_U4 * 16) + uwave * 2048;
+        ring_load(lane * 16, sb, dst);
+        ring_load(lane * 16, sb + 1024, dst + 1024);
+    };
+    // RING: called when the next stage is about to be consumed; on return it is readable in slot ring_cur
+    auto ring_advance = [&]() __attribute__((always_inline)) {
+        ring_cur = ring_cur + 1 == RING_SLOTS ? 0 : ring_cur + 1;
+        // this wave's loads of that stage have landed once at most the RING_DEPTH - 1 younger stages' are outstanding
+        // (loads retire in order; any other load or store in flight only makes the wait stricter) ...
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (RING_DEPTH - 1)) : "memory");
+        lds_barrier();                                // ... and every wave's have; every wave is done reading the stage before
+        ring_issue(pnext, ring_cur == 0 ? RING_SLOTS - 1 : ring_cur - 1);      // its slot takes the stage RING_DEPTH ahead
+        pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
+    };
+    // RING: the working waves keep the NEXT stage's eight fragments in registers (wnext), fetched from LDS while the
+    // current stage is being computed: a lone working wave would otherwise sit out one LDS round trip per stage
+    // (~100 stages per forward) with nothing else to run.  ring_take hands out the fragments of the stage about to be
+    // computed, advances the ring and requests the stage after it.  The LDS reads are asm so that they are issued HERE
+    // (the compiler would sink plain loads to their use); the lgkmcnt wait that makes them usable carries wnext as an
+    // operand so that no use of it can be scheduled above the wait.
+    s16x8 wnext[RING ? STAGE_FRAGS : 1];
+    auto ring_fetch = [&]() __attribute__((always_inline)) {
+        const uint32_t addr = ring_base + ring_cur * (STAGE_U4 * 16) + lane * 16;
+#pragma unroll
+        for (int f = 0; f < STAGE_FRAGS; ++f)
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wnext[RING ? f : 0]) : "v"(addr), "n"(f * 1024));
+    };
+    auto ring_take = [&](s16x8 (&W)[STAGE_FRAGS]) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wnext[0]), "+v"(wnext[RING ? 1 : 0]), "+v"(wnext[RING ? 2 : 0]), "+v"(wnext[RING ? 3 : 0]),
+                       "+v"(wnext[RING ? 4 : 0]), "+v"(wnext[RING ? 5 : 0]), "+v"(wnext[RING ? 6 : 0]), "+v"(wnext[RING ? 7 : 0])
+                     :: "memory");
+#pragma unroll
+        for (int f = 0; f < STAGE_FRAGS; ++f) W[f] = wnext[RING ? f : 0];
+        ring_advance();
+        ring_fetch();
+    };
+    if (RING) {
+        // prologue: RING_DEPTH stages in flight (the weight image holds at least that many), then the vectors
+        int st = a.s_begin;
+#pragma unroll
+        for (int i = 0; i < RING_DEPTH; ++i) { ring_issue(st, i); st = st + 1 == a.s_end ? a.s_begin : st + 1; }
+        pnext = st;
+        const int nv4 = vec_floats(a.n_layers, a.F) / 4;
+        for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        lds_barrier();
+        ring_advance();             // the first stage is readable ...
+        ring_fetch();               // ... and on its way to registers (every wave: the waves without an env never wait for it)
+    } else {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
         const int s0 = a.s_begin;
         const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
         if (MODE == MODE_TAIL) {
@@ -198,7 +275,14 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
     }
 
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
+        const int64_t env0 = RING ? tile * a.ring_epw + uwave : tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
+        if (RING && (uwave >= a.ring_epw || env0 >= a.B)) {
+            // a wave without an env: it keeps its share of the weight ring moving (loads, waits, barriers - exactly one
+            // advance per stage, like the working waves) and reads no fragment, so the workgroup's LDS reads are those
+            // of its working waves only
+            for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
+            continue;
+        }
         // every lambda below is force-inlined: one left out of line would take the residual registers by reference,
         // i.e. through scratch memory (seen with the bf16 instantiations, whose pack helper is larger)
         float kmask[RT][4];     // additive key mask for keys 4g..4g+3 of each env: 0 (attendable) or -inf
@@ -382,9 +466,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                 // compiler could no longer count the loads in flight at the loop head and drained the whole prefetch queue
                 // (s_waitcnt vmcnt(0)) before every stage - one L2 round trip per stage, 32 times per tile.
                 auto up = [&](int ch, int slot) __attribute__((always_inline)) {
-                    s16x8 w1[STAGE_FRAGS];
-#pragma unroll
-                    for (int f = 0; f < STAGE_FRAGS; ++f) w1[f] = slot ? WFRAG(1, f) : WFRAG(0, f);
+                    LOAD_STAGE_SLOT(slot, w1);
                     up_init(ch, accA);
 #pragma unroll
                     for (int c = 0; c < KC; ++c)
@@ -392,9 +474,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         for (int ntl = 0; ntl < 2; ++ntl) accA[ntl][0] = DT::mfma32(w1[ntl * KC + c], hf[0][c].v, accA[ntl][0]);
                 };
                 auto down = [&](int slot) __attribute__((always_inline)) {
-                    s16x8 w2[STAGE_FRAGS];
-#pragma unroll
-                    for (int f = 0; f < STAGE_FRAGS; ++f) w2[f] = slot ? WFRAG(1, f) : WFRAG(0, f);
+                    LOAD_STAGE_SLOT(slot, w2);
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) x[0][nt] = DT::mfma32(w2[nt], hidA[0].v, x[0][nt]);
                 };
@@ -657,6 +737,11 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
                         for (int w = 0; w < 4; ++w) e[rt][c].w[w] = pack2<DT>(ev[c][2 * w], ev[c][2 * w + 1]);
                 }
             }
+            // RING: the tile's own loads (obs, key counts) are waited for HERE, with the wait the compiler can see
+            // (vmcnt(0); expcnt / lgkmcnt left at their maxima).  It does not know of the ring's loads, so wherever it
+            // later met a value of its own still in flight - or reused such a register - it would wait for "all
+            // outstanding loads", i.e. drain the ring in mid-tile; after this it has nothing pending.
+            if (RING) __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 bp = *reinterpret_cast<const float4*>(vlds + V_BP + 16 * nt + 4 * g);
@@ -742,6 +827,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void cfg_forward_kernel(FwdAr
             heads(yf, env0, TAIL_ENVS, fv);
         }
     }
+    if (RING) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
 }
 
@@ -983,24 +1069,34 @@ __global__ __launch_bounds__(PAIR_THREADS) void cfg_pair_kernel(const int32_t* n
     if (blockIdx.x == 0 && tid == 0) *n_packed = (int32_t)(first_long + (B - tt - tm - th));
 }
 
-template <typename DT, int RT, int ACT, int MODE, bool PACK = false>
+constexpr size_t LDS_PER_WG = 160 * 1024;
+size_t ring_dyn_bytes(int n_layers, int F) {
+    return (size_t)((vec_floats(n_layers, F) / 4 + 63) & ~63) * 16 + (size_t)RING_SLOTS * STAGE_U4 * 16;
+}
+
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false>
 int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
-    const size_t dyn = (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
-    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK>;
+    const size_t dyn = RING ? ring_dyn_bytes(a.n_layers, a.F) : (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
+    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK, RING>;
     if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
     }
-    const int64_t per_wg = 4 * RT * (MODE == MODE_TAIL ? TAIL_ENVS : 1);
+    const int64_t per_wg = RING ? a.ring_epw : 4 * RT * (MODE == MODE_TAIL ? TAIL_ENVS : 1);
     const int64_t ntiles = (a.B + per_wg - 1) / per_wg;
-    const int64_t resident = (int64_t)cus * (RT <= 2 ? 2 : 1);
+    const int64_t resident = (int64_t)cus * ((RT <= 2 && !RING) ? 2 : 1);
     hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < resident ? ntiles : resident)), dim3(256), dyn, st, a);
     return BSRL_OK;
 }
 
 template <typename DT, int ACT>
-int launch_all(FwdArgs a, bool pruned, bool pack, int cus, hipStream_t st) {
+int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStream_t st) {
     const int ls = layer_stages(a.F), total = total_stages(a.n_layers, a.F);
+    if (latency) {
+        a.s_begin = 0; a.s_end = total;
+        a.ring_epw = (int)((a.B + cus - 1) / cus);              // 1..4 (B <= 4 CUs): as few working waves per CU as the batch allows
+        return launch_one<DT, 1, ACT, MODE_FULL, false, true>(a, cus, st);
+    }
     if (!pruned) {
         a.s_begin = 0; a.s_end = total;
         return launch_one<DT, 2, ACT, MODE_FULL>(a, cus, st);
@@ -1094,6 +1190,7 @@ int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed
     a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
     a.ws = static_cast<uint32_t*>(rows);
+    a.ring_epw = 4;
     // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
     const bool pruned = rows && d->ffn % 64 == 0;
     // short envs share tiles when the caller gives key counts, there is room for the tile table and the descriptor
@@ -1109,11 +1206,17 @@ int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    // the latency form (one launch, one env per wave, deep direct-to-LDS weight ring) for small batches, unless the
+    // descriptor switches it off or vectors + ring exceed one workgroup's LDS; same output bits as the other forms
+    // (and the batch is one pass of one workgroup per CU: past that the persistent loop would drain the ring once per
+    // tile and the throughput forms win anyway)
+    const bool latency = !(d->flags & BSRL_CFG_NO_LATENCY) && ring_dyn_bytes(d->n_layers, d->ffn) + 2048 <= LDS_PER_WG &&
+                         total_stages(d->n_layers, d->ffn) >= RING_DEPTH && B <= 4 * (int64_t)cus;
     int rc;
     if (d->dtype == BSRL_F16)
-        rc = d->act == BSRL_ACT_GELU ? launch_all<F16, BSRL_ACT_GELU>(a, pruned, pack, cus, st) : launch_all<F16, BSRL_ACT_RELU>(a, pruned, pack, cus, st);
+        rc = d->act == BSRL_ACT_GELU ? launch_all<F16, BSRL_ACT_GELU>(a, pruned, pack, latency, cus, st) : launch_all<F16, BSRL_ACT_RELU>(a, pruned, pack, latency, cus, st);
     else
-        rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, pack, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, pack, cus, st);
+        rc = d->act == BSRL_ACT_GELU ? launch_all<BF16, BSRL_ACT_GELU>(a, pruned, pack, latency, cus, st) : launch_all<BF16, BSRL_ACT_RELU>(a, pruned, pack, latency, cus, st);
     if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH(who);
     return BSRL_OK;

@@ -162,10 +162,23 @@ int bsrl_cfg_embed(const void* obs, int64_t obs_ld, int obs_dtype,
  * step, its address must not move while a captured graph replays. */
 typedef struct {
     int32_t n_layers, d, n_heads, ffn, T, n_gears, act, final_ln;
-    int32_t prop_dim, obj_dim, dtype, flags;      /* flags: 0, or BSRL_CFG_NO_PACK */
+    int32_t prop_dim, obj_dim, dtype, flags;      /* flags: 0, or BSRL_CFG_NO_PACK | BSRL_CFG_NO_LATENCY */
 } bsrl_cfg_desc;
 /* bsrl_cfg_forward: keep every env in a tile of its own (see below). */
 #define BSRL_CFG_NO_PACK 1
+/* bsrl_cfg_forward: never take the latency form.  By default a batch of at
+ * most 4 envs per CU (B <= 1024 on an MI355X) runs as ONE persistent launch
+ * whatever the workspace: one env per wave (1..4 working waves per workgroup,
+ * as few as the batch allows), the weight image streamed straight into a
+ * 14-slot LDS ring 13 stages ahead, the next stage's fragments fetched into
+ * registers while the current one is computed.  At such sizes a forward is one
+ * workgroup's walk through the ~100 stages of the image and its time is what a
+ * lone CU takes to pull 0.9 MB and to run the dependent chain of each stage
+ * (B = 1: 33 us against 52 us for the throughput forms).  The output bits are
+ * those of the other forms (tested), so an env's result does not change with
+ * the batch it is in.  Shapes whose vectors + ring exceed a workgroup's LDS
+ * (n_layers * (9 d + ffn) floats + 112 KB > 158 KB) always take the other forms. */
+#define BSRL_CFG_NO_LATENCY 2
 
 /* fp32 master parameter pointers of one transformer block, in the reference's
  * registration order (python/policy.py:492-522); device memory. */

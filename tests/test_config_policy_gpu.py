@@ -156,12 +156,14 @@ def test_weights_version_refreshes_replicas(route):
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("B", [1, 8, 64, 1000, 4096])
 def test_fused_route_config1(dtype, B, prune):
-    """prune=False: one persistent kernel, every token of the last block; prune=True: the
-    two-launch form with final-block query pruning (same results to the precision class)."""
+    """The throughput forms at every batch size (the latency form that small batches take by default is switched off):
+    prune=False: one persistent kernel, every token of the last block; prune=True: the two-launch form with
+    final-block query pruning."""
     c = cm.CONFIGS[1]
     spec = c["spec"]
     p, m = _build(spec, c["w_seed"], dtype, "fused")
     m.prune_final = prune
+    m.latency_form = False
     assert m.fused_supported()
     obs, k = cm.make_inputs(spec, B, c["obs_seed"], c["mask"])
     lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
@@ -176,6 +178,7 @@ def test_fused_route_config1(dtype, B, prune):
 def test_fused_route_variants(act, final_ln, L, ffn, dtype, ceil, margin):
     spec = cm.ConfigSpec(L, 128, 4, ffn, 16, act=act, final_ln=final_ln)
     p, m = _build(spec, 31, dtype, "fused")
+    m.latency_form = False
     obs, k = cm.make_inputs(spec, 333, 32, "quarter_empty")
     for prune in (False, True):
         m.prune_final = prune
@@ -201,6 +204,7 @@ def test_fused_route_invariants(prune):
     spec = c["spec"]
     p, m = _build(spec, 1, "f16", "fused")
     m.prune_final = prune
+    m.latency_form = False
     obs, k = cm.make_inputs(spec, 700, 3, "uniform")
     od, kd = obs.to(DEV), k.to(DEV)
     lg, v = m.forward_stacked(od, kd)
@@ -251,6 +255,7 @@ def test_fused_route_packed_tiles_give_the_unpacked_bits(dtype, case, B):
     c = cm.CONFIGS[1]
     spec = c["spec"]
     p, m = _build(spec, c["w_seed"], dtype, "fused")
+    m.latency_form = False                       # the packed first launch is a throughput form: keep small batches on it
     obs, k = cm.make_inputs(spec, B, 40 + B, "uniform")
     if case == "all_short":
         k = k % 8
@@ -303,6 +308,7 @@ def test_fused_route_packed_forward_replays_in_a_graph_with_new_key_counts():
     c = cm.CONFIGS[1]
     spec = c["spec"]
     _, m = _build(spec, c["w_seed"], "f16", "fused")
+    m.latency_form = False
     B = 3000
     obs0, k0 = cm.make_inputs(spec, B, 1, "uniform")
     s_obs, s_k = obs0.to(DEV), k0.to(DEV)
@@ -319,6 +325,93 @@ def test_fused_route_packed_forward_replays_in_a_graph_with_new_key_counts():
         got_lg, got_v = g_lg.clone(), g_v.clone()
         x = torch.randn(300, 300, device=DEV)
         (x @ x).sum().item()                                       # unrelated eager work and a sync between replays
+        lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+        assert torch.equal(got_lg, lg) and torch.equal(got_v, v), seed
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("B", [1, 8, 64, 257, 700, 1024])
+def test_fused_route_latency_form(dtype, B):
+    """The form small batches take by default (B <= 4 per CU): one persistent launch, one env per wave (1..4 working
+    waves per workgroup), weights through the deep direct-to-LDS ring.  Its output BITS are those of both throughput
+    forms - so an env's result does not depend on the batch size picking the kernel - and it holds the same literal
+    ceilings against the oracle, batch-slice invariance and masked-junk invariance."""
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    p, m = _build(spec, c["w_seed"], dtype, "fused")
+    assert m.latency_form
+    obs, k = cm.make_inputs(spec, B, c["obs_seed"], c["mask"])
+    od, kd = obs.to(DEV), k.to(DEV)
+    lg, v = m.forward_stacked(od, kd)
+    assert lg.shape == (B, 29, 7) and lg.dtype is torch.float32 and v.shape == (B,)
+    # (bf16 at B = 1024, a batch the other tests do not run: 4.44e-2 / 2.99e-2 / 2.84e-2)
+    ceil, margin = ((6.4e-3, 4.9e-3, 3.4e-3), None) if dtype == "f16" else ((5.6e-2, 4.2e-2, 3.6e-2), 0.11)
+    _check16(lg, v, p, spec, obs, k, dtype, round_residual=False, ceil=ceil, margin=margin)
+    l2, v2 = m.forward_stacked(od, kd)
+    assert torch.equal(l2, lg) and torch.equal(v2, v)                         # reproducible
+    if B >= 64:
+        for lo, hi in ((0, 1), (5, 9), (33, 64)):
+            l3, v3 = m.forward_stacked(od[lo:hi].contiguous(), kd[lo:hi].contiguous())
+            assert torch.equal(l3, lg[lo:hi]) and torch.equal(v3, v[lo:hi])   # batch / wave position invariance
+    obs2 = obs.clone()
+    for e in range(B):
+        obs2[e, spec.prop_dim + int(k[e]) * spec.obj_dim:] = 55.0
+    l4, v4 = m.forward_stacked(obs2.to(DEV), kd)
+    assert torch.equal(l4, lg) and torch.equal(v4, v)                         # masked junk cannot leak
+    m.latency_form = False
+    for prune in (False, True):                                               # the throughput forms: the same bits
+        m.prune_final = prune
+        l5, v5 = m.forward_stacked(od, kd)
+        assert torch.equal(l5, lg) and torch.equal(v5, v), prune
+
+
+@pytest.mark.parametrize("act,final_ln,L,ffn,dtype,ceil,margin", [
+    ("relu", True, 3, 256, "f16", (3.8e-3, 2.7e-3, 2.1e-3), None), ("gelu", True, 1, 512, "bf16", (2.5e-2, 1.8e-2, 1.1e-2), 0.05),
+    ("gelu", False, 6, 64, "f16", (1.4e-2, 1.2e-2, 5.9e-3), None)])
+def test_fused_route_latency_form_variants(act, final_ln, L, ffn, dtype, ceil, margin):
+    spec = cm.ConfigSpec(L, 128, 4, ffn, 16, act=act, final_ln=final_ln)
+    p, m = _build(spec, 31, dtype, "fused")
+    obs, k = cm.make_inputs(spec, 333, 32, "quarter_empty")
+    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    _check16(lg, v, p, spec, obs, k, dtype, round_residual=False, ceil=ceil, margin=margin)
+    lg0, v0 = m.forward_stacked(obs.to(DEV), None)                             # no mask == full mask
+    full = torch.full((333,), spec.T - 1, dtype=torch.int32, device=DEV)
+    lg1, v1 = m.forward_stacked(obs.to(DEV), full)
+    assert torch.equal(lg0, lg1) and torch.equal(v0, v1)
+    m.latency_form = False
+    lg2, v2 = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    assert torch.equal(lg2, lg) and torch.equal(v2, v)
+
+
+def test_fused_route_eight_layer_model_has_no_latency_form():
+    """Vectors + ring beyond a workgroup's LDS: small batches take the throughput forms, silently."""
+    spec = cm.ConfigSpec(8, 128, 4, 2048, 16)
+    p, m = _build(spec, 31, "f16", "fused")
+    obs, k = cm.make_inputs(spec, 5, 32, "uniform")
+    a = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    m.latency_form = False
+    b = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_fused_route_latency_form_replays_in_a_graph():
+    c = cm.CONFIGS[1]
+    spec = c["spec"]
+    _, m = _build(spec, c["w_seed"], "f16", "fused")
+    obs0, k0 = cm.make_inputs(spec, 64, 1, "uniform")
+    s_obs, s_k = obs0.to(DEV), k0.to(DEV)
+    m.forward_stacked(s_obs, s_k)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        g_lg, g_v = m.forward_stacked(s_obs, s_k)
+    for seed in (5, 6, 7):
+        obs, k = cm.make_inputs(spec, 64, seed, "uniform")
+        s_obs.copy_(obs.to(DEV)); s_k.copy_(k.to(DEV))
+        g.replay()
+        got_lg, got_v = g_lg.clone(), g_v.clone()
+        x = torch.randn(300, 300, device=DEV)
+        (x @ x).sum().item()
         lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
         assert torch.equal(got_lg, lg) and torch.equal(got_v, v), seed
 
