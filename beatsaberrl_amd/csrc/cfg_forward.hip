@@ -27,6 +27,7 @@
 // flat fp16 replica buffer (python/fp16_linear.py:249-346).
 #include "bsrl_common.h"
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -63,6 +64,7 @@ struct FwdArgs {
                                   // before it), written by cfg_pair_kernel
     const int32_t* n_packed;      // PACK: number of tiles in `pairs`
     int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
+    int cus;          // CUs of the device (PACK: the remainder split below)
     int ring_epw;     // RING: envs per workgroup (1..4): one per wave, the other waves only feed the weight ring
 };
 
@@ -174,11 +176,11 @@ constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 
 // LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
 // multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
 // and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
-template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false>
-__global__ __launch_bounds__(256, (RT <= 2 && !RING) ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
+template <typename DT, int KRT, int ACT, int MODE, bool PACK = false, bool RING = false>
+__global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
     static_assert(!RING || MODE == MODE_FULL, "the ring pipeline is the one-launch latency form");
-    static_assert(RT == 1 || RT == 2, "the softmax butterflies pair the row tiles");
+    static_assert(KRT == 1 || KRT == 2, "the softmax butterflies pair the row tiles");
     __shared__ uint4 lds[RING ? 1 : 2][RING ? 64 : STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256, (RT <= 2 && !RING) ? 2 : 1) void cfg_forward_k
     const int r16 = lane & 15, g = lane >> 4;
     const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
     constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? TAIL_ENVS : 1;     // envs per 16-row MFMA tile
-    constexpr int ENVS_PER_WG = 4 * RT * ENVS_PER_TILE;
+    constexpr int ENVS_PER_WG = 4 * KRT * ENVS_PER_TILE;
     const int64_t n_units = PACK ? (int64_t)*a.n_packed : a.B;           // 16-row tiles (PACK) or envs to cover
     const int64_t ntiles = RING ? (a.B + a.ring_epw - 1) / a.ring_epw : (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
@@ -274,15 +276,11 @@ __global__ __launch_bounds__(256, (RT <= 2 && !RING) ? 2 : 1) void cfg_forward_k
         lds_barrier();
     }
 
-    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t env0 = RING ? tile * a.ring_epw + uwave : tile * ENVS_PER_WG + (int64_t)wave * RT * ENVS_PER_TILE;
-        if (RING && (uwave >= a.ring_epw || env0 >= a.B)) {
-            // a wave without an env: it keeps its share of the weight ring moving (loads, waits, barriers - exactly one
-            // advance per stage, like the working waves) and reads no fragment, so the workgroup's LDS reads are those
-            // of its working waves only
-            for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
-            continue;
-        }
+    // One pass of this wave over the weight stream with RT row tiles.  A generic lambda so that the packed first launch
+    // can hold two bodies: two row tiles per wave for the bulk, ONE for the remainder tiles of the last round (below).
+    // env0: the wave's first env (or first tile, PACK).
+    auto pass = [&](auto rt_tag, const int64_t env0) __attribute__((always_inline)) {
+        constexpr int RT = decltype(rt_tag)::value;
         // every lambda below is force-inlined: one left out of line would take the residual registers by reference,
         // i.e. through scratch memory (seen with the bf16 instantiations, whose pack helper is larger)
         float kmask[RT][4];     // additive key mask for keys 4g..4g+3 of each env: 0 (attendable) or -inf
@@ -826,6 +824,38 @@ __global__ __launch_bounds__(256, (RT <= 2 && !RING) ? 2 : 1) void cfg_forward_k
             norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
             heads(yf, env0, TAIL_ENVS, fv);
         }
+    };
+    typedef std::integral_constant<int, KRT> rt_bulk;
+
+    // PACK: the remainder of the last round runs as ONE-tile passes.  A SIMD turns out tiles at a fixed rate whether it
+    // holds one wave or two, so what counts is tiles per SIMD; workgroups b and b + CUs share a CU.  With P two-tile
+    // workgroup passes, the r = P mod CUs passes past the last multiple of the CU count put a second (or third) pass on r
+    // CUs: those few tiles then cost a whole two-tile pass time at the end of the launch (the headline batch: 1283 passes,
+    // r = 3: 23 tiles = the last 24 us of 143).  When r is small, the tiles of those r passes go instead, four to a
+    // workgroup and one to a wave, to the workgroups that idle in that round: half the added time, on twice the CUs.
+    int64_t n_bulk = ntiles;                 // workgroup passes of the bulk body
+    int64_t rem_tile0 = 0; int rem_first_wg = 0, rem_passes = 0;
+    if (PACK && KRT == 2 && a.cus > 0) {
+        const int64_t r = ntiles % a.cus;
+        const int64_t p2 = ntiles - r;
+        const int64_t nrem = n_units - p2 * ENVS_PER_WG;                 // tiles left for one-tile passes
+        const int q = (int)((nrem + 3) / 4), fb = (int)(p2 % gridDim.x);
+        if (r > 0 && r <= 32 && p2 > 0 && fb + q <= (int)gridDim.x) { n_bulk = p2; rem_tile0 = p2 * ENVS_PER_WG; rem_first_wg = fb; rem_passes = q; }
+    }
+    for (int64_t tile = blockIdx.x; tile < n_bulk; tile += gridDim.x) {
+        const int64_t env0 = RING ? tile * a.ring_epw + uwave : tile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE;
+        if (RING && (uwave >= a.ring_epw || env0 >= a.B)) {
+            // a wave without an env: it keeps its share of the weight ring moving (loads, waits, barriers - exactly one
+            // advance per stage, like the working waves) and reads no fragment, so the workgroup's LDS reads are those
+            // of its working waves only
+            for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
+            continue;
+        }
+        pass(rt_bulk(), env0);
+    }
+    if (PACK && KRT == 2) {
+        const int qi = (int)blockIdx.x - rem_first_wg;
+        if (qi >= 0 && qi < rem_passes) pass(std::integral_constant<int, 1>(), rem_tile0 + (int64_t)qi * 4 + wave);
     }
     if (RING) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
@@ -1190,7 +1220,7 @@ int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed
     a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
     a.ws = static_cast<uint32_t*>(rows);
-    a.ring_epw = 4;
+    a.ring_epw = 4; a.cus = 0;
     // the TAIL launch's 4-deep weight pipeline counts stages modulo 4: it needs a hidden width that is a multiple of 64
     const bool pruned = rows && d->ffn % 64 == 0;
     // short envs share tiles when the caller gives key counts, there is room for the tile table and the descriptor
@@ -1206,6 +1236,7 @@ int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    a.cus = cus;
     // the latency form (one launch, one env per wave, deep direct-to-LDS weight ring) for small batches, unless the
     // descriptor switches it off or vectors + ring exceed one workgroup's LDS; same output bits as the other forms
     // (and the batch is one pass of one workgroup per CU: past that the persistent loop would drain the ring once per
