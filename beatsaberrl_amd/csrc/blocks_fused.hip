@@ -414,6 +414,397 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 }
 
 
+
+// ---- the same stack with ONE WAVE PER ENV ---------------------------------------------------------------------
+// Mapping.  A wave owns both 16-row tiles of an env (all its <= 32 tokens) and carries their fp32 residual stream in
+// registers; a workgroup is 8 waves = 8 envs, one workgroup per CU, two waves per SIMD in 256 registers each.
+// Against blocks_kernel (a wave per row tile, an env a wave pair, 4 envs per workgroup):
+//   * every weight fragment read from LDS feeds TWO MFMAs (one per row tile) instead of one, and a stage streamed from
+//     L2 serves 8 envs instead of 4: half the LDS read instructions, barriers and stage loads per env;
+//   * attention needs no LDS: a wave holds the K and V^T fragments of both key tiles of the head it just projected;
+//   * stages go global -> LDS directly (global_load_lds_dwordx4, one 1 KB fragment per wave instruction) several
+//     stages ahead into a ring of SLOTS stage slots: no register staging, depth bounded by LDS only;
+//   * the row reductions of LayerNorm and softmax are lane-row swaps on the VALU, not shuffles through LDS.
+// Per-row arithmetic, its order and the weight image are those of blocks_kernel: an env's output bits are the same.
+template <int D> struct EnvRing {
+    static constexpr int NW = 8;
+    static constexpr int SLOTS = D == 128 ? 10 : 7;                                    // stage slots
+    static constexpr int AHEAD = SLOTS - 2;     // stages that may be in flight at a stage's entry: all but it and the one being refilled
+    static constexpr int STAGE_BYTES = Geo<D>::SF * 1024;
+    // fragment f of a stage is loaded by wave f % NW: LPW_HI loads for waves < N_HI, LPW_HI - 1 for the others
+    static constexpr int LPW_HI = (Geo<D>::SF + NW - 1) / NW, N_HI = Geo<D>::SF - (LPW_HI - 1) * NW;
+    static_assert(LPW_HI * (AHEAD + 1) < 64, "vmcnt is 6 bits");
+};
+// m0 (the LDS base of the transfer) is written without telling the compiler, which rejects reserved registers in a
+// clobber list: nothing else in the kernel uses it.  No "memory" clobber: what orders these asynchronous LDS writes
+// against the fragment reads is the vmcnt wait + barrier of the stage advance.
+__device__ __forceinline__ void env_ring_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr));
+}
+
+template <typename DT, int D, int DH, int ACT>
+__global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
+    typedef Geo<D> G;
+    typedef EnvRing<D> R;
+    constexpr int NW = R::NW;
+    constexpr int NT = G::NT, KC = G::KC, H = D / DH, TPH = DH / 16;
+    constexpr int NB = G::NB, KB = G::KB, SF = G::SF;
+    // a stage is consumed in 2 * NB sub-bursts of KB fragments (a burst of blocks_kernel is two of them: the k chunks
+    // [b * KB, +KB) of the stage's first tile, then of its second; in a W2 stage KB consecutive feature tiles)
+    constexpr int NSUB = 2 * NB;
+    static_assert(G::FB == 2 * KB, "a burst is two sub-bursts");
+    extern __shared__ float4 bvl4[];          // fp32 vectors of every block, then the stage ring (1 KB aligned)
+    const float* vlds = reinterpret_cast<const float*>(bvl4);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const float scale_l2e = (DH == 32 ? 0.17677669529663688110f : 0.14433756729740644113f) * 1.44269504088896340736f;
+    const int64_t ntiles = (a.B + NW - 1) / NW;
+    const int ring_off_u4 = (a.n_layers * G::lv_size(a.F) / 4 + 63) & ~63;
+    const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
+    const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
+    const char* img = reinterpret_cast<const char*>(a.frags);
+
+    int cur = R::SLOTS - 1, pnext;
+    auto issue = [&](int stage, int slot) __attribute__((always_inline)) {
+        const char* sb = img + (int64_t)stage * R::STAGE_BYTES;
+        const uint32_t dst = ring_base + slot * R::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < R::LPW_HI; ++i)
+            if (i + 1 < R::LPW_HI || wave < R::N_HI) env_ring_load(lane * 16, sb + (wave + NW * i) * 1024, dst + (wave + NW * i) * 1024);
+    };
+    // entry of the next stage: on return it is readable in slot `cur`
+    auto advance = [&]() __attribute__((always_inline)) {
+        cur = cur + 1 == R::SLOTS ? 0 : cur + 1;
+        // this wave's loads of that stage have landed once at most the AHEAD younger stages' are outstanding (loads
+        // retire in order; any other load or store in flight only makes the wait stricter) ...
+        if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
+        blk_barrier();                 // ... and every wave's have; every wave is done reading the stage before it
+        issue(pnext, cur == 0 ? R::SLOTS - 1 : cur - 1);
+        pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+    };
+    // sub-burst j of the current stage -> registers, then `body` on them
+    auto sub = [&](auto j_, auto&& body) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_)::value;
+        s16x8 w[KB];
+#pragma unroll
+        for (int f = 0; f < KB; ++f) w[f] = __builtin_bit_cast(s16x8, ring[cur * (SF * 64) + (j * KB + f) * 64 + lane]);
+        body(w);
+    };
+    {   // prologue: SLOTS - 1 stages in flight (every stack has more), then the vectors
+        int st = 0;
+#pragma unroll
+        for (int i = 0; i < R::SLOTS - 1; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
+        pnext = st;
+        const int nv4 = a.n_layers * G::lv_size(a.F) / 4;
+        for (int i = tid; i < nv4; i += NW * 64) bvl4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        blk_barrier();
+    }
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t env = tile * NW + wave;
+        const int64_t envc = env < a.B ? env : a.B - 1;
+        f32x4 x[2][NT];
+        BFrag8 hf[2][KC];    // LayerNorm output as operand fragments
+        BFrag8 of[2][KC];    // attention output fragments
+        float kmask[2][4];   // additive key bias * log2(e) for keys 16*kt + 4g + i; -inf past T
+        // the tile's own loads are all issued, then waited for ONCE, with the wait the compiler can see (vmcnt(0); expcnt /
+        // lgkmcnt at their maxima).  It does not know of the ring's loads: wherever it later met a value of its own still
+        // in flight - or reused such a register - it would wait for every outstanding load, i.e. drain the ring in mid-tile.
+        uint2 raw[2][NT];
+        u16 kraw[2][4];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int row = 16 * rt + r16;
+            const u16* xr = a.x_in + (envc * a.T + (row < a.T ? row : 0)) * D;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) raw[rt][nt] = *reinterpret_cast<const uint2*>(xr + 16 * nt + 4 * g);
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = 16 * kt + 4 * g + i;
+                kraw[kt][i] = a.key_bias[envc * a.T + (key < a.T ? key : 0)];
+            }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const bool row_ok = 16 * rt + r16 < a.T;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const uint32_t lo = row_ok ? raw[rt][nt].x : 0u, hi = row_ok ? raw[rt][nt].y : 0u;      // 0 bits = +0.0
+                x[rt][nt][0] = DT::to_f((u16)(lo & 0xffff)); x[rt][nt][1] = DT::to_f((u16)(lo >> 16));
+                x[rt][nt][2] = DT::to_f((u16)(hi & 0xffff)); x[rt][nt][3] = DT::to_f((u16)(hi >> 16));
+            }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                kmask[kt][i] = 16 * kt + 4 * g + i < a.T ? DT::to_f(kraw[kt][i]) * 1.44269504088896340736f : -INFINITY;
+
+        // LayerNorm of both row tiles (of row tile 0 only: `both` false) -> operand fragments; the statistics of the two
+        // tiles go through the lane-row butterfly together
+        auto norm_to_frags = [&](bool both, const float* gptr, const float* bptr) __attribute__((always_inline)) {
+            // one pass: var = E[x^2] - mean^2 clamped at 0 (python/beat_arena_env/csrc/layer_norm.cu:14-21)
+            float s[2] = {0.f, 0.f}, q[2] = {0.f, 0.f};
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt == 1 && !both) break;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { s[rt] += x[rt][nt][i]; q[rt] = fmaf(x[rt][nt][i], x[rt][nt][i], q[rt]); }
+            }
+            rows_reduce2(s[0], q[0], OpAdd());
+            if (both) rows_reduce2(s[1], q[1], OpAdd());
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt == 1 && !both) break;
+                const float mean = s[rt] * (1.0f / D);
+                const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q[rt] * (1.0f / D)), 0.f) + 1e-5f);
+                const float shift = -mean * rstd;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4 gm = *reinterpret_cast<const float4*>(gptr + 16 * nt + 4 * g);
+                    const float4 bt = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+                    const float y0 = fmaf(fmaf(x[rt][nt][0], rstd, shift), gm.x, bt.x);
+                    const float y1 = fmaf(fmaf(x[rt][nt][1], rstd, shift), gm.y, bt.y);
+                    const float y2 = fmaf(fmaf(x[rt][nt][2], rstd, shift), gm.z, bt.z);
+                    const float y3 = fmaf(fmaf(x[rt][nt][3], rstd, shift), gm.w, bt.w);
+                    hf[rt][nt >> 1].w[(nt & 1) * 2] = bpack2<DT>(y0, y1);
+                    hf[rt][nt >> 1].w[(nt & 1) * 2 + 1] = bpack2<DT>(y2, y3);
+                }
+            }
+        };
+        auto add_bias = [&](auto rt_, const float* bptr) __attribute__((always_inline)) {
+            constexpr int rt = decltype(rt_)::value;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const float4 b = *reinterpret_cast<const float4*>(bptr + 16 * nt + 4 * g);
+                x[rt][nt][0] += b.x; x[rt][nt][1] += b.y; x[rt][nt][2] += b.z; x[rt][nt][3] += b.w;
+            }
+        };
+        auto store_rows = [&](auto rt_, u16* dst, int rows_per_env, int nrows_valid) __attribute__((always_inline)) {
+            constexpr int rt = decltype(rt_)::value;
+            const int row = 16 * rt + r16;
+            if (env < a.B && row < nrows_valid) {
+                u16* o = dst + (env * rows_per_env + row) * D;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    uint2 v;
+                    v.x = bpack2<DT>(x[rt][nt][0], x[rt][nt][1]); v.y = bpack2<DT>(x[rt][nt][2], x[rt][nt][3]);
+                    *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                }
+            }
+        };
+        typedef std::integral_constant<int, 0> T0;
+        typedef std::integral_constant<int, 1> T1;
+
+        // one block; the pruned final block computes queries, output projection and FFN for row tile 0 only (keys and
+        // values of both).  `pruned` is a compile-time constant: the full blocks carry no branches around their MFMAs.
+        auto layer = [&](int l, auto pruned_) __attribute__((always_inline)) {
+            constexpr bool pruned = decltype(pruned_)::value;
+            constexpr int QT = pruned ? 1 : 2;                 // query row tiles
+            const float* lv = vlds + l * G::lv_size(a.F);
+            if (pruned && a.x_res) { store_rows(T0(), a.x_res, a.T, a.T); store_rows(T1(), a.x_res, a.T, a.T); }
+
+            norm_to_frags(true, lv + G::LN1G, lv + G::LN1B);
+
+            uint2 q[2][2][TPH];                                // Q fragments [head parity][row tile][feature tile]
+            uint2 kk[2][TPH], vv[2][TPH];                      // K, V^T fragments of the head in flight [key tile][feature tile]
+
+            // attention of head hd: the env's (up to) 32 queries over its 32 key slots, both query tiles together
+            auto attention = [&](auto hd_) __attribute__((always_inline)) {
+                constexpr int hd = decltype(hd_)::value;
+                float sv[2][2][4], m[2], sum[2];
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) {
+                    f32x4 sc[2];
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt) {
+                        BFrag8 kf, qf;
+                        kf.h[0] = kk[kt][0]; kf.h[1] = kk[kt][1];
+                        qf.h[0] = q[hd & 1][qt][0]; qf.h[1] = q[hd & 1][qt][1];
+                        sc[kt] = DT::mfma32(kf.v, qf.v, (f32x4){0.f, 0.f, 0.f, 0.f});
+                        if (TPH == 3) {
+                            // features 32..47: a K = 16 MFMA into its OWN accumulator (chaining it onto the
+                            // 16x16x32 accumulator loses the first product on this hardware), summed on the VALU
+                            BFrag4 k2, q2;
+                            k2.h = kk[kt][TPH - 1]; q2.h = q[hd & 1][qt][TPH - 1];
+                            const f32x4 s2 = DT::mfma16(k2.v, q2.v, (f32x4){0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) sc[kt][i] += s2[i];
+                        }
+                    }
+                    m[qt] = -INFINITY;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { sv[qt][kt][i] = fmaf(sc[kt][i], scale_l2e, kmask[kt][i]); m[qt] = fmaxf(m[qt], sv[qt][kt][i]); }
+                }
+                if (QT == 1) m[1] = m[0];
+                rows_reduce2(m[0], m[1], OpMax());
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) {
+                    sum[qt] = 0.f;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { sv[qt][kt][i] = __builtin_amdgcn_exp2f(sv[qt][kt][i] - m[qt]); sum[qt] += sv[qt][kt][i]; }
+                }
+                if (QT == 1) sum[1] = sum[0];
+                rows_reduce2(sum[0], sum[1], OpAdd());
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) {
+                    const float inv = __builtin_amdgcn_rcpf(sum[qt]);
+                    BFrag8 pf;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt) {
+                        pf.w[2 * kt] = bpack2<DT>(sv[qt][kt][0] * inv, sv[qt][kt][1] * inv);
+                        pf.w[2 * kt + 1] = bpack2<DT>(sv[qt][kt][2] * inv, sv[qt][kt][3] * inv);
+                    }
+#pragma unroll
+                    for (int t = 0; t < TPH; ++t) {
+                        BFrag8 vf;
+                        vf.h[0] = vv[0][t]; vf.h[1] = vv[1][t];
+                        const float4 bv = *reinterpret_cast<const float4*>(lv + G::BV + DH * hd + 16 * t + 4 * g);
+                        const f32x4 o = DT::mfma32(vf.v, pf.v, (f32x4){bv.x, bv.y, bv.z, bv.w});
+                        const int nt = hd * TPH + t;
+                        of[qt][nt >> 1].w[(nt & 1) * 2] = bpack2<DT>(o[0], o[1]);
+                        of[qt][nt >> 1].w[(nt & 1) * 2 + 1] = bpack2<DT>(o[2], o[3]);
+                    }
+                }
+            };
+
+            // ---- packed q|k|v projection: 3 * NT feature tiles in head-major order [q | k | v] per head, two per stage ----
+            static_for<0, 3 * NT / 2>([&](auto st_) __attribute__((always_inline)) {
+                constexpr int st = decltype(st_)::value;
+                advance();
+                // a head whose last tile was computed in an earlier stage is complete now: its attention runs before
+                // this stage's results overwrite the K / V registers (a stage that straddles two heads holds the LAST
+                // tile of one and the FIRST - a query tile, double-buffered by head parity - of the next)
+                if constexpr (st > 0) {
+                    constexpr int done = (2 * st) / (3 * TPH);
+                    constexpr int done_prev = (2 * st - 2) / (3 * TPH);
+                    if constexpr (done > done_prev) attention(std::integral_constant<int, done - 1>{});
+                }
+                f32x4 acc[2][2];                                 // [tile of the stage][row tile]
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
+                    float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? G::BQ : G::BK) + DH * hd + 16 * t + 4 * g);
+                    acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
+                }
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;    // k chunks [half * KB, +KB) of tile ntl
+                    sub(j_, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int ci = 0; ci < KB; ++ci)
+#pragma unroll
+                            for (int rt = 0; rt < 2; ++rt) {
+                                const int c = half * KB + ci;
+                                const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
+                                if (part == 0 && rt >= QT) continue;     // the pruned block needs no queries from row tile 1
+                                if (part < 2) acc[ntl][rt] = DT::mfma32(wf[ci], hf[rt][c].v, acc[ntl][rt]);
+                                else acc[ntl][rt] = DT::mfma32(hf[rt][c].v, wf[ci], acc[ntl][rt]);   // V^T: operand roles swapped
+                            }
+                    });
+                });
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl)
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt) {
+                        const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
+                        if (part == 0 && rt >= QT) continue;
+                        uint2 pk;
+                        pk.x = bpack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]); pk.y = bpack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
+                        if (part == 0) q[hd & 1][rt][t] = pk;
+                        else if (part == 1) kk[rt][t] = pk;
+                        else vv[rt][t] = pk;
+                    }
+            });
+
+            // ---- output projection onto the residual (NT / 2 stages) ----
+            add_bias(T0(), lv + G::BOUT);
+            if (!pruned) add_bias(T1(), lv + G::BOUT);
+            static_for<0, NT / 2>([&](auto st_) __attribute__((always_inline)) {
+                constexpr int st = decltype(st_)::value;
+                advance();
+                if constexpr (st == 0) attention(std::integral_constant<int, H - 1>{});      // the last head completed in the previous stage
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;
+                    sub(j_, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int ci = 0; ci < KB; ++ci)
+#pragma unroll
+                            for (int qt = 0; qt < QT; ++qt)
+                                x[qt][2 * st + ntl] = DT::mfma32(wf[ci], of[qt][half * KB + ci].v, x[qt][2 * st + ntl]);
+                    });
+                });
+            });
+
+            // ---- LayerNorm + FFN: stage order W1(0), {W1(ch+1), W2(ch)}..., W2(last); the hidden of a 32-unit chunk
+            //      lives in two accumulators per row tile, activated and packed into one operand fragment ----
+            norm_to_frags(!pruned, lv + G::LN2G, lv + G::LN2B);
+            add_bias(T0(), lv + G::b2(a.F));
+            if (!pruned) add_bias(T1(), lv + G::b2(a.F));
+            const int nch = a.F / 32;
+            f32x4 acc[2][2];                                     // [tile of the chunk][row tile]
+            auto up = [&](int ch) __attribute__((always_inline)) {
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const float4 b = *reinterpret_cast<const float4*>(lv + G::B1 + 32 * ch + 16 * ntl + 4 * g);
+                    acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
+                }
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;
+                    sub(j_, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int ci = 0; ci < KB; ++ci)
+#pragma unroll
+                            for (int qt = 0; qt < QT; ++qt)
+                                acc[ntl][qt] = DT::mfma32(wf[ci], hf[qt][half * KB + ci].v, acc[ntl][qt]);
+                    });
+                });
+            };
+            advance();
+            up(0);
+            for (int ch = 0; ch < nch; ++ch) {
+                BFrag8 hid[2];
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+                    for (int ntl = 0; ntl < 2; ++ntl) {
+                        hid[qt].w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(acc[ntl][qt][0]), apply_act16<ACT>(acc[ntl][qt][1]));
+                        hid[qt].w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(acc[ntl][qt][2]), apply_act16<ACT>(acc[ntl][qt][3]));
+                    }
+                if (ch + 1 < nch) { advance(); up(ch + 1); }
+                advance();
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int j = decltype(j_)::value;           // feature tiles [j * KB, +KB)
+                    sub(j_, [&](const s16x8 (&w2)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int i = 0; i < KB; ++i)
+#pragma unroll
+                            for (int qt = 0; qt < QT; ++qt) x[qt][j * KB + i] = DT::mfma32(w2[i], hid[qt].v, x[qt][j * KB + i]);
+                    });
+                });
+            }
+        };
+        const int n_full = a.n_queries > 0 ? a.n_layers - 1 : a.n_layers;
+        for (int l = 0; l < n_full; ++l) layer(l, std::false_type{});
+        if (a.n_queries > 0) layer(a.n_layers - 1, std::true_type{});
+        if (a.n_queries > 0) store_rows(T0(), a.x_out, a.n_queries, a.n_queries);
+        else { store_rows(T0(), a.x_out, a.T, a.T); store_rows(T1(), a.x_out, a.T, a.T); }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
+    blk_barrier();
+}
+
 // ---- weight image ------------------------------------------------------------------
 struct BlkPackArgs {
     bsrl_blocks_params p;
@@ -509,8 +900,31 @@ void pack_launch(const BlkPackArgs& pa, int64_t nfrags, hipStream_t st) {
     hipLaunchKernelGGL(blocks_pack_vec_kernel<D>, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, st, pa);
 }
 
+// dynamic LDS of the env-per-wave kernel: vectors (rounded to 1 KB) + ring
+template <int D> size_t env_dyn_bytes(int n_layers, int F) {
+    return (size_t)((n_layers * Geo<D>::lv_size(F) / 4 + 63) & ~63) * 16 + (size_t)EnvRing<D>::SLOTS * EnvRing<D>::STAGE_BYTES;
+}
+// The env-per-wave kernel runs where a wave's state fits 256 registers (d = 128 and 192: at d = 256 it would spill
+// several hundred values), the vectors and the stage ring fit a workgroup's LDS, and the stack is at least as long as
+// the ring; the wave-pair kernel otherwise.
+template <int D> bool env_kernel_ok(const BlkArgs& a) {
+    if (D == 256) return false;
+    return env_dyn_bytes<D>(a.n_layers, a.F) + 1024 <= (size_t)LDS_BUDGET && a.total_stages >= EnvRing<D>::SLOTS;
+}
+
 template <typename DT, int D, int DH, int ACT>
 int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
+    if constexpr (D != 256) {
+        if (env_kernel_ok<D>(a)) {
+            const size_t dyn = env_dyn_bytes<D>(a.n_layers, a.F);
+            const int64_t ntiles = (a.B + EnvRing<D>::NW - 1) / EnvRing<D>::NW;
+            auto kern = blocks_env_kernel<DT, D, DH, ACT>;
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+                return BSRL_UNSUPPORTED;
+            hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(EnvRing<D>::NW * 64), dyn, st, a);
+            return BSRL_OK;
+        }
+    }
     const size_t dyn = (size_t)a.n_layers * Geo<D>::lv_size(a.F) * sizeof(float);
     const int64_t ntiles = (a.B + 3) / 4;
     const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));

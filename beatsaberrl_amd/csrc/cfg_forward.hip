@@ -87,26 +87,6 @@ template <> __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
 union Frag8 { s16x8 v; uint32_t w[4]; uint4 u; };
 union Frag4 { s16x4 v; uint32_t w[2]; };
 
-// gfx950's lane-row exchanges, as plain VALU instructions (no LDS round trip, no lgkmcnt wait behind the weight
-// fragment reads).  A wave is four rows of 16 lanes.  v_permlane16_swap_b32 a, b: rows 1 and 3 of a change places
-// with rows 0 and 2 of b; v_permlane32_swap_b32 a, b: rows 2..3 of a with rows 0..1 of b.  Written as asm because
-// the compiler builtin returns the first result twice in this toolchain; the s_nop is the two wait states the
-// instruction needs after a VALU write of either operand (the compiler does not look inside an asm statement).
-__device__ __forceinline__ void row_swap16(float& a, float& b) { asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-__device__ __forceinline__ void row_swap32(float& a, float& b) { asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-// The lane-row butterfly (combine with lane ^ 16, then with lane ^ 32) of TWO values at once: on return every lane
-// holds the combination of its column over the four rows, for both values, associated (r0 . r1) . (r2 . r3) exactly
-// as the two-step shuffle butterfly associates it.  8 VALU ops for the pair.
-template <typename OP> __device__ __forceinline__ void rows_reduce2(float& s, float& q, OP op) {
-    row_swap16(s, q);                   // s = {s0, q0, s2, q2}, q = {s1, q1, s3, q3} (by row)
-    float z = op(s, q), w = z;          // {s0.s1, q0.q1, s2.s3, q2.q3}
-    row_swap32(z, w);                   // z = {z0, z1, z0, z1}, w = {z2, z3, z2, z3}
-    float t = op(z, w), u = t;          // {S, Q, S, Q}
-    row_swap16(t, u);                   // t = {S, S, S, S}, u = {Q, Q, Q, Q}
-    s = t; q = u;
-}
-struct OpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
-struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
 // RING variant of the weight pipeline (the latency form): stages go global -> LDS directly (global_load_lds_dwordx4:
 // one wave instruction lands one 1 KB fragment, lane l's 16 bytes at slot l), RING_DEPTH stages ahead of the one being
