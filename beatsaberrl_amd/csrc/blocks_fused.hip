@@ -429,11 +429,13 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 template <int D> struct EnvRing {
     static constexpr int NW = 8;
     static constexpr int SLOTS = D == 128 ? 10 : 7;                                    // stage slots
-    static constexpr int AHEAD = SLOTS - 2;     // stages that may be in flight at a stage's entry: all but it and the one being refilled
+    // Stages are entered in PAIRS (every block has an even number of them): one wait + barrier admits two stages and
+    // refills the two slots behind them.  Stages that may still be in flight then: all but those four.
+    static constexpr int AHEAD = SLOTS - 4;
     static constexpr int STAGE_BYTES = Geo<D>::SF * 1024;
     // fragment f of a stage is loaded by wave f % NW: LPW_HI loads for waves < N_HI, LPW_HI - 1 for the others
     static constexpr int LPW_HI = (Geo<D>::SF + NW - 1) / NW, N_HI = Geo<D>::SF - (LPW_HI - 1) * NW;
-    static_assert(LPW_HI * (AHEAD + 1) < 64, "vmcnt is 6 bits");
+    static_assert(SLOTS >= 5 && LPW_HI * (AHEAD + 2) < 64, "vmcnt is 6 bits");
 };
 // m0 (the LDS base of the transfer) is written without telling the compiler, which rejects reserved registers in a
 // clobber list: nothing else in the kernel uses it.  No "memory" clobber: what orders these asynchronous LDS writes
@@ -473,17 +475,24 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
         for (int i = 0; i < R::LPW_HI; ++i)
             if (i + 1 < R::LPW_HI || wave < R::N_HI) env_ring_load(lane * 16, sb + (wave + NW * i) * 1024, dst + (wave + NW * i) * 1024);
     };
-    // entry of the next stage: on return it is readable in slot `cur`
-    auto advance = [&]() __attribute__((always_inline)) {
+    // entry of the next stage (parity = its index in its block, mod 2): on return it is readable in slot `cur`
+    auto advance = [&](auto parity_) __attribute__((always_inline)) {
         cur = cur + 1 == R::SLOTS ? 0 : cur + 1;
-        // this wave's loads of that stage have landed once at most the AHEAD younger stages' are outstanding (loads
-        // retire in order; any other load or store in flight only makes the wait stricter) ...
-        if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
-        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
-        blk_barrier();                 // ... and every wave's have; every wave is done reading the stage before it
-        issue(pnext, cur == 0 ? R::SLOTS - 1 : cur - 1);
-        pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+        if constexpr (decltype(parity_)::value == 0) {
+            // this wave's loads of this stage and the next have landed once at most the AHEAD younger stages' are
+            // outstanding (loads retire in order; any other load or store in flight only makes the wait stricter) ...
+            if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
+            blk_barrier();             // ... and every wave's have; every wave is done reading the two stages before this one
+            const int s1 = cur == 0 ? R::SLOTS - 1 : cur - 1, s2 = s1 == 0 ? R::SLOTS - 1 : s1 - 1;
+            issue(pnext, s2);
+            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+            issue(pnext, s1);
+            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+        }
     };
+    typedef std::integral_constant<int, 0> Even;
+    typedef std::integral_constant<int, 1> Odd;
     // sub-burst j of the current stage -> registers, then `body` on them
     auto sub = [&](auto j_, auto&& body) __attribute__((always_inline)) {
         constexpr int j = decltype(j_)::value;
@@ -492,10 +501,10 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
         for (int f = 0; f < KB; ++f) w[f] = __builtin_bit_cast(s16x8, ring[cur * (SF * 64) + (j * KB + f) * 64 + lane]);
         body(w);
     };
-    {   // prologue: SLOTS - 1 stages in flight (every stack has more), then the vectors
+    {   // prologue: SLOTS - 2 stages in flight (every stack has more), then the vectors
         int st = 0;
 #pragma unroll
-        for (int i = 0; i < R::SLOTS - 1; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
+        for (int i = 0; i < R::SLOTS - 2; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
         pnext = st;
         const int nv4 = a.n_layers * G::lv_size(a.F) / 4;
         for (int i = tid; i < nv4; i += NW * 64) bvl4[i] = reinterpret_cast<const float4*>(a.vec)[i];
@@ -682,7 +691,7 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
             // ---- packed q|k|v projection: 3 * NT feature tiles in head-major order [q | k | v] per head, two per stage ----
             static_for<0, 3 * NT / 2>([&](auto st_) __attribute__((always_inline)) {
                 constexpr int st = decltype(st_)::value;
-                advance();
+                advance(std::integral_constant<int, st & 1>{});
                 // a head whose last tile was computed in an earlier stage is complete now: its attention runs before
                 // this stage's results overwrite the K / V registers (a stage that straddles two heads holds the LAST
                 // tile of one and the FIRST - a query tile, double-buffered by head parity - of the next)
@@ -733,7 +742,7 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
             if (!pruned) add_bias(T1(), lv + G::BOUT);
             static_for<0, NT / 2>([&](auto st_) __attribute__((always_inline)) {
                 constexpr int st = decltype(st_)::value;
-                advance();
+                advance(std::integral_constant<int, st & 1>{});
                 if constexpr (st == 0) attention(std::integral_constant<int, H - 1>{});      // the last head completed in the previous stage
                 static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
                     constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;
@@ -771,7 +780,8 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
                     });
                 });
             };
-            advance();
+            static_assert((3 * NT / 2) % 2 == 0 && (NT / 2) % 2 == 0, "the FFN starts on an even stage");
+            advance(Even{});
             up(0);
             for (int ch = 0; ch < nch; ++ch) {
                 BFrag8 hid[2];
@@ -782,8 +792,9 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
                         hid[qt].w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(acc[ntl][qt][0]), apply_act16<ACT>(acc[ntl][qt][1]));
                         hid[qt].w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(acc[ntl][qt][2]), apply_act16<ACT>(acc[ntl][qt][3]));
                     }
-                if (ch + 1 < nch) { advance(); up(ch + 1); }
-                advance();
+                // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
+                if (ch + 1 < nch) { advance(Odd{}); up(ch + 1); advance(Even{}); }
+                else advance(Odd{});
                 static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
                     constexpr int j = decltype(j_)::value;           // feature tiles [j * KB, +KB)
                     sub(j_, [&](const s16x8 (&w2)[KB]) __attribute__((always_inline)) {
@@ -909,13 +920,15 @@ template <int D> size_t env_dyn_bytes(int n_layers, int F) {
 // the ring; the wave-pair kernel otherwise.
 template <int D> bool env_kernel_ok(const BlkArgs& a) {
     if (D == 256) return false;
-    return env_dyn_bytes<D>(a.n_layers, a.F) + 1024 <= (size_t)LDS_BUDGET && a.total_stages >= EnvRing<D>::SLOTS;
+    return env_dyn_bytes<D>(a.n_layers, a.F) + 1024 <= (size_t)LDS_BUDGET && a.total_stages >= EnvRing<D>::SLOTS && a.total_stages % 2 == 0;
 }
 
 template <typename DT, int D, int DH, int ACT>
 int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
     if constexpr (D != 256) {
-        if (env_kernel_ok<D>(a)) {
+        // ... and the batch fills the CUs with 8-env tiles: up to 4 envs per CU the wave-pair kernel's 4-env tiles
+        // spread over twice as many CUs (both kernels produce the same bits for an env)
+        if (env_kernel_ok<D>(a) && a.B > 4 * (int64_t)cus) {
             const size_t dyn = env_dyn_bytes<D>(a.n_layers, a.F);
             const int64_t ntiles = (a.B + EnvRing<D>::NW - 1) / EnvRing<D>::NW;
             auto kern = blocks_env_kernel<DT, D, DH, ACT>;

@@ -115,6 +115,51 @@ def test_unpruned_stack_and_invariants():
     assert torch.equal(lead4, lead) and torch.equal(res4, res)
 
 
+def _run_act(sd, L, d, F, T, dtype, x, bias, n_queries, act):
+    tdt, H = TDT[dtype], _heads(d)
+    image = torch.empty(ops.blocks_pack_size(L, d, H, F, T, act, n_queries, tdt), dtype=torch.uint8, device=DEV)
+    params = [[sd[f"blocks.{i}.{f}"].to(DEV).contiguous() for f in FIELDS] for i in range(L)]
+    ops.blocks_pack(params, image, d, H, F, T, act, n_queries, tdt)
+    return ops.blocks_forward(image, x.to(DEV).to(tdt).contiguous(), bias.to(DEV).to(tdt).contiguous(), L, H, F, act, n_queries)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("d,L,T,nq,act", [(128, 2, 29, 5, "gelu"), (192, 3, 26, 6, "gelu"), (192, 2, 32, 0, "relu"),
+                                          (128, 1, 7, 7, "relu"), (192, 1, 17, 16, "gelu")])
+def test_large_batches_take_the_env_per_wave_kernel_and_give_the_same_bits(dtype, d, L, T, nq, act):
+    """Batches of more than 4 envs per CU run the env-per-wave kernel (8-env tiles), smaller ones the wave-pair
+    kernel (4-env tiles): an env's output may not depend on which of them its batch size selects.  B = 2053 is
+    ragged for both (2053 = 256 * 8 + 5); the chunks of 500 (<= 1024 on any gfx950 part with >= 125 CUs) take the
+    wave-pair kernel, which the oracle cases above pin."""
+    B, F = 2053, 4 * d
+    sd = _weights(L, d, F, 21 + d + L)
+    x, bias = _inputs(B, T, d, 5)
+    big, big_res = _run_act(sd, L, d, F, T, dtype, x, bias, nq, act)
+    for lo in range(0, B, 500):
+        hi = min(B, lo + 500)
+        small, small_res = _run_act(sd, L, d, F, T, dtype, x[lo:hi], bias[lo:hi], nq, act)
+        assert torch.equal(small, big[lo:hi]), (lo, (small.float() - big[lo:hi].float()).abs().max().item())
+        if nq > 0:
+            assert torch.equal(small_res, big_res[lo:hi]), lo
+    assert torch.isfinite(big.float()).all()
+
+
+def test_env_per_wave_kernel_matches_oracle():
+    """One direct oracle case for the large-batch kernel (its bits equal the wave-pair kernel's, which the cases above
+    pin; this one guards the equality test's own premise).  Ceilings: the batch maxima measured on this seeded case
+    (4.90e-3, 4.26e-3) plus 25 %."""
+    d, L, B, T, F, dtype = 192, 3, 1100, 29, 768, "f16"
+    sd = _weights(L, d, F, 10 + L + d)
+    x, bias = _inputs(B, T, d, 3 + B)
+    arch = {"n_heads": _heads(d), "n_blocks": L}
+    lead32, res32 = nr.blocks_forward(sd, arch, x.to(TDT[dtype]), bias)
+    out, res = _run(sd, L, d, F, T, dtype, x, bias, 5)
+    e_lead = (out.float().cpu() - lead32).abs().max().item()
+    e_res = (res.float().cpu() - res32).abs().max().item()
+    print(f"\nenv-per-wave d={d} L={L} B={B}: lead vs fp32 {e_lead:.3e}, x_res vs fp32 {e_res:.3e}")
+    assert e_lead <= 6.2e-3 and e_res <= 5.4e-3, (e_lead, e_res)
+
+
 def test_unsupported_shapes_are_reported():
     assert ops.blocks_pack_size(2, 384, 12, 1536, 32, "relu", 0, torch.float16) == 0
     assert ops.blocks_pack_size(2, 256, 4, 1024, 32, "relu", 0, torch.float16) == 0
