@@ -94,6 +94,11 @@ union Frag4 { s16x4 v; uint32_t w[2]; };
 // A lone workgroup walking ~100 stages is bound by the L2 round trip divided by the stages in flight: 3 in the
 // register-staged pipeline, 13 here.
 constexpr int RING_DEPTH = 13, RING_SLOTS = RING_DEPTH + 1;
+// DMA variant (the throughput forms: whole forward / first launch): the same direct-to-LDS transfers into a ring of
+// DMA_SLOTS stage slots, stages admitted in PAIRS - one vmcnt wait + barrier per two stages, then the two slots behind
+// them are refilled - against one barrier, two LDS stores and two register-staged loads per stage in the
+// register-staged pipeline.  While a pair is consumed, DMA_SLOTS - 4 further stages are in flight.
+constexpr int DMA_SLOTS = 6, DMA_AHEAD = DMA_SLOTS - 4;
 // m0 (the LDS base of the transfer) is written without telling the compiler, which rejects reserved registers in a
 // clobber list: nothing else in these kernels uses it (no dynamically indexed register arrays, no instruction that
 // reads m0).  No "memory" clobber: what orders the asynchronous LDS writes against the fragment reads is the explicit
@@ -119,7 +124,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
         pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1; \
     } while (0)
 // (RING: the advance happens inside the fragment fetch, one stage ahead - see ring_take)
-#define ADVANCE(par) do { if (RING) { } else if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
+// (DMA: the throughput forms' direct-to-LDS pipeline - see dma_advance)
+#define ADVANCE(par) do { if (RING) { } else if (DMA) dma_advance(par); else if (par) ADVANCE_P(1, pr0a, pr0b); else ADVANCE_P(0, pr1a, pr1b); } while (0)
 // TAIL launch: a workgroup streams its 44 stages for ONE tile with little arithmetic per stage, so the
 // step time is the L2 latency of the weight stream divided by the stages in flight.  Four register
 // sets (q0..q3) keep four stages in flight instead of two: ADVANCE4(Q), Q = index of the stage about to
@@ -131,7 +137,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // ADV(sidx): sidx = stage index counted from the start of the block (HEAD / FULL: only its parity
 // matters) or from the start of the TAIL launch's own stage range (its value modulo 4 matters)
 #define ADV(sidx) do { if (MODE == MODE_TAIL) ADVANCE4((sidx) & 3); else ADVANCE((sidx) & 1); } while (0)
-#define WFRAG(par, f) (__builtin_bit_cast(s16x8, lds[RING ? 0 : (par)][RING ? 0 : (f) * 64 + lane]))
+#define WFRAG(par, f) (__builtin_bit_cast(s16x8, DMA ? ring[dma_cur * STAGE_U4 + (f) * 64 + lane] : lds[(RING || DMA) ? 0 : (par)][(RING || DMA) ? 0 : (f) * 64 + lane]))
 // all 8 fragments of the current stage -> registers in one burst of LDS reads (one wait instead of 8)
 #define LOAD_STAGE(par, W) s16x8 W[STAGE_FRAGS]; if (RING) ring_take(W); else _Pragma("unroll") for (int f_ = 0; f_ < STAGE_FRAGS; ++f_) W[f_] = WFRAG(par, f_)
 // the same with the slot chosen at run time among the two (a wave-uniform value)
@@ -156,12 +162,13 @@ constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 
 // LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
 // multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
 // and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
-template <typename DT, int KRT, int ACT, int MODE, bool PACK = false, bool RING = false>
+template <typename DT, int KRT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false>
 __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
     static_assert(!RING || MODE == MODE_FULL, "the ring pipeline is the one-launch latency form");
+    static_assert(!DMA || (!RING && MODE != MODE_TAIL), "the paired direct-to-LDS pipeline serves the throughput forms");
     static_assert(KRT == 1 || KRT == 2, "the softmax butterflies pair the row tiles");
-    __shared__ uint4 lds[RING ? 1 : 2][RING ? 64 : STAGE_U4];
+    __shared__ uint4 lds[(RING || DMA) ? 1 : 2][(RING || DMA) ? 64 : STAGE_U4];
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
     // RING: the stage ring sits behind the vectors (1 KB aligned) in the dynamic region
@@ -200,6 +207,23 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         ring_issue(pnext, ring_cur == 0 ? RING_SLOTS - 1 : ring_cur - 1);      // its slot takes the stage RING_DEPTH ahead
         pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
     };
+    // DMA: entry of the next stage (par = its parity in the launch's stage range): on return it is readable in slot
+    // dma_cur.  An even stage admits itself and its successor: this wave's loads of both have landed once at most the
+    // DMA_AHEAD younger stages' are outstanding, the barrier says the same of every wave's and that every wave is done
+    // reading the two stages before; their slots take the next two stages.
+    int dma_cur = DMA_SLOTS - 1;
+    auto dma_advance = [&](int par) __attribute__((always_inline)) {
+        dma_cur = dma_cur + 1 == DMA_SLOTS ? 0 : dma_cur + 1;
+        if (par == 0) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_AHEAD) : "memory");
+            lds_barrier();
+            const int s1 = dma_cur == 0 ? DMA_SLOTS - 1 : dma_cur - 1, s2 = s1 == 0 ? DMA_SLOTS - 1 : s1 - 1;
+            ring_issue(pnext, s2);
+            pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
+            ring_issue(pnext, s1);
+            pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
+        }
+    };
     // RING: the working waves keep the NEXT stage's eight fragments in registers (wnext), fetched from LDS while the
     // current stage is being computed: a lone working wave would otherwise sit out one LDS round trip per stage
     // (~100 stages per forward) with nothing else to run.  ring_take hands out the fragments of the stage about to be
@@ -234,6 +258,15 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         lds_barrier();
         ring_advance();             // the first stage is readable ...
         ring_fetch();               // ... and on its way to registers (every wave: the waves without an env never wait for it)
+    } else if (DMA) {
+        // prologue: DMA_SLOTS - 2 stages in flight (every launch's stage range is longer and even), then the vectors
+        int st = a.s_begin;
+#pragma unroll
+        for (int i = 0; i < DMA_SLOTS - 2; ++i) { ring_issue(st, i); st = st + 1 == a.s_end ? a.s_begin : st + 1; }
+        pnext = st;
+        const int nv4 = vec_floats(a.n_layers, a.F) / 4;
+        for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        lds_barrier();
     } else {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
         const int s0 = a.s_begin;
         const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
@@ -719,7 +752,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             // (vmcnt(0); expcnt / lgkmcnt left at their maxima).  It does not know of the ring's loads, so wherever it
             // later met a value of its own still in flight - or reused such a register - it would wait for "all
             // outstanding loads", i.e. drain the ring in mid-tile; after this it has nothing pending.
-            if (RING) __builtin_amdgcn_s_waitcnt(0x0F70);
+            if (RING || DMA) __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 bp = *reinterpret_cast<const float4*>(vlds + V_BP + 16 * nt + 4 * g);
@@ -837,7 +870,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         const int qi = (int)blockIdx.x - rem_first_wg;
         if (qi >= 0 && qi < rem_passes) pass(std::integral_constant<int, 1>(), rem_tile0 + (int64_t)qi * 4 + wave);
     }
-    if (RING) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
+    if (RING || DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
 }
 
@@ -1084,10 +1117,16 @@ size_t ring_dyn_bytes(int n_layers, int F) {
     return (size_t)((vec_floats(n_layers, F) / 4 + 63) & ~63) * 16 + (size_t)RING_SLOTS * STAGE_U4 * 16;
 }
 
-template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false>
+size_t dma_dyn_bytes(int n_layers, int F) {
+    return (size_t)((vec_floats(n_layers, F) / 4 + 63) & ~63) * 16 + (size_t)DMA_SLOTS * STAGE_U4 * 16;
+}
+// two workgroups share a CU in the throughput forms: both rings must fit
+bool dma_fits(int n_layers, int F) { return 2 * (dma_dyn_bytes(n_layers, F) + 2048) <= LDS_PER_WG; }
+
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false>
 int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
-    const size_t dyn = RING ? ring_dyn_bytes(a.n_layers, a.F) : (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
-    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK, RING>;
+    const size_t dyn = RING ? ring_dyn_bytes(a.n_layers, a.F) : DMA ? dma_dyn_bytes(a.n_layers, a.F) : (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
+    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK, RING, DMA>;
     if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
@@ -1107,9 +1146,10 @@ int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStre
         a.ring_epw = (int)((a.B + cus - 1) / cus);              // 1..4 (B <= 4 CUs): as few working waves per CU as the batch allows
         return launch_one<DT, 1, ACT, MODE_FULL, false, true>(a, cus, st);
     }
+    const bool dma = dma_fits(a.n_layers, a.F);
     if (!pruned) {
         a.s_begin = 0; a.s_end = total;
-        return launch_one<DT, 2, ACT, MODE_FULL>(a, cus, st);
+        return dma ? launch_one<DT, 2, ACT, MODE_FULL, false, false, true>(a, cus, st) : launch_one<DT, 2, ACT, MODE_FULL>(a, cus, st);
     }
     const int split = EMB_STAGES + (a.n_layers - 1) * ls + 3 * H;
     a.s_begin = 0; a.s_end = split;
@@ -1124,9 +1164,9 @@ int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStre
         wgs = (a.B + span - 1) / span;
         hipLaunchKernelGGL(cfg_pair_kernel, dim3((unsigned)wgs), dim3(PAIR_THREADS), 0, st, a.n_valid, a.B, span, per,
                            const_cast<int4*>(a.pairs), const_cast<int32_t*>(a.n_packed));
-        rc = launch_one<DT, 2, ACT, MODE_HEAD, true>(a, cus, st);
+        rc = dma ? launch_one<DT, 2, ACT, MODE_HEAD, true, false, true>(a, cus, st) : launch_one<DT, 2, ACT, MODE_HEAD, true>(a, cus, st);
     } else {
-        rc = launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
+        rc = dma ? launch_one<DT, 2, ACT, MODE_HEAD, false, false, true>(a, cus, st) : launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
     }
     if (rc != BSRL_OK) return rc;
     a.s_begin = split; a.s_end = total;
