@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 10
+ABI_VERSION = 11
 CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
 CFG_NO_LATENCY = 2              # bsrl_cfg_desc.flags: small batches take the throughput forms too
 CFG_STATIC_MAX_ENVS = 16384     # BSRL_CFG_STATIC_MAX_ENVS: batch limit of bsrl_cfg_forward_static
@@ -84,6 +84,7 @@ SIGNATURES = {
     "bsrl_wgrad": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_vres_mix": (_i32, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_hsphere": (_i32, [_i32, _p, _p, C.c_float, _p, _p, _p, _i64, _i64, _i32, _p]),
+    "bsrl_softmax_expect": (_i32, [_p, _p, _p, _i64, _i64, _p]),
 }
 
 _lib = None

@@ -170,7 +170,39 @@ int mix_entry(const char* what, bool relu, const void* v, int64_t ldv, const voi
     return mix_launch<BF16>(m, vec, relu, st);
 }
 
+// softmax(logits) . centers per row: one wave per row, the row's lanes strided over the bins (three passes over
+// registers: max, sum of exponentials, weighted sum)
+__global__ __launch_bounds__(256) void softmax_expect_kernel(const float* __restrict__ logits, const float* __restrict__ centers,
+                                                             float* __restrict__ out, int64_t rows, int n) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* lr = logits + row * n;
+    float m = -INFINITY;
+    for (int i = lane; i < n; i += 64) m = fmaxf(m, lr[i]);
+    m = group_max<64>(m);
+    float se = 0.f, sc = 0.f;
+    for (int i = lane; i < n; i += 64) {
+        const float e = expf(lr[i] - m);
+        se += e; sc = fmaf(e, centers[i], sc);
+    }
+    se = group_sum<64>(se); sc = group_sum<64>(sc);
+    if (lane == 0) out[row] = sc / se;
+}
+
 }  // namespace
+
+extern "C" int bsrl_softmax_expect(const float* logits, const float* centers, float* out, int64_t rows, int64_t n,
+                                   bsrl_stream stream) {
+    if (!logits || !centers || !out) BSRL_FAIL(BSRL_EINVAL, "bsrl_softmax_expect: null pointer");
+    if (rows < 0 || n < 1 || n > 65536) BSRL_FAIL(BSRL_EINVAL, "bsrl_softmax_expect: need rows >= 0 and 1 <= n <= 65536");
+    if (rows == 0) return BSRL_OK;
+    if ((rows + 3) / 4 > 0x7fffffff) BSRL_FAIL(BSRL_EINVAL, "bsrl_softmax_expect: too many rows");
+    hipLaunchKernelGGL(softmax_expect_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       logits, centers, out, rows, (int)n);
+    BSRL_CHECK_LAUNCH("bsrl_softmax_expect");
+    return BSRL_OK;
+}
 
 extern "C" int bsrl_vres_mix(const void* v, int64_t ldv, const void* v0, int64_t ldv0, const float* a, const float* b,
                              void* out, int64_t ldo, int64_t rows, int64_t d, int dtype, bsrl_stream stream) {

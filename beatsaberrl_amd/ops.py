@@ -544,6 +544,24 @@ def relu_bwd(g, y):
 HS_SCALE_L2N, HS_SCALE_RELU, HS_L2N_LERP = 0, 1, 2
 
 
+def softmax_expect(logits, centers):
+    """sum_i softmax(logits)_i * centers_i per row: the HL-Gauss value readout (reference
+    NotePolicy._critic, python/policy.py:1394-1403, `softmax(logits) @ value_centers`).
+    logits (rows, n) fp32, centers (n) fp32 -> (rows,) fp32."""
+    _need_cuda(logits, centers)
+    if logits.dim() != 2 or logits.dtype is not torch.float32 or not logits.is_contiguous():
+        raise TypeError("softmax_expect: logits must be a contiguous fp32 (rows, n) tensor")
+    rows, n = logits.shape
+    if centers.dtype is not torch.float32 or centers.numel() != n or not centers.is_contiguous():
+        raise TypeError(f"softmax_expect: centers must be {n} contiguous fp32 values")
+    out = torch.empty(rows, device=logits.device, dtype=torch.float32)
+    with torch.cuda.device(logits.device):
+        rc = _lib.load().bsrl_softmax_expect(logits.data_ptr(), centers.data_ptr(), out.data_ptr(), rows, n, _stream(logits))
+    if not _lib.check(rc, "bsrl_softmax_expect"):
+        raise Unsupported(f"softmax_expect rows={rows} n={n}")
+    return out
+
+
 def hsphere(op, t, s, c=1.0, x32=None):
     """One fp32 row stage of the SimBaV2 trunk on a GEMM output t (rows, D)
     (reference NotePolicy._trunk_v2, python/policy.py:1140-1155):

@@ -681,7 +681,8 @@ class NotePolicy(nn.Module):
         packed k|v -> 1-query attention pool -> out -> MLP -> HL-Gauss expectation."""
         B, T, d = x_res.shape
         H = self.n_heads
-        if self.critic_pool and not self.rollout_matches_update and ops.critic_pool_supported(T, d, H, x_res.dtype):
+        pooled_route = self.critic_pool and not self.rollout_matches_update and ops.critic_pool_supported(T, d, H, x_res.dtype)
+        if pooled_route:
             # one query per env: the k | v projections commute with the pool, so keys and values are never formed
             wqk, wvo, bvo = self._critic_pool_weights(x_res.dtype)
             q = _lin(self.critic_q, self.critic_ln(x_res[:, 2].contiguous()))          # (B, d), the torso token's query
@@ -702,7 +703,10 @@ class NotePolicy(nn.Module):
         m = self.critic_mlp[4]
         logits = ops.linear(z, _fl._replica(m.weight, z.dtype), _fl._bias32(m.bias), out_dtype=torch.float32)
         self._value_logits = None
-        return torch.softmax(logits, dim=-1) @ self.value_centers
+        if not pooled_route:
+            # the reference's op order: the update path evaluates this very expression, and the two stay bit-equal
+            return torch.softmax(logits, dim=-1) @ self.value_centers
+        return ops.softmax_expect(logits, self.value_centers)
 
     def forward(self, obs):
         logits, value = self.forward_stacked(obs)

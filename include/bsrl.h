@@ -440,6 +440,13 @@ int bsrl_hsphere(int op, const void* t, const float* s, float c,
                  const float* x32_in, float* x32_out, void* x_out,
                  int64_t rows, int64_t D, int dtype, bsrl_stream stream);
 
+/* out[r] = sum_i softmax(logits[r, :])_i * centers[i]: the expectation that ends the HL-Gauss critic,
+ * `torch.softmax(logits, -1) @ self.value_centers` (python/policy.py:1394-1403), as one kernel on the
+ * fp32 bin logits instead of a softmax pass, a gemv and their temporaries.  logits (rows, n) fp32
+ * contiguous, centers (n) fp32, out (rows) fp32; fp32 arithmetic, max-subtracted. */
+int bsrl_softmax_expect(const float* logits, const float* centers, float* out, int64_t rows, int64_t n,
+                        bsrl_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -672,3 +672,26 @@ def test_critic_pool_unsupported_shapes_say_so():
         qk = _rand(2, H, d, dtype=dtype, seed=2)
         with pytest.raises(ops.Unsupported):
             ops.critic_pool(x, _rand(d, seed=3), _rand(d, seed=4), 1e-5, qk, None, H)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 101), (7, 101), (4099, 101), (33, 64), (5, 1), (3, 257)])
+def test_softmax_expect_matches_float64(rows, n):
+    """bsrl_softmax_expect = softmax(logits) @ centers (reference python/policy.py:1394-1403): against the same
+    expression in float64, 2e-6 of the centers' span (fp32 sums of <= 257 terms); rows of huge and of equal logits."""
+    g = torch.Generator().manual_seed(rows * 1000 + n)
+    logits = torch.randn(rows, n, generator=g) * 6.0
+    logits[0] = 0.0                                     # uniform row: the plain mean of the centers
+    if rows > 2:
+        logits[1] += 3.0e4                              # max-subtraction keeps this finite
+        logits[2, n // 2] = 80.0                        # one bin takes everything
+    centers = torch.linspace(-12.5, 37.0, n) if n > 1 else torch.tensor([3.25])
+    want = (torch.softmax(logits.double(), -1) @ centers.double())
+    got = ops.softmax_expect(logits.to(DEV), centers.to(DEV)).cpu()
+    span = float(centers.max() - centers.min()) + float(centers.abs().max())
+    assert got.shape == (rows,) and got.dtype is torch.float32
+    assert (got.double() - want).abs().max().item() <= 2e-6 * span
+    assert abs(got[0].item() - centers.double().mean().item()) <= 2e-6 * span
+    with pytest.raises(TypeError):
+        ops.softmax_expect(logits.to(DEV).half(), centers.to(DEV))
+    with pytest.raises(TypeError):
+        ops.softmax_expect(logits.to(DEV), centers[:-1].to(DEV) if n > 1 else torch.zeros(2, device=DEV))
