@@ -625,11 +625,10 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
             uint2 q[2][2][TPH];                                // Q fragments [head parity][row tile][feature tile]
             uint2 kk[2][TPH], vv[2][TPH];                      // K, V^T fragments of the head in flight [key tile][feature tile]
 
-            // attention of head hd: the env's (up to) 32 queries over its 32 key slots, one query tile after the other
-            // (the row maximum and the row sum each ride a lane-row swap butterfly beside a copy of themselves: the
-            // joint form for both tiles keeps 8 more values live where the registers are scarcest)
+            // attention of head hd: the env's (up to) 32 queries over its 32 key slots, both query tiles together
             auto attention = [&](auto hd_) __attribute__((always_inline)) {
                 constexpr int hd = decltype(hd_)::value;
+                float sv[2][2][4], m[2], sum[2];
 #pragma unroll
                 for (int qt = 0; qt < QT; ++qt) {
                     f32x4 sc[2];
@@ -649,27 +648,32 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
                             for (int i = 0; i < 4; ++i) sc[kt][i] += s2[i];
                         }
                     }
-                    float sv[2][4];
-                    float m = -INFINITY;
+                    m[qt] = -INFINITY;
 #pragma unroll
                     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) { sv[kt][i] = fmaf(sc[kt][i], scale_l2e, kmask[kt][i]); m = fmaxf(m, sv[kt][i]); }
-                    float m2 = m;
-                    rows_reduce2(m, m2, OpMax());
-                    float sum = 0.f;
+                        for (int i = 0; i < 4; ++i) { sv[qt][kt][i] = fmaf(sc[kt][i], scale_l2e, kmask[kt][i]); m[qt] = fmaxf(m[qt], sv[qt][kt][i]); }
+                }
+                if (QT == 1) m[1] = m[0];
+                rows_reduce2(m[0], m[1], OpMax());
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) {
+                    sum[qt] = 0.f;
 #pragma unroll
                     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) { sv[kt][i] = __builtin_amdgcn_exp2f(sv[kt][i] - m); sum += sv[kt][i]; }
-                    float sum2 = sum;
-                    rows_reduce2(sum, sum2, OpAdd());
-                    const float inv = __builtin_amdgcn_rcpf(sum);
+                        for (int i = 0; i < 4; ++i) { sv[qt][kt][i] = __builtin_amdgcn_exp2f(sv[qt][kt][i] - m[qt]); sum[qt] += sv[qt][kt][i]; }
+                }
+                if (QT == 1) sum[1] = sum[0];
+                rows_reduce2(sum[0], sum[1], OpAdd());
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) {
+                    const float inv = __builtin_amdgcn_rcpf(sum[qt]);
                     BFrag8 pf;
 #pragma unroll
                     for (int kt = 0; kt < 2; ++kt) {
-                        pf.w[2 * kt] = bpack2<DT>(sv[kt][0] * inv, sv[kt][1] * inv);
-                        pf.w[2 * kt + 1] = bpack2<DT>(sv[kt][2] * inv, sv[kt][3] * inv);
+                        pf.w[2 * kt] = bpack2<DT>(sv[qt][kt][0] * inv, sv[qt][kt][1] * inv);
+                        pf.w[2 * kt + 1] = bpack2<DT>(sv[qt][kt][2] * inv, sv[qt][kt][3] * inv);
                     }
 #pragma unroll
                     for (int t = 0; t < TPH; ++t) {
@@ -696,39 +700,41 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
                     constexpr int done_prev = (2 * st - 2) / (3 * TPH);
                     if constexpr (done > done_prev) attention(std::integral_constant<int, done - 1>{});
                 }
-                // one feature tile at a time (its sub-bursts over all k chunks, then the other tile's): one accumulator
-                // pair is live, and a tile is packed away before the next one starts
-                static_for<0, 2>([&](auto ntl_) __attribute__((always_inline)) {
-                    constexpr int ntl = decltype(ntl_)::value;
-                    constexpr int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
-                    f32x4 acc[2];                                // [row tile]
+                f32x4 acc[2][2];                                 // [tile of the stage][row tile]
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
                     float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
                     if (part < 2) b = *reinterpret_cast<const float4*>(lv + (part == 0 ? G::BQ : G::BK) + DH * hd + 16 * t + 4 * g);
-                    acc[0] = (f32x4){b.x, b.y, b.z, b.w}; acc[1] = acc[0];
-                    static_for<0, NB>([&](auto half_) __attribute__((always_inline)) {
-                        constexpr int half = decltype(half_)::value;          // k chunks [half * KB, +KB)
-                        sub(std::integral_constant<int, 2 * half + ntl>{}, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
+                    acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
+                }
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;    // k chunks [half * KB, +KB) of tile ntl
+                    sub(j_, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
 #pragma unroll
-                            for (int ci = 0; ci < KB; ++ci)
+                        for (int ci = 0; ci < KB; ++ci)
 #pragma unroll
-                                for (int rt = 0; rt < 2; ++rt) {
-                                    const int c = half * KB + ci;
-                                    if (part == 0 && rt >= QT) continue;     // the pruned block needs no queries from row tile 1
-                                    if (part < 2) acc[rt] = DT::mfma32(wf[ci], hf[rt][c].v, acc[rt]);
-                                    else acc[rt] = DT::mfma32(hf[rt][c].v, wf[ci], acc[rt]);   // V^T: operand roles swapped
-                                }
-                        });
+                            for (int rt = 0; rt < 2; ++rt) {
+                                const int c = half * KB + ci;
+                                const int j = 2 * st + ntl, part = (j % (3 * TPH)) / TPH;
+                                if (part == 0 && rt >= QT) continue;     // the pruned block needs no queries from row tile 1
+                                if (part < 2) acc[ntl][rt] = DT::mfma32(wf[ci], hf[rt][c].v, acc[ntl][rt]);
+                                else acc[ntl][rt] = DT::mfma32(hf[rt][c].v, wf[ci], acc[ntl][rt]);   // V^T: operand roles swapped
+                            }
                     });
+                });
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl)
 #pragma unroll
                     for (int rt = 0; rt < 2; ++rt) {
+                        const int j = 2 * st + ntl, hd = j / (3 * TPH), r = j % (3 * TPH), part = r / TPH, t = r % TPH;
                         if (part == 0 && rt >= QT) continue;
                         uint2 pk;
-                        pk.x = bpack2<DT>(acc[rt][0], acc[rt][1]); pk.y = bpack2<DT>(acc[rt][2], acc[rt][3]);
+                        pk.x = bpack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]); pk.y = bpack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
                         if (part == 0) q[hd & 1][rt][t] = pk;
                         else if (part == 1) kk[rt][t] = pk;
                         else vv[rt][t] = pk;
                     }
-                });
             });
 
             // ---- output projection onto the residual (NT / 2 stages) ----
