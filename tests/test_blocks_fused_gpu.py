@@ -144,6 +144,39 @@ def test_large_batches_take_the_env_per_wave_kernel_and_give_the_same_bits(dtype
     assert torch.isfinite(big.float()).all()
 
 
+def test_env_per_wave_kernel_replays_from_a_captured_graph():
+    """The large-batch kernel inside a captured graph: three replays, with eager launches of both kernels and
+    synchronisations between them, all bit-equal to the eager result."""
+    d, L, B, T, F, nq = 192, 2, 1500, 26, 768, 6
+    sd = _weights(L, d, F, 91)
+    x, bias = _inputs(B, T, d, 17)
+    tdt, H = TDT["f16"], _heads(d)
+    image = torch.empty(ops.blocks_pack_size(L, d, H, F, T, "relu", nq, tdt), dtype=torch.uint8, device=DEV)
+    params = [[sd[f"blocks.{i}.{f}"].to(DEV).contiguous() for f in FIELDS] for i in range(L)]
+    ops.blocks_pack(params, image, d, H, F, T, "relu", nq, tdt)
+    xd, bd = x.to(DEV).to(tdt).contiguous(), bias.to(DEV).to(tdt).contiguous()
+    fn = lambda: ops.blocks_forward(image, xd, bd, L, H, F, "relu", nq)
+    want, want_res = fn()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got, got_res = fn()
+    for i in range(3):
+        got.zero_(); got_res.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_res, want_res), i
+        small, _ = ops.blocks_forward(image, xd[:300], bd[:300], L, H, F, "relu", nq)       # the wave-pair kernel, eager
+        assert torch.equal(small, want[:300])
+        again, _ = fn()
+        assert torch.equal(again, want)
+
+
 def test_env_per_wave_kernel_matches_oracle():
     """One direct oracle case for the large-batch kernel (its bits equal the wave-pair kernel's, which the cases above
     pin; this one guards the equality test's own premise).  Ceilings: the batch maxima measured on this seeded case
