@@ -292,7 +292,12 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     // One pass of this wave over the weight stream with RT row tiles.  A generic lambda so that the packed first launch
     // can hold two bodies: two row tiles per wave for the bulk, ONE for the remainder tiles of the last round (below).
     // env0: the wave's first env (or first tile, PACK).
-    auto pass = [&](auto rt_tag, const int64_t env0) __attribute__((always_inline)) {
+    // PACK: the table entries of the wave's NEXT pass ride along with this pass's own input loads (one wait for both) and
+    // stay in scalar registers, so that a pass starts its key-count and observation loads without first waiting for
+    // its table entries (one L2 round trip per pass).  next0 < 0: no next pass of the bulk body.
+    int pre_pr[PACK ? KRT : 1][4];
+    bool have_pre = false;
+    auto pass = [&](auto rt_tag, const int64_t env0, const int64_t next0) __attribute__((always_inline)) {
         constexpr int RT = decltype(rt_tag)::value;
         // every lambda below is force-inlined: one left out of line would take the residual registers by reference,
         // i.e. through scratch memory (seen with the bf16 instantiations, whose pack helper is larger)
@@ -669,10 +674,15 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 if (PACK) {
-                    int64_t tix = env0 + rt; tix = tix < n_units ? tix : n_units - 1;
-                    const int4 pr = a.pairs[tix];
-                    const int e0 = __builtin_amdgcn_readfirstlane(pr.x), e1 = __builtin_amdgcn_readfirstlane(pr.y);
-                    const int e2 = __builtin_amdgcn_readfirstlane(pr.z), e3 = __builtin_amdgcn_readfirstlane(pr.w);
+                    int e0, e1, e2, e3;
+                    if (RT == KRT && have_pre) {
+                        e0 = pre_pr[PACK ? rt : 0][0]; e1 = pre_pr[PACK ? rt : 0][1]; e2 = pre_pr[PACK ? rt : 0][2]; e3 = pre_pr[PACK ? rt : 0][3];
+                    } else {
+                        int64_t tix = env0 + rt; tix = tix < n_units ? tix : n_units - 1;
+                        const int4 pr = a.pairs[tix];
+                        e0 = __builtin_amdgcn_readfirstlane(pr.x); e1 = __builtin_amdgcn_readfirstlane(pr.y);
+                        e2 = __builtin_amdgcn_readfirstlane(pr.z); e3 = __builtin_amdgcn_readfirstlane(pr.w);
+                    }
                     // the slot (rows 4 s .. 4 s + 3) an env starts in, for this lane's row and for its 4 keys (one slot)
                     auto owner = [&](int sl) __attribute__((always_inline)) {
                         int o = 0;
@@ -694,6 +704,14 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                     const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
+                }
+            }
+            int4 nxt[PACK ? RT : 1];
+            if (PACK && RT == KRT && next0 >= 0) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    int64_t tix = next0 + rt; tix = tix < n_units ? tix : n_units - 1;
+                    nxt[PACK ? rt : 0] = a.pairs[tix];
                 }
             }
             if (a.tok_vec) {
@@ -753,6 +771,18 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             // later met a value of its own still in flight - or reused such a register - it would wait for "all
             // outstanding loads", i.e. drain the ring in mid-tile; after this it has nothing pending.
             if (RING || DMA) __builtin_amdgcn_s_waitcnt(0x0F70);
+            if (PACK && RT == KRT) {
+                have_pre = next0 >= 0;
+                if (have_pre) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        pre_pr[PACK ? rt : 0][0] = __builtin_amdgcn_readfirstlane(nxt[PACK ? rt : 0].x);
+                        pre_pr[PACK ? rt : 0][1] = __builtin_amdgcn_readfirstlane(nxt[PACK ? rt : 0].y);
+                        pre_pr[PACK ? rt : 0][2] = __builtin_amdgcn_readfirstlane(nxt[PACK ? rt : 0].z);
+                        pre_pr[PACK ? rt : 0][3] = __builtin_amdgcn_readfirstlane(nxt[PACK ? rt : 0].w);
+                    }
+                }
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const float4 bp = *reinterpret_cast<const float4*>(vlds + V_BP + 16 * nt + 4 * g);
@@ -864,11 +894,12 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
             continue;
         }
-        pass(rt_bulk(), env0);
+        const int64_t ntile = tile + gridDim.x;
+        pass(rt_bulk(), env0, (PACK && ntile < n_bulk) ? ntile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE : -1);
     }
     if (PACK && KRT == 2) {
         const int qi = (int)blockIdx.x - rem_first_wg;
-        if (qi >= 0 && qi < rem_passes) pass(std::integral_constant<int, 1>(), rem_tile0 + (int64_t)qi * 4 + wave);
+        if (qi >= 0 && qi < rem_passes) pass(std::integral_constant<int, 1>(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
     }
     if (RING || DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
