@@ -948,7 +948,322 @@ int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
     return BSRL_OK;
 }
 
+// ---- the FFN half of a block as a kernel of its own: xo = x + act(h2 W0^T + b0) W2^T + b2 (+ LayerNorm) ------------
+// The FFN phase of blocks_env_kernel on plain rows: a wave owns 32 rows (two 16-row tiles; fp32 accumulator and the
+// LayerNorm-ed input as operand fragments in registers), a workgroup is 8 waves = 256 rows, one workgroup per CU; the
+// weight chunks stream through the same direct-to-LDS ring from a pre-permuted image (stage order W1(0), {W1(ch+1),
+// W2(ch)}..., W2(last), admitted in pairs), every fragment feeds both row tiles, the 32-unit hidden chunk lives in
+// accumulators and goes into the down-projection as one operand fragment.  Rounding points are those of the
+// reference's fused kernel (python/beat_arena_env/csrc/fused_ffn.cu:551-619): hidden rounded once, fp32 accumulate,
+// xo rounded once, LayerNorm statistics on the ROUNDED xo, ho rounded once.
+struct FfnArgs {
+    const uint2* frags; const float* vec;        // image: 2 * F / 32 stages, then b0 (F) | b2 (d) fp32
+    const u16* x; const u16* h2; u16* xo; u16* ho;
+    const float* ln_w; const float* ln_b; float eps;
+    int64_t rows; int F, total_stages;
+};
+
+template <int D> struct FfnRing {
+    static constexpr int NW = 8;
+    static constexpr int SLOTS = D == 128 ? 10 : D == 192 ? 7 : 6;
+    static constexpr int AHEAD = SLOTS - 4;
+    static constexpr int STAGE_BYTES = Geo<D>::SF * 1024;
+    static constexpr int LPW_HI = (Geo<D>::SF + NW - 1) / NW, N_HI = Geo<D>::SF - (LPW_HI - 1) * NW;
+    static_assert(SLOTS >= 5 && LPW_HI * (AHEAD + 2) < 64, "vmcnt is 6 bits");
+};
+
+template <typename DT, int D, int ACT, bool LN>
+__global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
+    typedef Geo<D> G;
+    typedef FfnRing<D> R;
+    constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, SF = G::SF, NSUB = 2 * NB;
+    extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
+    float* vlds = reinterpret_cast<float*>(bvl4);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int nvec = a.F + 3 * D;
+    const int ring_off_u4 = (nvec / 4 + 63) & ~63;
+    const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
+    const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
+    const char* img = reinterpret_cast<const char*>(a.frags);
+    const float* B1 = vlds; const float* B2 = vlds + a.F; const float* LNG = B2 + D; const float* LNB = LNG + D;
+    const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
+
+    int cur = R::SLOTS - 1, pnext;
+    auto issue = [&](int stage, int slot) __attribute__((always_inline)) {
+        const char* sb = img + (int64_t)stage * R::STAGE_BYTES;
+        const uint32_t dst = ring_base + slot * R::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < R::LPW_HI; ++i)
+            if (i + 1 < R::LPW_HI || wave < R::N_HI) env_ring_load(lane * 16, sb + (wave + NW * i) * 1024, dst + (wave + NW * i) * 1024);
+    };
+    auto advance = [&](auto parity_) __attribute__((always_inline)) {
+        cur = cur + 1 == R::SLOTS ? 0 : cur + 1;
+        if constexpr (decltype(parity_)::value == 0) {
+            if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
+            blk_barrier();
+            const int s1 = cur == 0 ? R::SLOTS - 1 : cur - 1, s2 = s1 == 0 ? R::SLOTS - 1 : s1 - 1;
+            issue(pnext, s2);
+            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+            issue(pnext, s1);
+            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
+        }
+    };
+    typedef std::integral_constant<int, 0> Even;
+    typedef std::integral_constant<int, 1> Odd;
+    auto sub = [&](auto j_, auto&& body) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_)::value;
+        s16x8 w[KB];
+#pragma unroll
+        for (int f = 0; f < KB; ++f) w[f] = __builtin_bit_cast(s16x8, ring[cur * (SF * 64) + (j * KB + f) * 64 + lane]);
+        body(w);
+    };
+    {   // prologue: SLOTS - 2 stages in flight (the host checks that the image is longer), then the vectors
+        int st = 0;
+#pragma unroll
+        for (int i = 0; i < R::SLOTS - 2; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
+        pnext = st;
+        for (int i = tid; i < a.F + D; i += NW * 64) vlds[i] = a.vec[i];
+        if (LN) for (int i = tid; i < D; i += NW * 64) { vlds[a.F + D + i] = a.ln_w[i]; vlds[a.F + 2 * D + i] = a.ln_b[i]; }
+        blk_barrier();
+    }
+
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t row0 = (tile * NW + wave) * 32;
+        f32x4 x[2][NT];
+        BFrag8 hf[2][KC];
+        {   // the tile's own loads: all issued, one wait the compiler can see (it does not know of the ring's transfers)
+            uint2 rx[2][NT], rh[2][NT];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
+                const u16* xr = a.x + row * D; const u16* hr = a.h2 + row * D;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    rx[rt][nt] = *reinterpret_cast<const uint2*>(xr + 16 * nt + 4 * g);
+                    rh[rt][nt] = *reinterpret_cast<const uint2*>(hr + 16 * nt + 4 * g);
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4 b = *reinterpret_cast<const float4*>(B2 + 16 * nt + 4 * g);
+                    x[rt][nt][0] = DT::to_f((u16)(rx[rt][nt].x & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(rx[rt][nt].x >> 16)) + b.y;
+                    x[rt][nt][2] = DT::to_f((u16)(rx[rt][nt].y & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(rx[rt][nt].y >> 16)) + b.w;
+                    hf[rt][nt >> 1].h[nt & 1] = rh[rt][nt];       // a lane's 4 features of tile nt are half of chunk nt / 2's operand fragment
+                }
+        }
+        const int nch = a.F / 32;
+        f32x4 acc[2][2];                                     // [tile of the chunk][row tile]
+        auto up = [&](int ch) __attribute__((always_inline)) {
+#pragma unroll
+            for (int ntl = 0; ntl < 2; ++ntl) {
+                const float4 b = *reinterpret_cast<const float4*>(B1 + 32 * ch + 16 * ntl + 4 * g);
+                acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
+            }
+            static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                constexpr int half = decltype(j_)::value / 2, ntl = decltype(j_)::value % 2;
+                sub(j_, [&](const s16x8 (&wf)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int ci = 0; ci < KB; ++ci)
+#pragma unroll
+                        for (int rt = 0; rt < 2; ++rt)
+                            acc[ntl][rt] = DT::mfma32(wf[ci], hf[rt][half * KB + ci].v, acc[ntl][rt]);
+                });
+            });
+        };
+        advance(Even{});
+        up(0);
+        for (int ch = 0; ch < nch; ++ch) {
+            BFrag8 hid[2];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                for (int ntl = 0; ntl < 2; ++ntl) {
+                    hid[rt].w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
+                    hid[rt].w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
+                }
+            // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
+            if (ch + 1 < nch) { advance(Odd{}); up(ch + 1); advance(Even{}); }
+            else advance(Odd{});
+            static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                constexpr int j = decltype(j_)::value;           // feature tiles [j * KB, +KB)
+                sub(j_, [&](const s16x8 (&w2)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int i = 0; i < KB; ++i)
+#pragma unroll
+                        for (int rt = 0; rt < 2; ++rt) x[rt][j * KB + i] = DT::mfma32(w2[i], hid[rt].v, x[rt][j * KB + i]);
+                });
+            });
+        }
+        // epilogue: round, store, optional LayerNorm on the rounded row
+        float s[2] = {0.f, 0.f}, q[2] = {0.f, 0.f};
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int64_t row = row0 + 16 * rt + r16;
+            u16* o = a.xo + row * D;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                uint2 v;
+                v.x = bpack2<DT>(x[rt][nt][0], x[rt][nt][1]); v.y = bpack2<DT>(x[rt][nt][2], x[rt][nt][3]);
+                if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                if (LN) {
+                    x[rt][nt][0] = DT::to_f((u16)(v.x & 0xffff)); x[rt][nt][1] = DT::to_f((u16)(v.x >> 16));
+                    x[rt][nt][2] = DT::to_f((u16)(v.y & 0xffff)); x[rt][nt][3] = DT::to_f((u16)(v.y >> 16));
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { s[rt] += x[rt][nt][i]; q[rt] = fmaf(x[rt][nt][i], x[rt][nt][i], q[rt]); }
+                }
+            }
+        }
+        if (LN) {
+            rows_reduce2(s[0], q[0], OpAdd());
+            rows_reduce2(s[1], q[1], OpAdd());
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                const int64_t row = row0 + 16 * rt + r16;
+                u16* o = a.ho + row * D;
+                // one pass: var = E[x^2] - mean^2 clamped at 0 (python/beat_arena_env/csrc/layer_norm.cu:14-21)
+                const float mean = s[rt] * (1.0f / D);
+                const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q[rt] * (1.0f / D)), 0.f) + a.eps);
+                const float shift = -mean * rstd;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4 gm = *reinterpret_cast<const float4*>(LNG + 16 * nt + 4 * g);
+                    const float4 bt = *reinterpret_cast<const float4*>(LNB + 16 * nt + 4 * g);
+                    uint2 v;
+                    v.x = bpack2<DT>(fmaf(fmaf(x[rt][nt][0], rstd, shift), gm.x, bt.x), fmaf(fmaf(x[rt][nt][1], rstd, shift), gm.y, bt.y));
+                    v.y = bpack2<DT>(fmaf(fmaf(x[rt][nt][2], rstd, shift), gm.z, bt.z), fmaf(fmaf(x[rt][nt][3], rstd, shift), gm.w, bt.w));
+                    if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                }
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
+    blk_barrier();
+}
+
+struct FfnPackArgs { const u16* w0; const float* b0; const u16* w2; const float* b2; void* frags; float* vec; int F; };
+// fragments of the 2 * F / 32 FFN stages from the 16-bit weights (a copy in fragment order, no rounding); one wave
+// per fragment, one lane per 16-byte slot
+template <int D>
+__global__ __launch_bounds__(256) void ffn_pack_frags_kernel(FfnPackArgs a) {
+    typedef Geo<D> G;
+    constexpr int SF = G::SF;
+    const int lane = threadIdx.x & 63, n16 = lane & 15, gg = lane >> 4;
+    const int nch = a.F / 32;
+    const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= 2 * nch * SF) return;
+    const int s3 = f / SF, i = f % SF;
+    bool upw; int ch;
+    if (s3 == 0) { upw = true; ch = 0; }
+    else if (s3 == 2 * nch - 1) { upw = false; ch = nch - 1; }
+    else { upw = ((s3 - 1) & 1) == 0; ch = (s3 - 1) / 2 + (upw ? 1 : 0); }
+    const u16* src; int ld, n, kbase = 0, c = 0;
+    if (upw) {
+        const int burst = i / G::FB, rem = i % G::FB, ntl = rem / G::KB;
+        c = burst * G::KB + rem % G::KB;
+        src = a.w0; ld = D; n = 32 * ch + 16 * ntl + n16;
+    } else { src = a.w2; ld = a.F; n = 16 * i + n16; kbase = 32 * ch; }
+    u16 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + bperm_k(c, gg, j)];
+    uint4 o;
+    o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+    o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+    static_cast<uint4*>(a.frags)[(int64_t)f * 64 + lane] = o;
+    if (f == 0) for (int k = lane; k < a.F + D; k += 64) a.vec[k] = k < a.F ? a.b0[k] : a.b2[k - a.F];
+}
+
+bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
+    if (d != 128 && d != 192 && d != 256) return false;
+    if (F < 64 || F % 32 != 0 || F > 16384 || (dtype != BSRL_F16 && dtype != BSRL_BF16)) return false;
+    const int slots = d == 128 ? 10 : d == 192 ? 7 : 6;
+    return 2 * (F / 32) >= slots;
+}
+int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
+template <int D> size_t ffn_dyn_bytes(int F) {
+    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D>::SLOTS * FfnRing<D>::STAGE_BYTES;
+}
+template <typename DT, int D, int ACT>
+int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
+    const size_t dyn = ffn_dyn_bytes<D>(a.F);
+    if (dyn + 1024 > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
+    const int64_t ntiles = (a.rows + 255) / 256;
+    const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));
+    auto launch = [&](auto kern) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+            return (int)BSRL_UNSUPPORTED;
+        hipLaunchKernelGGL(kern, grid, dim3(512), dyn, st, a);
+        return (int)BSRL_OK;
+    };
+    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true>) : launch(ffn_rows_kernel<DT, D, ACT, false>);
+}
+
 }  // namespace
+
+extern "C" int64_t bsrl_ffn_pack_size(int64_t d, int64_t F, int dtype) {
+    if (!ffn_packed_shape_ok(d, F, dtype)) return 0;
+    return ffn_frag_bytes(d, F) + (F + d) * 4;
+}
+
+extern "C" int bsrl_ffn_pack(const void* w0, const float* b0, const void* w2, const float* b2, int64_t d, int64_t F,
+                             int dtype, void* image, bsrl_stream stream) {
+    if (!w0 || !b0 || !w2 || !b2 || !image) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_pack: null pointer");
+    if (!ffn_packed_shape_ok(d, F, dtype)) return BSRL_UNSUPPORTED;
+    if (!bsrl_aligned(image, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_pack: image must be 16-byte aligned");
+    FfnPackArgs pa{static_cast<const u16*>(w0), b0, static_cast<const u16*>(w2), b2, image,
+                   reinterpret_cast<float*>(static_cast<char*>(image) + ffn_frag_bytes(d, F)), (int)F};
+    const int64_t nfrags = 2 * (F / 32) * (d / 16);
+    const dim3 grid((unsigned)((nfrags + 3) / 4));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (d == 128) hipLaunchKernelGGL(ffn_pack_frags_kernel<128>, grid, dim3(256), 0, st, pa);
+    else if (d == 192) hipLaunchKernelGGL(ffn_pack_frags_kernel<192>, grid, dim3(256), 0, st, pa);
+    else hipLaunchKernelGGL(ffn_pack_frags_kernel<256>, grid, dim3(256), 0, st, pa);
+    BSRL_CHECK_LAUNCH("bsrl_ffn_pack");
+    return BSRL_OK;
+}
+
+extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const float* ln_w, const float* ln_b,
+                               float eps, void* xo, void* ho, int64_t rows, int64_t d, int64_t F, int act, int dtype,
+                               bsrl_stream stream) {
+    if (!image || !x || !h2 || !xo) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: null pointer");
+    if ((ln_w == nullptr) != (ho == nullptr) || (ln_w == nullptr) != (ln_b == nullptr))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: ln_w, ln_b and ho go together");
+    if (!ffn_packed_shape_ok(d, F, dtype) || (act != BSRL_ACT_RELU && act != BSRL_ACT_GELU)) return BSRL_UNSUPPORTED;
+    if (rows < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: rows < 0");
+    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(h2, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: image must be 16-byte, rows 8-byte aligned");
+    if (rows == 0) return BSRL_OK;
+    FfnArgs a;
+    a.frags = static_cast<const uint2*>(image);
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + ffn_frag_bytes(d, F));
+    a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(h2);
+    a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho);
+    a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F; a.total_stages = (int)(2 * (F / 32));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    const bool relu = act == BSRL_ACT_RELU, f16 = dtype == BSRL_F16, ln = ln_w != nullptr;
+    int rc;
+    if (d == 128) {
+        if (f16) rc = relu ? ffn_launch<F16, 128, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 128, BSRL_ACT_GELU>(a, ln, cus, st);
+        else rc = relu ? ffn_launch<BF16, 128, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 128, BSRL_ACT_GELU>(a, ln, cus, st);
+    } else if (d == 192) {
+        if (f16) rc = relu ? ffn_launch<F16, 192, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 192, BSRL_ACT_GELU>(a, ln, cus, st);
+        else rc = relu ? ffn_launch<BF16, 192, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 192, BSRL_ACT_GELU>(a, ln, cus, st);
+    } else {
+        if (f16) rc = relu ? ffn_launch<F16, 256, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 256, BSRL_ACT_GELU>(a, ln, cus, st);
+        else rc = relu ? ffn_launch<BF16, 256, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 256, BSRL_ACT_GELU>(a, ln, cus, st);
+    }
+    if (rc != BSRL_OK) return rc;
+    BSRL_CHECK_LAUNCH("bsrl_ffn_packed");
+    return BSRL_OK;
+}
 
 extern "C" int64_t bsrl_blocks_pack_size(const bsrl_blocks_desc* d) {
     if (!blocks_shape_ok(d)) return 0;

@@ -355,12 +355,51 @@ def ffn_fused_profitable(d, F, dtype) -> bool:
     0.54 + 0.09 (streaming / ring-buffered linears); d = 256: 4.0 vs 2.7 at 3.1M rows; d = 384: 44 vs 16.5 - past
     d = 128 the per-workgroup row tile that fits in registers is too small for the weight stream, so the unfused
     pair (hidden through HBM) wins."""
+    if ffn_pack_supported(d, F, dtype):
+        return True          # the packed-image kernel: 0.33 ms at d = 192 (F = 768), 0.2 ms at d = 128 for the same rows
     return d <= 128 and ffn_fused_supported(d, F, dtype)
 
 
-def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5):
+def ffn_pack_supported(d, F, dtype) -> bool:
+    return dtype in (torch.float16, torch.bfloat16) and _lib.load().bsrl_ffn_pack_size(d, F, dt_code(dtype)) > 0
+
+
+# weight images of ffn_fused's packed route, keyed by the identity and in-place version of the four tensors (the
+# 16-bit replicas are rewritten or replaced after every optimizer step: either changes the key); a few entries only
+_FFN_IMAGES: dict = {}
+_FFN_IMAGES_MAX = 64
+
+
+def ffn_pack(w0, b0, w2, b2):
+    """Weight image of the packed fused FFN (bsrl_ffn_pack) from w0 (F, d), w2 (d, F) in a 16-bit dtype and the fp32
+    biases; cached while the four tensors are unchanged."""
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) for t in (w0, b0, w2, b2))
+    img = _FFN_IMAGES.get(key)
+    if img is not None:
+        return img
+    Fh, d = w0.shape
+    n = _lib.load().bsrl_ffn_pack_size(d, Fh, dt_code(w0.dtype))
+    if n <= 0:
+        raise Unsupported(f"ffn_pack d={d} F={Fh} dtype={w0.dtype}")
+    img = torch.empty(n, dtype=torch.uint8, device=w0.device)
+    with torch.cuda.device(w0.device):
+        rc = _lib.load().bsrl_ffn_pack(w0.data_ptr(), _f32c(b0, "b0").data_ptr(), w2.data_ptr(), _f32c(b2, "b2").data_ptr(),
+                                       d, Fh, dt_code(w0.dtype), img.data_ptr(), _stream(w0))
+    if not _lib.check(rc, "bsrl_ffn_pack"):
+        raise Unsupported(f"ffn_pack d={d} F={Fh} dtype={w0.dtype}")
+    if len(_FFN_IMAGES) >= _FFN_IMAGES_MAX:
+        _FFN_IMAGES.clear()
+    # the key's data pointers stay valid only while the tensors live: hold them with the image
+    _FFN_IMAGES[key] = img
+    img._bsrl_sources = (w0, b0, w2, b2)
+    return img
+
+
+def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5, packed="auto"):
     """xo = x + act(h2 w0^T + b0) w2^T + b2; ho = LN(xo) when ln_w is given.
-    Returns (xo, ho) (ho None without LN), or None when unsupported."""
+    Returns (xo, ho) (ho None without LN), or None when unsupported.
+    packed: "auto" takes the packed-image kernel (bsrl_ffn_packed: d <= 256, weights streamed straight into LDS,
+    32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter."""
     _need_cuda(x, h2, w0, w2)
     d = x.shape[-1]
     Fh = w0.shape[0]
@@ -375,6 +414,15 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5)
     rows = x.numel() // d
     xo = torch.empty_like(x)
     ho = torch.empty_like(x) if ln_w is not None else None
+    if packed and ffn_pack_supported(d, Fh, x.dtype):
+        img = ffn_pack(w0, _f32c(b0, "b0"), w2, _f32c(b2, "b2"))
+        with torch.cuda.device(x.device):
+            rc = _lib.load().bsrl_ffn_packed(img.data_ptr(), x.data_ptr(), h2.data_ptr(), _ptr(_f32c(ln_w, "ln_w")),
+                                             _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), rows, d, Fh,
+                                             _ACT[act], dt_code(x.dtype), _stream(x))
+        if not _lib.check(rc, "bsrl_ffn_packed"):
+            return None
+        return xo, ho
     with torch.cuda.device(x.device):
         rc = _lib.load().bsrl_ffn_fused(x.data_ptr(), h2.data_ptr(), w0.data_ptr(), _f32c(b0, "b0").data_ptr(),
                                         w2.data_ptr(), _f32c(b2, "b2").data_ptr(), _ptr(_f32c(ln_w, "ln_w")),

@@ -217,17 +217,20 @@ def test_linear_rows_are_batch_invariant():
 @pytest.mark.parametrize("rows,d,Fh", [(1, 128, 512), (127, 128, 512), (129, 192, 768), (1000, 192, 768),
                                        (300, 256, 1024), (77, 384, 1536), (513, 128, 64)])
 @pytest.mark.parametrize("act,with_ln", [("relu", True), ("gelu", False), ("gelu", True)])
-def test_ffn_fused(dtype, rows, d, Fh, act, with_ln):
+@pytest.mark.parametrize("packed", ["auto", False])
+def test_ffn_fused(dtype, rows, d, Fh, act, with_ln, packed):
     """Closed form with the reference's rounding points (python/tests/test_fused_ffn.py:252-266):
-    hidden rounded once, fp32 accumulate, out = round(x + (O + b2)), LN on the rounded out."""
+    hidden rounded once, fp32 accumulate, out = round(x + (O + b2)), LN on the rounded out.  Both kernels: the one on
+    a packed weight image (d <= 256 with enough FFN stages; `packed="auto"`) and the one on the plain weights."""
     assert ops.ffn_fused_supported(d, Fh, dtype)
+    assert ops.ffn_pack_supported(d, Fh, dtype) == (d <= 256 and Fh >= 192)
     x = _rand(rows, d, dtype=dtype, seed=1)
     h2 = _rand(rows, d, dtype=dtype, seed=2)
     w0 = _rand(Fh, d, dtype=dtype, seed=3, scale=1 / math.sqrt(d))
     w2 = _rand(d, Fh, dtype=dtype, seed=4, scale=1 / math.sqrt(Fh))
     b0, b2 = _rand(Fh, seed=5) * 0.3, _rand(d, seed=6) * 0.3
     lw, lb = (_rand(d, seed=7) * 0.2 + 1.0, _rand(d, seed=8) * 0.2) if with_ln else (None, None)
-    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act=act, ln_w=lw, ln_b=lb)
+    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act=act, ln_w=lw, ln_b=lb, packed=packed)
     pre = h2.double() @ w0.double().t() + b0.double()
     hid = (torch.relu(pre) if act == "relu" else 0.5 * pre * (1 + torch.erf(pre / math.sqrt(2.0)))).to(dtype).double()
     ref = x.double() + hid @ w2.double().t() + b2.double()
@@ -246,17 +249,42 @@ def test_ffn_fused(dtype, rows, d, Fh, act, with_ln):
         assert ho is None
 
 
-def test_ffn_fused_rows_are_batch_invariant():
+@pytest.mark.parametrize("packed", ["auto", False])
+def test_ffn_fused_rows_are_batch_invariant(packed):
     d, Fh = 192, 768
     x = _rand(400, d, dtype=torch.float16, seed=1)
     h2 = _rand(400, d, dtype=torch.float16, seed=2)
     w0 = _rand(Fh, d, dtype=torch.float16, seed=3, scale=0.07)
     w2 = _rand(d, Fh, dtype=torch.float16, seed=4, scale=0.04)
     b0, b2, lw, lb = _rand(Fh, seed=5), _rand(d, seed=6), _rand(d, seed=7) + 1, _rand(d, seed=8)
-    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb)
+    xo, ho = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb, packed=packed)
     for lo, hi in ((0, 1), (3, 130), (127, 256), (271, 400)):
-        a, b = ops.ffn_fused(x[lo:hi].contiguous(), h2[lo:hi].contiguous(), w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb)
+        a, b = ops.ffn_fused(x[lo:hi].contiguous(), h2[lo:hi].contiguous(), w0, b0, w2, b2, act="relu", ln_w=lw, ln_b=lb,
+                             packed=packed)
         assert torch.equal(a, xo[lo:hi]) and torch.equal(b, ho[lo:hi])
+
+
+def test_ffn_fused_packed_image_follows_the_weights_and_large_row_counts():
+    """The image cache is keyed by the weight tensors' identity and in-place version: an in-place edit of a weight
+    must show in the next call.  Plus a persistent-grid case (more 256-row tiles than CUs, ragged tail)."""
+    d, Fh, rows = 128, 512, 70001
+    x = _rand(rows, d, dtype=torch.float16, seed=1)
+    h2 = _rand(rows, d, dtype=torch.float16, seed=2)
+    w0 = _rand(Fh, d, dtype=torch.float16, seed=3, scale=0.09)
+    w2 = _rand(d, Fh, dtype=torch.float16, seed=4, scale=0.04)
+    b0, b2 = _rand(Fh, seed=5) * 0.3, _rand(d, seed=6) * 0.3
+    a1, _ = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu")
+    ref, _ = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu", packed=False)
+    scale = ref.float().abs().max().item()
+    assert (a1.float() - ref.float()).abs().max().item() <= 2 * EPS16[torch.float16] * scale
+    small, _ = ops.ffn_fused(x[69000:].contiguous(), h2[69000:].contiguous(), w0, b0, w2, b2, act="relu")
+    assert torch.equal(small, a1[69000:])
+    w2.mul_(0.5)
+    b0.add_(0.25)
+    a2, _ = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu")
+    ref2, _ = ops.ffn_fused(x, h2, w0, b0, w2, b2, act="relu", packed=False)
+    assert not torch.equal(a1, a2)
+    assert (a2.float() - ref2.float()).abs().max().item() <= 2 * EPS16[torch.float16] * scale
 
 
 def test_ffn_fused_unsupported_shapes_say_so():
