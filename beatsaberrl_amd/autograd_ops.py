@@ -13,7 +13,8 @@ What runs where in a backward pass:
   * Linear weight / bias gradient: `ops.wgrad` on the 16-bit stream (MFMA, LDS transpose loads); on the
     fp32 stream the vendor GEMM through torch (`g.t() @ x`), as the reference does;
   * attention: `ops.attn_bwd`, writing dq | dk | dv into one packed gradient buffer;
-  * block FFN with the fused forward kernel (`FusedFfnFn`): the chain's backward over a recomputed hidden.
+  * block FFN with the fused forward kernel (`FusedFfnFn`): the chain's backward over the hidden the kernel wrote, or over
+    a recomputed one.
 """
 from __future__ import annotations
 
@@ -181,32 +182,46 @@ class FusedFfnFn(torch.autograd.Function):
     """x + W2 relu(W0 h2 + b0) + b2 with the forward as ONE kernel, the block FFN of the update path when the
     fused FFN is on (reference python/fp16_linear.py:1197-1251 `_FusedFfn`).  The backward is the unfused chain's:
     (dW2, db2) = wgrad(g, hidden), gm = (g @ W2) * [hidden > 0] as one gated GEMM, (dW0, db0) = wgrad(gm, h2),
-    dh2 = gm @ W0, dx = g.  Where the reference's kernel writes the hidden for the backward, this forward keeps
-    h2 only and the backward recomputes the hidden with the Linear kernel (one more rows x d x F GEMM per
-    step, rows x F activations less held between forward and backward)."""
+    dh2 = gm @ W0, dx = g.  save_hidden: the forward kernel also writes the activated hidden for the backward, as the
+    reference's does (its mask is hidden > 0); otherwise the forward keeps h2 only and the backward recomputes the
+    hidden with the Linear kernel (one more rows x d x F GEMM per step, rows x F activations less held between
+    forward and backward).  Shapes without the packed-image kernel always recompute."""
 
     @staticmethod
-    def forward(ctx, x, h2, w0, b0, w2, b2):
+    def forward(ctx, x, h2, w0, b0, w2, b2, save_hidden=False):
         w0h, w2h = _w_for(w0, x.dtype), _w_for(w2, x.dtype)
         b0f, b2f = b0.detach().float().contiguous(), b2.detach().float().contiguous()
-        r = ops.ffn_fused(x.contiguous(), h2.contiguous(), w0h, b0f, w2h, b2f, act="relu")
+        xc, hc = x.contiguous(), h2.contiguous()
+        r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu", want_hidden=True) if save_hidden else None
+        hid = None
+        if r is not None:
+            hid = r[2]
+        else:
+            r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu")
         if r is None:
             raise ops.Unsupported(f"fused FFN d={x.shape[-1]} F={w0.shape[0]} dtype={x.dtype}")
-        ctx.save_for_backward(h2, w0h, w2h, b0f)
+        ctx.has_hid = hid is not None
+        if hid is not None:
+            ctx.save_for_backward(h2, w0h, w2h, b0f, hid)
+        else:
+            ctx.save_for_backward(h2, w0h, w2h, b0f)
         return r[0]
 
     @staticmethod
     def backward(ctx, g):
-        h2, w0h, w2h, b0f = ctx.saved_tensors
+        if ctx.has_hid:
+            h2, w0h, w2h, b0f, hid = ctx.saved_tensors
+        else:
+            h2, w0h, w2h, b0f = ctx.saved_tensors
+            hid = ops.linear(h2, w0h, b0f, act="relu")
         need = ctx.needs_input_grad                              # x, h2, w0, b0, w2, b2
         g = g.contiguous()
-        hid = ops.linear(h2, w0h, b0f, act="relu")
         dw2, db2 = _wgrad(_rows(g), _rows(hid), need[4], need[5])
         gm = ops.linear_gated(g, w2h.t().contiguous(), hid)
         del hid
         dw0, db0 = _wgrad(_rows(gm), _rows(h2), need[2], need[3])
         dh2 = ops.linear(gm, w0h.t().contiguous()) if need[1] else None
-        return (g if need[0] else None), dh2, dw0, db0, dw2, db2
+        return (g if need[0] else None), dh2, dw0, db0, dw2, db2, None
 
 
 class AttnPackedFn(torch.autograd.Function):

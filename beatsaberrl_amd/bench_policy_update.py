@@ -80,7 +80,8 @@ def main(argv=None):
     ap.add_argument("--fp16", action="store_true", help="the 16-bit stream (production configuration)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 as the 16-bit stream dtype")
     ap.add_argument("--legacy-arch", action="store_true", help="ctor defaults (128 / 256 / 3 blocks) instead of the recipe")
-    ap.add_argument("--fused-ffn", action="store_true", help="block FFNs forward as the fused kernel (hidden recomputed in the backward)")
+    ap.add_argument("--fused-ffn", action="store_true", help="block FFNs forward as the fused kernel, which also writes the hidden for the backward")
+    ap.add_argument("--fused-ffn-recompute", action="store_true", help="fused FFN forward that keeps no hidden: the backward recomputes it (less memory)")
     ap.add_argument("--no-step", action="store_true", help="forward + backward only (no clip, no optimizer)")
     args = ap.parse_args(argv)
     dev = torch.device("cuda:0")
@@ -93,8 +94,8 @@ def main(argv=None):
     if args.fp16 or args.bf16:
         policy.fp16 = True
         policy.stream_dtype = torch.bfloat16 if args.bf16 else torch.float16
-    if args.fused_ffn:
-        policy.fused_ffn = policy.arch["fused_ffn"] = "on"
+    if args.fused_ffn or args.fused_ffn_recompute:
+        policy.fused_ffn = policy.arch["fused_ffn"] = "recompute" if args.fused_ffn_recompute else "on"
     scale = 4096.0 if policy.fp16 else 1.0
     opt = torch.optim.Adam(policy.parameters(), lr=LR)
     print(f"gpu: {torch.cuda.get_device_name(0)}  torch {torch.__version__}  stream "

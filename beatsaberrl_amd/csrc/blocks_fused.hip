@@ -958,7 +958,7 @@ int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
 // xo rounded once, LayerNorm statistics on the ROUNDED xo, ho rounded once.
 struct FfnArgs {
     const uint2* frags; const float* vec;        // image: 2 * F / 32 stages, then b0 (F) | b2 (d) fp32
-    const u16* x; const u16* h2; u16* xo; u16* ho;
+    const u16* x; const u16* h2; u16* xo; u16* ho; u16* hid;      // hid: (rows, F) activated hidden for a backward, or NULL
     const float* ln_w; const float* ln_b; float eps;
     int64_t rows; int F, total_stages;
 };
@@ -972,7 +972,7 @@ template <int D> struct FfnRing {
     static_assert(SLOTS >= 5 && LPW_HI * (AHEAD + 2) < 64, "vmcnt is 6 bits");
 };
 
-template <typename DT, int D, int ACT, bool LN>
+template <typename DT, int D, int ACT, bool LN, bool SAVE>
 __global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
     typedef FfnRing<D> R;
@@ -1087,6 +1087,20 @@ __global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
                     hid[rt].w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
                     hid[rt].w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
                 }
+            if (SAVE) {
+                // the rounded hidden exactly as the down-projection consumes it: a lane holds 4 consecutive units of its
+                // row per tile of the chunk (these stores sit in the vmcnt queue like any other: they can only make the
+                // ring's admission waits stricter)
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    const int64_t row = row0 + 16 * rt + r16;
+                    if (row < a.rows) {
+                        u16* hr = a.hid + row * a.F + 32 * ch + 4 * g;
+                        *reinterpret_cast<uint2*>(hr) = hid[rt].h[0];
+                        *reinterpret_cast<uint2*>(hr + 16) = hid[rt].h[1];
+                    }
+                }
+            }
             // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
             if (ch + 1 < nch) { advance(Odd{}); up(ch + 1); advance(Even{}); }
             else advance(Odd{});
@@ -1200,7 +1214,8 @@ int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
         hipLaunchKernelGGL(kern, grid, dim3(512), dyn, st, a);
         return (int)BSRL_OK;
     };
-    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true>) : launch(ffn_rows_kernel<DT, D, ACT, false>);
+    if (a.hid) return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, true>) : launch(ffn_rows_kernel<DT, D, ACT, false, true>);
+    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false>) : launch(ffn_rows_kernel<DT, D, ACT, false, false>);
 }
 
 }  // namespace
@@ -1228,21 +1243,22 @@ extern "C" int bsrl_ffn_pack(const void* w0, const float* b0, const void* w2, co
 }
 
 extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const float* ln_w, const float* ln_b,
-                               float eps, void* xo, void* ho, int64_t rows, int64_t d, int64_t F, int act, int dtype,
-                               bsrl_stream stream) {
+                               float eps, void* xo, void* ho, void* hid, int64_t rows, int64_t d, int64_t F, int act,
+                               int dtype, bsrl_stream stream) {
     if (!image || !x || !h2 || !xo) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: null pointer");
     if ((ln_w == nullptr) != (ho == nullptr) || (ln_w == nullptr) != (ln_b == nullptr))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: ln_w, ln_b and ho go together");
     if (!ffn_packed_shape_ok(d, F, dtype) || (act != BSRL_ACT_RELU && act != BSRL_ACT_GELU)) return BSRL_UNSUPPORTED;
     if (rows < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: rows < 0");
-    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(h2, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)))
+    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(h2, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)) ||
+        (hid && !bsrl_aligned(hid, 8)))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: image must be 16-byte, rows 8-byte aligned");
     if (rows == 0) return BSRL_OK;
     FfnArgs a;
     a.frags = static_cast<const uint2*>(image);
     a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + ffn_frag_bytes(d, F));
     a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(h2);
-    a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho);
+    a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho); a.hid = static_cast<u16*>(hid);
     a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F; a.total_stages = (int)(2 * (F / 32));
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;

@@ -28,7 +28,7 @@ import torch.nn as nn
 from . import ops
 
 ACCUM_MODES = ("off", "fwd", "all")
-FFN_MODES = ("off", "on", "up16")
+FFN_MODES = ("off", "on", "up16", "recompute")
 
 _weights_version = 0
 _accum_mode = "off"
@@ -73,7 +73,8 @@ class fp16_accum:
 
 class ffn_fusion:
     """Selects the fused block-FFN kernel inside the context (reference :1120-1140).
-    "up16" (fp16-accumulated up-projection in the reference) maps to "on"."""
+    "up16" (fp16-accumulated up-projection in the reference) maps to "on"; "recompute" differs from "on" in the
+    update path only (the fused forward keeps no hidden and the backward recomputes it)."""
 
     def __init__(self, mode):
         if mode not in FFN_MODES:

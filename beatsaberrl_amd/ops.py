@@ -395,9 +395,11 @@ def ffn_pack(w0, b0, w2, b2):
     return img
 
 
-def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5, packed="auto"):
+def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5, packed="auto", want_hidden=False):
     """xo = x + act(h2 w0^T + b0) w2^T + b2; ho = LN(xo) when ln_w is given.
     Returns (xo, ho) (ho None without LN), or None when unsupported.
+    want_hidden (packed route only; None is returned where that route has no kernel): (xo, ho, hid) with hid (.., F) the
+    activated hidden as the down-projection consumed it, for a backward (the reference's save mode).
     packed: "auto" takes the packed-image kernel (bsrl_ffn_packed: d <= 256, weights streamed straight into LDS,
     32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter."""
     _need_cuda(x, h2, w0, w2)
@@ -416,13 +418,16 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5,
     ho = torch.empty_like(x) if ln_w is not None else None
     if packed and ffn_pack_supported(d, Fh, x.dtype):
         img = ffn_pack(w0, _f32c(b0, "b0"), w2, _f32c(b2, "b2"))
+        hid = torch.empty(*x.shape[:-1], Fh, device=x.device, dtype=x.dtype) if want_hidden else None
         with torch.cuda.device(x.device):
             rc = _lib.load().bsrl_ffn_packed(img.data_ptr(), x.data_ptr(), h2.data_ptr(), _ptr(_f32c(ln_w, "ln_w")),
-                                             _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), rows, d, Fh,
-                                             _ACT[act], dt_code(x.dtype), _stream(x))
+                                             _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), _ptr(hid),
+                                             rows, d, Fh, _ACT[act], dt_code(x.dtype), _stream(x))
         if not _lib.check(rc, "bsrl_ffn_packed"):
             return None
-        return xo, ho
+        return (xo, ho, hid) if want_hidden else (xo, ho)
+    if want_hidden:
+        return None
     with torch.cuda.device(x.device):
         rc = _lib.load().bsrl_ffn_fused(x.data_ptr(), h2.data_ptr(), w0.data_ptr(), _f32c(b0, "b0").data_ptr(),
                                         w2.data_ptr(), _f32c(b2, "b2").data_ptr(), _ptr(_f32c(ln_w, "ln_w")),

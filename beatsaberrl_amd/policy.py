@@ -261,7 +261,8 @@ def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False, fused_f
     x = _lin_t(self.out_proj, att, residual=x)
     x, h2 = LnResFn.apply(x, self.ln_ffn.weight, self.ln_ffn.bias, self.ln_ffn.eps)
     if fused_ffn:
-        x = FusedFfnFn.apply(x, h2, self.ffn[0].weight, self.ffn[0].bias, self.ffn[2].weight, self.ffn[2].bias)
+        x = FusedFfnFn.apply(x, h2, self.ffn[0].weight, self.ffn[0].bias, self.ffn[2].weight, self.ffn[2].bias,
+                             fused_ffn != "recompute")
     else:
         x = _seq_t(self.ffn, h2, residual=x)
     return (x, v) if want_v else x
@@ -578,8 +579,10 @@ class NotePolicy(nn.Module):
             x = self.emb_ln(x)
         v0 = None
         ffn = self.blocks[0].ffn
+        # "on" / "up16": the forward kernel writes the hidden for the backward (the reference's form); "recompute":
+        # it keeps the block input only and the backward recomputes the hidden (less memory, one more GEMM)
         fuse = (self.fp16 and self.fused_ffn != "off" and isinstance(ffn[1], nn.ReLU)
-                and ops.ffn_fused_supported(ffn[0].in_features, ffn[0].out_features, dt))
+                and ops.ffn_fused_supported(ffn[0].in_features, ffn[0].out_features, dt)) and self.fused_ffn
         for i, blk in enumerate(self.blocks[:-1]):
             if self.value_residual and i == 0:
                 x, v0 = blk.forward_train(x, attn_bias, want_v=True, fused_ffn=fuse)

@@ -147,12 +147,14 @@ int bsrl_ffn_fused_supported(int64_t d, int64_t F, int dtype);
  * unsupported shape) from w0 (F, d) and w2 (d, F) in `dtype` and the fp32 biases - once per
  * weight update, like the 16-bit replicas the reference keeps (python/fp16_linear.py:150-192);
  * bsrl_ffn_packed is bsrl_ffn_fused with the image in place of w0, b0, w2, b2.  x, h2, xo, ho
- * (rows, d) contiguous in `dtype`, 8-byte aligned. */
+ * (rows, d) contiguous in `dtype`, 8-byte aligned.  hid, if not NULL, receives the activated
+ * hidden (rows, F) in `dtype` exactly as the down-projection consumed it - what the reference's
+ * kernel returns for the backward (fused_ffn.cu:551-619, `hid`; its ReLU mask is hid > 0). */
 int64_t bsrl_ffn_pack_size(int64_t d, int64_t F, int dtype);
 int bsrl_ffn_pack(const void* w0, const float* b0, const void* w2, const float* b2,
                   int64_t d, int64_t F, int dtype, void* image, bsrl_stream stream);
 int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const float* ln_w,
-                    const float* ln_b, float eps, void* xo, void* ho, int64_t rows,
+                    const float* ln_b, float eps, void* xo, void* ho, void* hid, int64_t rows,
                     int64_t d, int64_t F, int act, int dtype, bsrl_stream stream);
 
 /* ---- Config-model tokenizer -----------------------------------------------

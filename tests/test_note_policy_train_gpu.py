@@ -318,8 +318,10 @@ def test_functions_match_torch_autograd_on_the_same_forward(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rows,d,F", [(70, 128, 512), (4133, 192, 768)])
-def test_fused_ffn_function_matches_the_unfused_chain(dtype, rows, d, F):
-    """FusedFfnFn (fused forward kernel, chain backward over the recomputed hidden; reference
+@pytest.mark.parametrize("save", [False, True])
+def test_fused_ffn_function_matches_the_unfused_chain(dtype, rows, d, F, save):
+    """FusedFfnFn (fused forward kernel; chain backward over the hidden the kernel wrote - `save` - or over a
+    recomputed one; reference
     python/fp16_linear.py:1197-1251) against ChainFn on the same operands: outputs to 16-bit rounding of the
     stream, every gradient to 2 % of its largest entry (the two forwards accumulate in different k orders, so a
     hidden unit within a rounding of 0 may sit on the other side of the ReLU)."""
@@ -332,7 +334,7 @@ def test_fused_ffn_function_matches_the_unfused_chain(dtype, rows, d, F):
     for fn in ("fused", "chain"):
         leaves = [t.clone().requires_grad_(True) for t in (x0, h0, w0, b0, w2, b2)]
         x, h, a0, c0, a2, c2 = leaves
-        y = FusedFfnFn.apply(x, h, a0, c0, a2, c2) if fn == "fused" else ChainFn.apply(h, x, False, a0, c0, a2, c2)
+        y = FusedFfnFn.apply(x, h, a0, c0, a2, c2, save) if fn == "fused" else ChainFn.apply(h, x, False, a0, c0, a2, c2)
         y.backward(go)
         outs.append((y.detach(), [t.grad for t in leaves]))
     (yf, gf), (yc, gc) = outs
@@ -343,6 +345,33 @@ def test_fused_ffn_function_matches_the_unfused_chain(dtype, rows, d, F):
         err = (a.float() - b.float()).abs().max().item()
         assert err <= 2e-2 * b.float().abs().max().item(), (name, err)
     assert torch.equal(gf[0], go)                               # the residual branch passes the gradient through
+
+
+def test_fused_ffn_saved_hidden_is_the_hidden_the_kernel_used():
+    """want_hidden: the (rows, F) tensor the packed kernel writes is relu(h2 W0^T + b0) rounded once - within one
+    16-bit ulp of the Linear kernel's (another k order) - and the backward over it equals the backward over the
+    recomputed hidden wherever the two hiddens agree bitwise (here: gradients to 1e-3 of their largest entry)."""
+    from beatsaberrl_amd import ops
+    from beatsaberrl_amd.autograd_ops import FusedFfnFn
+    rows, d, F, dtype = 1000, 192, 768, torch.float16
+    g = torch.Generator().manual_seed(9)
+    mk = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).to(DEV)
+    w0, b0, w2, b2 = mk(F, d, sc=d ** -0.5), mk(F, sc=0.1), mk(d, F, sc=F ** -0.5), mk(d, sc=0.1)
+    x0, h0, go = mk(rows, d).to(dtype), mk(rows, d).to(dtype), mk(rows, d).to(dtype)
+    xo, ho, hid = ops.ffn_fused(x0, h0, w0.to(dtype), b0, w2.to(dtype), b2, act="relu", want_hidden=True)
+    ref = ops.linear(h0, w0.to(dtype), b0, act="relu")
+    assert hid.shape == (rows, F) and hid.dtype is dtype and ho is None
+    assert (hid.float() - ref.float()).abs().max().item() <= 2.0 ** -10 * ref.float().abs().max().item()
+    assert (hid == ref).float().mean().item() > 0.99
+    plain, _ = ops.ffn_fused(x0, h0, w0.to(dtype), b0, w2.to(dtype), b2, act="relu")
+    assert torch.equal(plain, xo)                               # writing the hidden changes nothing else
+    grads = []
+    for save in (True, False):
+        leaves = [t.clone().requires_grad_(True) for t in (x0, h0, w0, b0, w2, b2)]
+        FusedFfnFn.apply(*leaves, save).backward(go)
+        grads.append([t.grad for t in leaves])
+    for name, a, b in zip(("dx", "dh2", "dw0", "db0", "dw2", "db2"), *grads):
+        assert (a.float() - b.float()).abs().max().item() <= 1e-3 * b.float().abs().max().item(), name
 
 
 def test_update_path_with_the_fused_ffn_follows_the_unfused_update():
@@ -357,13 +386,16 @@ def test_update_path_with_the_fused_ffn_follows_the_unfused_update():
     action = (torch.rand(B, 29, generator=g) * 5).long().to(DEV)
     adv, ret = torch.randn(B, generator=g).to(DEV), torch.randn(B, generator=g).to(DEV)
     res = []
-    for mode in ("off", "on"):
+    for mode in ("off", "on", "recompute"):
         m.fused_ffn = mode
         m.zero_grad(set_to_none=True)
         logits, value = m.forward_stacked(obs)
         (_loss(logits, value, action, adv, ret) * 1024.0).backward()
         res.append((logits.detach(), value.detach(), {n: p.grad.detach().clone() / 1024.0 for n, p in m.named_parameters()}))
-    (l0, v0, g0), (l1, v1, g1) = res
+    (l0, v0, g0), (l1, v1, g1), (l2, v2, g2) = res
+    assert torch.equal(l1, l2) and torch.equal(v1, v2)         # one forward kernel, with or without the hidden written
+    for n in g1:                                                # and the same chain backward up to the hidden's k order
+        assert (g1[n] - g2[n]).norm().item() <= 2e-2 * g2[n].norm().item() + 1e-12, n
     assert not torch.equal(l0, l1)                              # the fused kernel did run
     assert (l0 - l1).abs().max().item() < 2e-2 and (v0 - v1).abs().max().item() < 2e-2
     gmax = max(t.abs().max().item() for t in g0.values())
