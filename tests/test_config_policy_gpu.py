@@ -172,6 +172,26 @@ def test_fused_route_config1(dtype, B, prune):
     _check16(lg, v, p, spec, obs, k, dtype, round_residual=False, ceil=ceil, margin=margin)
 
 
+@pytest.mark.parametrize("w_seed,obs_seed,mask", [(1, 2, "uniform"), (11, 12, "uniform"), (21, 22, "none"), (31, 32, "uniform"),
+                                                  (41, 42, "quarter_empty")])
+def test_fused_route_error_distribution_over_seeds(w_seed, obs_seed, mask):
+    """How close the 16-bit forward is to the fp32 oracle does not hang on one draw of weights and inputs: five
+    (weights, observations, mask) draws of the headline model at B = 4096, fp16, each with its share of logits within
+    2e-3 of the fp32 oracle, its 99.9th percentile and its maximum under literal bounds (the first draw is the
+    benchmark's own; measured over the five: share 0.973-0.993, p99.9 2.5e-3-3.1e-3, max 3.6e-3-5.0e-3)."""
+    spec, B = cm.CONFIGS[1]["spec"], 4096
+    p, m = _build(spec, w_seed, "f16", "fused", randomize_affine=False)
+    obs, k = cm.make_inputs(spec, B, obs_seed, mask)
+    lg, v = m.forward_stacked(obs.to(DEV), None if k is None else k.to(DEV))
+    ref_lg, ref_v = cm.forward(p, spec, obs, k)
+    err = (lg.float().cpu() - ref_lg).abs().flatten()
+    share = (err <= 2e-3).float().mean().item()
+    p999 = torch.quantile(err[torch.randperm(err.numel(), generator=torch.Generator().manual_seed(0))[:1000000]], 0.999).item()
+    print(f"\nDIST w_seed={w_seed} obs_seed={obs_seed} mask={mask}: within2e-3={share:.4f} p99.9={p999:.3e} max={err.max().item():.3e} "
+          f"value max={(v.float().cpu() - ref_v).abs().max().item():.3e}")
+    assert share >= 0.965 and p999 <= 3.6e-3 and err.max().item() <= 6.3e-3
+
+
 @pytest.mark.parametrize("act,final_ln,L,ffn,dtype,ceil,margin", [
     ("relu", True, 3, 256, "f16", (3.8e-3, 2.7e-3, 2.1e-3), None), ("gelu", True, 1, 512, "bf16", (2.5e-2, 1.8e-2, 1.1e-2), 0.05),
     ("relu", False, 4, 1024, "f16", (9.1e-3, 7.2e-3, 4.7e-3), None), ("gelu", False, 8, 64, "f16", (1.4e-2, 1.2e-2, 5.9e-3), None)])
