@@ -106,6 +106,12 @@ constexpr int DMA_SLOTS = 6, DMA_AHEAD = DMA_SLOTS - 4;
 __device__ __forceinline__ void ring_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr));
 }
+// two consecutive fragments: the instruction's immediate offset moves the global AND the LDS address, so the second
+// transfer needs no second m0 write and no address arithmetic
+__device__ __forceinline__ void ring_load2(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024"
+                 ::"v"(voff), "s"(sbase), "s"(lds_addr));
+}
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -191,37 +197,45 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     int pnext;
     // RING: this wave's two fragments of stage `stage` -> ring slot `slot` (every wave loads, working or not: leaving the
     // loads to the waves without an env - 3 + 3 + 2 fragments - measured slower, 36 against 33 us per forward)
-    auto ring_issue = [&](int stage, int slot) __attribute__((always_inline)) {
-        const char* sb = reinterpret_cast<const char*>(img) + (int64_t)stage * (STAGE_U4 * 16) + uwave * 2048;
-        const uint32_t dst = ring_base + slot * (STAGE_U4 * 16) + uwave * 2048;
-        ring_load(lane * 16, sb, dst);
-        ring_load(lane * 16, sb + 1024, dst + 1024);
+    // The transfers address the image and the ring by running BYTE offsets (a stage and a slot are both 8 KB): one
+    // 64-bit scalar add per issue instead of two multiplies per index.
+    constexpr uint32_t STAGE_B = STAGE_U4 * 16;
+    const char* wsrc = reinterpret_cast<const char*>(img) + uwave * 2048;      // this wave's two fragments of a stage
+    const uint32_t wdst = ring_base + uwave * 2048;
+    uint32_t src_off = 0;                             // byte offset of stage pnext
+    const uint32_t src_begin = (uint32_t)a.s_begin * STAGE_B, src_end = (uint32_t)a.s_end * STAGE_B;
+    auto ring_issue_off = [&](uint32_t slot_off) __attribute__((always_inline)) {     // stage pnext -> the slot at slot_off
+        ring_load2(lane * 16, wsrc + src_off, wdst + slot_off);
+        src_off = src_off + STAGE_B == src_end ? src_begin : src_off + STAGE_B;
     };
     // RING: called when the next stage is about to be consumed; on return it is readable in slot ring_cur
+    uint32_t ring_off = (RING_SLOTS - 1) * STAGE_B;   // byte offset of slot ring_cur
     auto ring_advance = [&]() __attribute__((always_inline)) {
+        const uint32_t freed = ring_off;              // the slot of the stage consumed last
         ring_cur = ring_cur + 1 == RING_SLOTS ? 0 : ring_cur + 1;
+        ring_off = ring_off + STAGE_B == RING_SLOTS * STAGE_B ? 0 : ring_off + STAGE_B;
         // this wave's loads of that stage have landed once at most the RING_DEPTH - 1 younger stages' are outstanding
         // (loads retire in order; any other load or store in flight only makes the wait stricter) ...
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (RING_DEPTH - 1)) : "memory");
         lds_barrier();                                // ... and every wave's have; every wave is done reading the stage before
-        ring_issue(pnext, ring_cur == 0 ? RING_SLOTS - 1 : ring_cur - 1);      // its slot takes the stage RING_DEPTH ahead
-        pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
+        ring_issue_off(freed);                        // its slot takes the stage RING_DEPTH ahead
     };
     // DMA: entry of the next stage (par = its parity in the launch's stage range): on return it is readable in slot
     // dma_cur.  An even stage admits itself and its successor: this wave's loads of both have landed once at most the
     // DMA_AHEAD younger stages' are outstanding, the barrier says the same of every wave's and that every wave is done
     // reading the two stages before; their slots take the next two stages.
     int dma_cur = DMA_SLOTS - 1;
+    uint32_t dma_off = (DMA_SLOTS - 1) * STAGE_B, dma_prev = (DMA_SLOTS - 2) * STAGE_B;     // byte offsets of slot dma_cur and the one before
     auto dma_advance = [&](int par) __attribute__((always_inline)) {
+        const uint32_t older = dma_prev;
+        dma_prev = dma_off;
         dma_cur = dma_cur + 1 == DMA_SLOTS ? 0 : dma_cur + 1;
+        dma_off = dma_off + STAGE_B == DMA_SLOTS * STAGE_B ? 0 : dma_off + STAGE_B;
         if (par == 0) {
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DMA_AHEAD) : "memory");
             lds_barrier();
-            const int s1 = dma_cur == 0 ? DMA_SLOTS - 1 : dma_cur - 1, s2 = s1 == 0 ? DMA_SLOTS - 1 : s1 - 1;
-            ring_issue(pnext, s2);
-            pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
-            ring_issue(pnext, s1);
-            pnext = pnext + 1 == a.s_end ? a.s_begin : pnext + 1;
+            ring_issue_off(older);                    // the two slots behind the pair being admitted
+            ring_issue_off(dma_prev);
         }
     };
     // RING: the working waves keep the NEXT stage's eight fragments in registers (wnext), fetched from LDS while the
@@ -232,7 +246,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     // operand so that no use of it can be scheduled above the wait.
     s16x8 wnext[RING ? STAGE_FRAGS : 1];
     auto ring_fetch = [&]() __attribute__((always_inline)) {
-        const uint32_t addr = ring_base + ring_cur * (STAGE_U4 * 16) + lane * 16;
+        const uint32_t addr = ring_base + ring_off + lane * 16;
 #pragma unroll
         for (int f = 0; f < STAGE_FRAGS; ++f)
             asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wnext[RING ? f : 0]) : "v"(addr), "n"(f * 1024));
@@ -249,10 +263,9 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     };
     if (RING) {
         // prologue: RING_DEPTH stages in flight (the weight image holds at least that many), then the vectors
-        int st = a.s_begin;
+        src_off = src_begin;
 #pragma unroll
-        for (int i = 0; i < RING_DEPTH; ++i) { ring_issue(st, i); st = st + 1 == a.s_end ? a.s_begin : st + 1; }
-        pnext = st;
+        for (int i = 0; i < RING_DEPTH; ++i) ring_issue_off(i * STAGE_B);
         const int nv4 = vec_floats(a.n_layers, a.F) / 4;
         for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
         lds_barrier();
@@ -260,10 +273,9 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         ring_fetch();               // ... and on its way to registers (every wave: the waves without an env never wait for it)
     } else if (DMA) {
         // prologue: DMA_SLOTS - 2 stages in flight (every launch's stage range is longer and even), then the vectors
-        int st = a.s_begin;
+        src_off = src_begin;
 #pragma unroll
-        for (int i = 0; i < DMA_SLOTS - 2; ++i) { ring_issue(st, i); st = st + 1 == a.s_end ? a.s_begin : st + 1; }
-        pnext = st;
+        for (int i = 0; i < DMA_SLOTS - 2; ++i) ring_issue_off(i * STAGE_B);
         const int nv4 = vec_floats(a.n_layers, a.F) / 4;
         for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
         lds_barrier();
