@@ -426,23 +426,79 @@ __global__ __launch_bounds__(512) void blocks_kernel(BlkArgs a) {
 //     stages ahead into a ring of SLOTS stage slots: no register staging, depth bounded by LDS only;
 //   * the row reductions of LayerNorm and softmax are lane-row swaps on the VALU, not shuffles through LDS.
 // Per-row arithmetic, its order and the weight image are those of blocks_kernel: an env's output bits are the same.
-template <int D> struct EnvRing {
-    static constexpr int NW = 8;
-    static constexpr int SLOTS = D == 128 ? 10 : 7;                                    // stage slots
-    // Stages are entered in PAIRS (every block has an even number of them): one wait + barrier admits two stages and
-    // refills the two slots behind them.  Stages that may still be in flight then: all but those four.
-    static constexpr int AHEAD = SLOTS - 4;
-    static constexpr int STAGE_BYTES = Geo<D>::SF * 1024;
-    // fragment f of a stage is loaded by wave f % NW: LPW_HI loads for waves < N_HI, LPW_HI - 1 for the others
-    static constexpr int LPW_HI = (Geo<D>::SF + NW - 1) / NW, N_HI = Geo<D>::SF - (LPW_HI - 1) * NW;
-    static_assert(SLOTS >= 5 && LPW_HI * (AHEAD + 2) < 64, "vmcnt is 6 bits");
-};
 // m0 (the LDS base of the transfer) is written without telling the compiler, which rejects reserved registers in a
 // clobber list: nothing else in the kernel uses it.  No "memory" clobber: what orders these asynchronous LDS writes
-// against the fragment reads is the vmcnt wait + barrier of the stage advance.
+// against the fragment reads is the vmcnt wait + barrier of the stage admission.  The instruction's immediate offset
+// moves BOTH addresses of a transfer, the global one and the LDS one: a wave's second fragment of a stage is the one
+// right after its first and costs no further scalar work.
 __device__ __forceinline__ void env_ring_load(uint32_t voff, const void* sbase, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr));
 }
+__device__ __forceinline__ void env_ring_load2(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024"
+                 ::"v"(voff), "s"(sbase), "s"(lds_addr));
+}
+
+// The weight-stage ring of the one-wave-per-env kernels: stages of SF 1 KB fragments go global -> LDS directly, SLOTS
+// stage slots deep.  Stages are entered in PAIRS (every block has an even number of them): one wait + barrier admits
+// two stages and refills the two slots behind them, so all but those four slots may be in flight (AHEAD).  A loading
+// wave moves FPW ADJACENT fragments of every stage (SF = 8: eight waves one each; 12: six waves two each; 16: eight
+// waves two each); image and ring are addressed by running byte offsets, no multiplies in the loop.
+template <int SF_, int SLOTS_> struct StageRing {
+    static constexpr int NW = 8, SF = SF_, SLOTS = SLOTS_, AHEAD = SLOTS - 4;
+    static constexpr int FPW = SF > NW ? 2 : 1, NLW = SF / FPW;
+    static constexpr uint32_t STAGE_BYTES = SF * 1024;
+    static_assert(SLOTS >= 5 && FPW * NLW == SF && NLW <= NW && FPW * (AHEAD + 2) < 64, "fragment split; vmcnt is 6 bits");
+    const uint4* ring;             // slot 0
+    const char* wsrc;              // this wave's fragments of stage 0
+    uint32_t wdst;                 // ... and their place in slot 0 (LDS byte address)
+    uint32_t voff;                 // lane * 16
+    uint32_t src_off, src_end;     // next stage to load, image length (bytes)
+    uint32_t cur, prev;            // slot of the current stage and of the one before it (bytes from slot 0)
+    bool loader;
+
+    __device__ __forceinline__ void issue(uint32_t slot_off) {
+        if (NLW == NW || loader) {
+            if constexpr (FPW == 2) env_ring_load2(voff, wsrc + src_off, wdst + slot_off);
+            else env_ring_load(voff, wsrc + src_off, wdst + slot_off);
+        }
+        src_off = src_off + STAGE_BYTES == src_end ? 0 : src_off + STAGE_BYTES;
+    }
+    // SLOTS - 2 stages in flight (the host checks that the image is longer)
+    __device__ __forceinline__ void start(const uint4* ring_, const void* img, int total_stages, int wave, int lane) {
+        ring = ring_;
+        wsrc = reinterpret_cast<const char*>(img) + wave * (FPW * 1024);
+        wdst = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring_) + wave * (FPW * 1024);
+        voff = lane * 16;
+        loader = wave < NLW;
+        src_off = 0;
+        src_end = (uint32_t)total_stages * STAGE_BYTES;
+        cur = (SLOTS - 1) * STAGE_BYTES;
+        prev = (SLOTS - 2) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < SLOTS - 2; ++i) issue(i * STAGE_BYTES);
+    }
+    // entry of the next stage (PARITY = its index in its block, mod 2): on return it is readable in slot `cur`
+    template <int PARITY> __device__ __forceinline__ void admit() {
+        const uint32_t older = prev;
+        prev = cur;
+        cur = cur + STAGE_BYTES == SLOTS * STAGE_BYTES ? 0 : cur + STAGE_BYTES;
+        if constexpr (PARITY == 0) {
+            // this wave's loads of this stage and the next have landed once at most the AHEAD younger stages' are
+            // outstanding (loads retire in order; any other load or store in flight, or a wave that loads nothing,
+            // only makes the wait stricter) ...
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FPW * AHEAD) : "memory");
+            blk_barrier();             // ... and every wave's have; every wave is done reading the two stages before this one
+            issue(older);
+            issue(prev);
+        }
+    }
+    // fragment i of the current stage, this lane's 16 bytes
+    __device__ __forceinline__ s16x8 frag(int i, int lane) const {
+        return __builtin_bit_cast(s16x8, ring[(cur >> 4) + i * 64 + lane]);
+    }
+};
+template <int D> struct EnvRing : StageRing<Geo<D>::SF, D == 128 ? 10 : 7> {};
 
 template <typename DT, int D, int DH, int ACT>
 __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
@@ -464,33 +520,8 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
     const int64_t ntiles = (a.B + NW - 1) / NW;
     const int ring_off_u4 = (a.n_layers * G::lv_size(a.F) / 4 + 63) & ~63;
     const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
-    const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
-    const char* img = reinterpret_cast<const char*>(a.frags);
-
-    int cur = R::SLOTS - 1, pnext;
-    auto issue = [&](int stage, int slot) __attribute__((always_inline)) {
-        const char* sb = img + (int64_t)stage * R::STAGE_BYTES;
-        const uint32_t dst = ring_base + slot * R::STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < R::LPW_HI; ++i)
-            if (i + 1 < R::LPW_HI || wave < R::N_HI) env_ring_load(lane * 16, sb + (wave + NW * i) * 1024, dst + (wave + NW * i) * 1024);
-    };
-    // entry of the next stage (parity = its index in its block, mod 2): on return it is readable in slot `cur`
-    auto advance = [&](auto parity_) __attribute__((always_inline)) {
-        cur = cur + 1 == R::SLOTS ? 0 : cur + 1;
-        if constexpr (decltype(parity_)::value == 0) {
-            // this wave's loads of this stage and the next have landed once at most the AHEAD younger stages' are
-            // outstanding (loads retire in order; any other load or store in flight only makes the wait stricter) ...
-            if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
-            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
-            blk_barrier();             // ... and every wave's have; every wave is done reading the two stages before this one
-            const int s1 = cur == 0 ? R::SLOTS - 1 : cur - 1, s2 = s1 == 0 ? R::SLOTS - 1 : s1 - 1;
-            issue(pnext, s2);
-            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
-            issue(pnext, s1);
-            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
-        }
-    };
+    R pipe;
+    auto advance = [&](auto parity_) __attribute__((always_inline)) { pipe.template admit<decltype(parity_)::value>(); };
     typedef std::integral_constant<int, 0> Even;
     typedef std::integral_constant<int, 1> Odd;
     // sub-burst j of the current stage -> registers, then `body` on them
@@ -498,14 +529,11 @@ __global__ __launch_bounds__(512, 1) void blocks_env_kernel(BlkArgs a) {
         constexpr int j = decltype(j_)::value;
         s16x8 w[KB];
 #pragma unroll
-        for (int f = 0; f < KB; ++f) w[f] = __builtin_bit_cast(s16x8, ring[cur * (SF * 64) + (j * KB + f) * 64 + lane]);
+        for (int f = 0; f < KB; ++f) w[f] = pipe.frag(j * KB + f, lane);
         body(w);
     };
     {   // prologue: SLOTS - 2 stages in flight (every stack has more), then the vectors
-        int st = 0;
-#pragma unroll
-        for (int i = 0; i < R::SLOTS - 2; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
-        pnext = st;
+        pipe.start(ring, a.frags, a.total_stages, wave, lane);
         const int nv4 = a.n_layers * G::lv_size(a.F) / 4;
         for (int i = tid; i < nv4; i += NW * 64) bvl4[i] = reinterpret_cast<const float4*>(a.vec)[i];
         blk_barrier();
@@ -963,20 +991,13 @@ struct FfnArgs {
     int64_t rows; int F, total_stages;
 };
 
-template <int D> struct FfnRing {
-    static constexpr int NW = 8;
-    static constexpr int SLOTS = D == 128 ? 10 : D == 192 ? 7 : 6;
-    static constexpr int AHEAD = SLOTS - 4;
-    static constexpr int STAGE_BYTES = Geo<D>::SF * 1024;
-    static constexpr int LPW_HI = (Geo<D>::SF + NW - 1) / NW, N_HI = Geo<D>::SF - (LPW_HI - 1) * NW;
-    static_assert(SLOTS >= 5 && LPW_HI * (AHEAD + 2) < 64, "vmcnt is 6 bits");
-};
+template <int D> struct FfnRing : StageRing<Geo<D>::SF, D == 128 ? 10 : D == 192 ? 7 : 6> {};
 
 template <typename DT, int D, int ACT, bool LN, bool SAVE>
 __global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
     typedef FfnRing<D> R;
-    constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, SF = G::SF, NSUB = 2 * NB;
+    constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
     extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
     float* vlds = reinterpret_cast<float*>(bvl4);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -985,46 +1006,22 @@ __global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
     const int nvec = a.F + 3 * D;
     const int ring_off_u4 = (nvec / 4 + 63) & ~63;
     const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
-    const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
-    const char* img = reinterpret_cast<const char*>(a.frags);
     const float* B1 = vlds; const float* B2 = vlds + a.F; const float* LNG = B2 + D; const float* LNB = LNG + D;
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
 
-    int cur = R::SLOTS - 1, pnext;
-    auto issue = [&](int stage, int slot) __attribute__((always_inline)) {
-        const char* sb = img + (int64_t)stage * R::STAGE_BYTES;
-        const uint32_t dst = ring_base + slot * R::STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < R::LPW_HI; ++i)
-            if (i + 1 < R::LPW_HI || wave < R::N_HI) env_ring_load(lane * 16, sb + (wave + NW * i) * 1024, dst + (wave + NW * i) * 1024);
-    };
-    auto advance = [&](auto parity_) __attribute__((always_inline)) {
-        cur = cur + 1 == R::SLOTS ? 0 : cur + 1;
-        if constexpr (decltype(parity_)::value == 0) {
-            if (R::N_HI == NW || wave < R::N_HI) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::LPW_HI * R::AHEAD) : "memory");
-            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((R::LPW_HI - 1) * R::AHEAD) : "memory");
-            blk_barrier();
-            const int s1 = cur == 0 ? R::SLOTS - 1 : cur - 1, s2 = s1 == 0 ? R::SLOTS - 1 : s1 - 1;
-            issue(pnext, s2);
-            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
-            issue(pnext, s1);
-            pnext = pnext + 1 == a.total_stages ? 0 : pnext + 1;
-        }
-    };
+    R pipe;
+    auto advance = [&](auto parity_) __attribute__((always_inline)) { pipe.template admit<decltype(parity_)::value>(); };
     typedef std::integral_constant<int, 0> Even;
     typedef std::integral_constant<int, 1> Odd;
     auto sub = [&](auto j_, auto&& body) __attribute__((always_inline)) {
         constexpr int j = decltype(j_)::value;
         s16x8 w[KB];
 #pragma unroll
-        for (int f = 0; f < KB; ++f) w[f] = __builtin_bit_cast(s16x8, ring[cur * (SF * 64) + (j * KB + f) * 64 + lane]);
+        for (int f = 0; f < KB; ++f) w[f] = pipe.frag(j * KB + f, lane);
         body(w);
     };
     {   // prologue: SLOTS - 2 stages in flight (the host checks that the image is longer), then the vectors
-        int st = 0;
-#pragma unroll
-        for (int i = 0; i < R::SLOTS - 2; ++i) { issue(st, i); st = st + 1 == a.total_stages ? 0 : st + 1; }
-        pnext = st;
+        pipe.start(ring, a.frags, a.total_stages, wave, lane);
         for (int i = tid; i < a.F + D; i += NW * 64) vlds[i] = a.vec[i];
         if (LN) for (int i = tid; i < D; i += NW * 64) { vlds[a.F + D + i] = a.ln_w[i]; vlds[a.F + 2 * D + i] = a.ln_b[i]; }
         blk_barrier();
