@@ -58,6 +58,9 @@ MASKED_LOGIT = L.MASKED_LOGIT
 TRUNK_ARCHS = ("simba", "simbav2")
 
 
+_SIDE_STREAMS = {}      # device index -> the forward's second stream
+
+
 def _mlp(sizes, act=nn.ReLU):
     layers = []
     for i in range(len(sizes) - 1):
@@ -393,6 +396,8 @@ class NotePolicy(nn.Module):
         # True: the critic's one-query attention runs as a pool over LN(x_res) with the k | v projections folded
         # around it (no (B T, 2d) keys / values); False: the reference's op order
         self.critic_pool = True
+        # batches from this size on run the critic's attention pool on a second stream beside the trunk and heads
+        self.critic_overlap_min_batch = 1024
         self._critic_pool_cache = None
         # The reference keeps the grad-free rollout forward and the grad-mode update forward bit-identical
         # (python/tests/test_fp16_accum.py:146-160): PPO's first-epoch ratio is then exactly 1.  The two fast rollout
@@ -548,10 +553,23 @@ class NotePolicy(nn.Module):
             lead, _ = self.blocks[-1](x, attn_bias, h=h, n_queries=self.n_lead, v0=v0)
         if self.final_ln is not None:
             lead = self.final_ln(lead)
+        # the critic's attention pool needs only the stream entering the final block: for a large batch it runs on a
+        # second stream beside the trunk and the action heads (every kernel of either chain is a small GEMM or a row op
+        # that leaves most of the chip idle), and joins before the value MLP, which needs the trunk's features
+        side = self._side_stream(obs.device) if B >= self.critic_overlap_min_batch else None
+        if side is not None:
+            main = torch.cuda.current_stream(obs.device)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                attended = self._critic_attend(x_res, attn_bias)
         hfeat = self._trunk(lead.reshape(B, self.n_lead * d))
         wh, bh = _fl.packed_halves(list(self.heads), dt)
         out = ops.linear(hfeat, wh, bh, out_dtype=torch.float32)           # (B, sum n_j) fp32
-        value = self._critic(x_res, hfeat, attn_bias)
+        if side is not None:
+            main.wait_stream(side)
+        else:
+            attended = self._critic_attend(x_res, attn_bias)
+        value = self._critic_value(attended, hfeat)
         if self._gear_idx is not None:
             out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
         return out.view(B, N_ACTION_HEADS, self.k_max), value
@@ -679,9 +697,24 @@ class NotePolicy(nn.Module):
             c[0] = _fl._weights_version
         return c[2].view(H * d, d), c[3].view(d, H * d), c[4]
 
+    @staticmethod
+    def _side_stream(device):
+        """The second stream of the forward (default priority), one per device and process, made on first use."""
+        key = torch.device(device).index
+        key = torch.cuda.current_device() if key is None else key
+        s = _SIDE_STREAMS.get(key)
+        if s is None:
+            s = _SIDE_STREAMS[key] = torch.cuda.Stream(device=device)
+        return s
+
     def _critic(self, x_res, hfeat, attn_bias):
         """adapool_v1 value path (policy.py:1346-1403): LN -> query from the torso token ->
         packed k|v -> 1-query attention pool -> out -> MLP -> HL-Gauss expectation."""
+        return self._critic_value(self._critic_attend(x_res, attn_bias), hfeat)
+
+    def _critic_attend(self, x_res, attn_bias):
+        """The attention half of the value path: ((B, d) pooled and out-projected, whether the pooled kernel ran);
+        independent of the trunk."""
         B, T, d = x_res.shape
         H = self.n_heads
         pooled_route = self.critic_pool and not self.rollout_matches_update and ops.critic_pool_supported(T, d, H, x_res.dtype)
@@ -699,7 +732,11 @@ class NotePolicy(nn.Module):
             wkv, bkv = _fl.packed_halves([self.critic_k, self.critic_v], x_res.dtype)
             kv = ops.linear(hv, wkv, bkv)
             a = ops.attn_fwd(q, kv[..., :d], kv[..., d:], H, key_bias=attn_bias).view(B, d)
-        a = _lin(self.critic_out, a)
+        return _lin(self.critic_out, a), pooled_route
+
+    def _critic_value(self, attended, hfeat):
+        """The value MLP over [attended | trunk features] and the HL-Gauss expectation."""
+        a, pooled_route = attended
         z = torch.cat([a, hfeat], dim=-1)
         z = _lin(self.critic_mlp[0], z, act="relu")
         z = _lin(self.critic_mlp[2], z, act="relu")

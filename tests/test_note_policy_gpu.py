@@ -193,6 +193,44 @@ def test_pooled_critic_matches_the_reference_op_order(dtype):
         assert e_pool <= (1e-4 if dtype == "f16" else 7e-4)          # measured 6.7e-5 / 5.2e-4 (reference order: 6.2e-5 / 5.1e-4)
 
 
+@pytest.mark.parametrize("pool", [True, False])
+def test_critic_on_the_second_stream_gives_the_same_bits(pool):
+    """From `critic_overlap_min_batch` envs on, the critic's attention half runs on a second stream beside the trunk
+    and the heads: same logits and values bit for bit as the one-stream order, eagerly (several forwards in a row,
+    so that memory handed back by one forward is taken again by the next) and from a captured graph replayed with
+    eager work between the replays."""
+    m, sd = _big(21, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True)
+    m = m.to(DEV)
+    m.fp16 = True
+    m.critic_pool = pool
+    obs = [_make_obs(1500, 40 + i).to(DEV) for i in range(3)]
+    m.critic_overlap_min_batch = 1 << 30
+    want = [tuple(t.clone() for t in m.forward_stacked(o)) for o in obs]
+    m.critic_overlap_min_batch = 1024
+    for rep in range(3):
+        for o, (lg0, v0) in zip(obs, want):
+            lg, v = m.forward_stacked(o)
+            assert torch.equal(lg, lg0) and torch.equal(v, v0), (pool, rep)
+    static = obs[0].clone()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            m.forward_stacked(static)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_lg, g_v = m.forward_stacked(static)
+    for rep in range(4):
+        o, (lg0, v0) = obs[rep % 3], want[rep % 3]
+        static.copy_(o)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_lg, lg0) and torch.equal(g_v, v0), (pool, "graph", rep)
+        lg, v = m.forward_stacked(obs[(rep + 1) % 3])               # eager work between the replays
+        assert torch.equal(lg, want[(rep + 1) % 3][0])
+
+
 @pytest.mark.parametrize("blocks", ["auto", "off"])
 def test_invariants_and_sampling_epilogue(blocks):
     m, sd = _big(9, embed=192, trunk_dim=384, n_blocks=2, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,
