@@ -188,9 +188,8 @@ def main():
 
     # FLOPs per forward: the dense figure (every token of every block), and the ALGORITHMIC figure of the path as
     # the reference runs it - the final block pruned to token 0 (its own n_queries path), every env's 16 token rows
-    # (padding rows included: the reference computes and masks them).  The roofline fraction is quoted on the
-    # algorithmic figure; what the matrix pipe is really issued (fewer tiles when short envs share them) is
-    # reported beside it as issued_frac.
+    # (padding rows included: the reference computes and masks them).  Both are side notes of the roofline object;
+    # its fraction is quoted on what the matrix pipe is really issued (below).
     dense_flops = cm.flops_per_env(spec) * B
     pruned = (route == "fused" and m.prune_final) or route == "blocks"
     exec_flops = dense_flops
