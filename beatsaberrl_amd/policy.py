@@ -396,8 +396,9 @@ class NotePolicy(nn.Module):
         # True: the critic's one-query attention runs as a pool over LN(x_res) with the k | v projections folded
         # around it (no (B T, 2d) keys / values); False: the reference's op order
         self.critic_pool = True
-        # batches from this size on run the critic's attention pool on a second stream beside the trunk and heads
-        self.critic_overlap_min_batch = 1024
+        # batches from this size on run the critic's attention pool on a second stream beside the trunk and heads (smaller
+        # ones are launch-bound on the host, where the fork and join only add calls)
+        self.critic_overlap_min_batch = 2048
         self._critic_pool_cache = None
         # The reference keeps the grad-free rollout forward and the grad-mode update forward bit-identical
         # (python/tests/test_fp16_accum.py:146-160): PPO's first-epoch ratio is then exactly 1.  The two fast rollout

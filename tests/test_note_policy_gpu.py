@@ -206,7 +206,7 @@ def test_critic_on_the_second_stream_gives_the_same_bits(pool):
     obs = [_make_obs(1500, 40 + i).to(DEV) for i in range(3)]
     m.critic_overlap_min_batch = 1 << 30
     want = [tuple(t.clone() for t in m.forward_stacked(o)) for o in obs]
-    m.critic_overlap_min_batch = 1024
+    m.critic_overlap_min_batch = 1024                            # the 1500-env batches fork
     for rep in range(3):
         for o, (lg0, v0) in zip(obs, want):
             lg, v = m.forward_stacked(o)
