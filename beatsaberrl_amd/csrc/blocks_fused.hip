@@ -438,15 +438,20 @@ __device__ __forceinline__ void env_ring_load2(uint32_t voff, const void* sbase,
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024"
                  ::"v"(voff), "s"(sbase), "s"(lds_addr));
 }
+__device__ __forceinline__ void env_ring_load3(uint32_t voff, const void* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\tglobal_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %0, %1 offset:2048" ::"v"(voff), "s"(sbase), "s"(lds_addr));
+}
 
 // The weight-stage ring of the one-wave-per-env kernels: stages of SF 1 KB fragments go global -> LDS directly, SLOTS
 // stage slots deep.  Stages are entered in PAIRS (every block has an even number of them): one wait + barrier admits
 // two stages and refills the two slots behind them, so all but those four slots may be in flight (AHEAD).  A loading
-// wave moves FPW ADJACENT fragments of every stage (SF = 8: eight waves one each; 12: six waves two each; 16: eight
-// waves two each); image and ring are addressed by running byte offsets, no multiplies in the loop.
-template <int SF_, int SLOTS_> struct StageRing {
-    static constexpr int NW = 8, SF = SF_, SLOTS = SLOTS_, AHEAD = SLOTS - 4;
-    static constexpr int FPW = SF > NW ? 2 : 1, NLW = SF / FPW;
+// wave moves FPW ADJACENT fragments of every stage (eight waves: SF = 8 one each; 12: six waves two each; 16: two each;
+// four waves: 8: two each; 12: three each); image and ring are addressed by running byte offsets, no multiplies in the
+// loop.
+template <int SF_, int SLOTS_, int NW_ = 8> struct StageRing {
+    static constexpr int NW = NW_, SF = SF_, SLOTS = SLOTS_, AHEAD = SLOTS - 4;
+    static constexpr int FPW = (SF + NW - 1) / NW <= 1 ? 1 : SF % 2 == 0 && SF / 2 <= NW ? 2 : 3, NLW = SF / FPW;
     static constexpr uint32_t STAGE_BYTES = SF * 1024;
     static_assert(SLOTS >= 5 && FPW * NLW == SF && NLW <= NW && FPW * (AHEAD + 2) < 64, "fragment split; vmcnt is 6 bits");
     const uint4* ring;             // slot 0
@@ -459,7 +464,8 @@ template <int SF_, int SLOTS_> struct StageRing {
 
     __device__ __forceinline__ void issue(uint32_t slot_off) {
         if (NLW == NW || loader) {
-            if constexpr (FPW == 2) env_ring_load2(voff, wsrc + src_off, wdst + slot_off);
+            if constexpr (FPW == 3) env_ring_load3(voff, wsrc + src_off, wdst + slot_off);
+            else if constexpr (FPW == 2) env_ring_load2(voff, wsrc + src_off, wdst + slot_off);
             else env_ring_load(voff, wsrc + src_off, wdst + slot_off);
         }
         src_off = src_off + STAGE_BYTES == src_end ? 0 : src_off + STAGE_BYTES;
@@ -991,12 +997,15 @@ struct FfnArgs {
     int64_t rows; int F, total_stages;
 };
 
-template <int D> struct FfnRing : StageRing<Geo<D>::SF, D == 128 ? 10 : D == 192 ? 7 : 6> {};
+// Eight waves, one workgroup per CU - or four waves, TWO workgroups per CU (d = 128 / 192, where two rings fit): the
+// waves of a workgroup walk the ring in lockstep, so all of them load and store their rows at the same time with
+// nothing to run meanwhile; a second, independent workgroup drifts out of phase and computes through it.
+template <int D, int NW> struct FfnRing : StageRing<Geo<D>::SF, NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : 6), NW> {};
 
-template <typename DT, int D, int ACT, bool LN, bool SAVE>
-__global__ __launch_bounds__(512, 1) void ffn_rows_kernel(FfnArgs a) {
+template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_>
+__global__ __launch_bounds__(NW_ * 64, 8 / NW_) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
-    typedef FfnRing<D> R;
+    typedef FfnRing<D, NW_> R;
     constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
     extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
     float* vlds = reinterpret_cast<float*>(bvl4);
@@ -1196,23 +1205,34 @@ bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
     return 2 * (F / 32) >= slots;
 }
 int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
-template <int D> size_t ffn_dyn_bytes(int F) {
-    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D>::SLOTS * FfnRing<D>::STAGE_BYTES;
+template <int D, int NW> size_t ffn_dyn_bytes(int F) {
+    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW>::SLOTS * FfnRing<D, NW>::STAGE_BYTES;
 }
-template <typename DT, int D, int ACT>
-int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
-    const size_t dyn = ffn_dyn_bytes<D>(a.F);
-    if (dyn + 1024 > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
-    const int64_t ntiles = (a.rows + 255) / 256;
-    const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));
+template <typename DT, int D, int ACT, int NW>
+int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
+    const size_t dyn = ffn_dyn_bytes<D, NW>(a.F);
+    if ((8 / NW) * (dyn + 1024) > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
+    const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32), slots = (int64_t)cus * (8 / NW);
+    const dim3 grid((unsigned)(ntiles < slots ? ntiles : slots));
     auto launch = [&](auto kern) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return (int)BSRL_UNSUPPORTED;
-        hipLaunchKernelGGL(kern, grid, dim3(512), dyn, st, a);
+        hipLaunchKernelGGL(kern, grid, dim3(NW * 64), dyn, st, a);
         return (int)BSRL_OK;
     };
-    if (a.hid) return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, true>) : launch(ffn_rows_kernel<DT, D, ACT, false, true>);
-    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false>) : launch(ffn_rows_kernel<DT, D, ACT, false, false>);
+    if (a.hid) return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, true, NW>) : launch(ffn_rows_kernel<DT, D, ACT, false, true, NW>);
+    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW>);
+}
+template <typename DT, int D, int ACT>
+int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
+    if constexpr (D != 256) {
+        // two 4-wave workgroups per CU where two rings fit and the image is longer than the shorter ring
+        if (a.total_stages >= FfnRing<D, 4>::SLOTS) {
+            const int rc = ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
+            if (rc != BSRL_UNSUPPORTED) return rc;
+        }
+    }
+    return ffn_launch_nw<DT, D, ACT, 8>(a, ln, cus, st);
 }
 
 }  // namespace
