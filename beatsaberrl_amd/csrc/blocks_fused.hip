@@ -984,7 +984,7 @@ int fwd_launch(const BlkArgs& a, int cus, hipStream_t st) {
 
 // ---- the FFN half of a block as a kernel of its own: xo = x + act(h2 W0^T + b0) W2^T + b2 (+ LayerNorm) ------------
 // The FFN phase of blocks_env_kernel on plain rows: a wave owns 32 rows (two 16-row tiles; fp32 accumulator and the
-// LayerNorm-ed input as operand fragments in registers), a workgroup is 8 waves = 256 rows, one workgroup per CU; the
+// LayerNorm-ed input as operand fragments in registers), a workgroup is 4 waves = 128 rows, two per CU (d = 256: 8 waves, one); the
 // weight chunks stream through the same direct-to-LDS ring from a pre-permuted image (stage order W1(0), {W1(ch+1),
 // W2(ch)}..., W2(last), admitted in pairs), every fragment feeds both row tiles, the 32-unit hidden chunk lives in
 // accumulators and goes into the down-projection as one operand fragment.  Rounding points are those of the
