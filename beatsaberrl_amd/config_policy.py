@@ -296,17 +296,24 @@ class ConfigPolicy(nn.Module):
         if obs.dtype not in (torch.float32, dt):
             obs = obs.float()
         x = self._tokens(obs, r, dt)                                                          # (B, T, d)
-        for blk, w in zip(self.blocks, r["blk"]):
-            h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
+        h = None                                                # LN1 of the block, when the previous block's FFN kernel wrote it
+        for i, (blk, w) in enumerate(zip(self.blocks, r["blk"])):
+            if h is None:
+                h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
             qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                       # (B, T, 3d)
             att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
             x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                           # x + out(att)
             h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)
-            fused = None
+            fused = h = None
             if dt is not torch.float32 and ops.ffn_fused_profitable(d, self.ffn_dim, dt):
-                fused = ops.ffn_fused(x, h2, w["w0"], w["b0"], w["w2"], w["b2"], act=self.act)
+                # the fused kernel also writes the next block's LN1 (same arithmetic as ln_fwd on the rounded stream)
+                nxt = self.blocks[i + 1].ln_attn if i + 1 < len(self.blocks) else None
+                fused = ops.ffn_fused(x, h2, w["w0"], w["b0"], w["w2"], w["b2"], act=self.act,
+                                      ln_w=nxt.weight.detach() if nxt is not None else None,
+                                      ln_b=nxt.bias.detach() if nxt is not None else None,
+                                      eps=nxt.eps if nxt is not None else 1e-5)
             if fused is not None:
-                x = fused[0]
+                x, h = fused
             else:
                 hid = ops.linear(h2, w["w0"], w["b0"], act=self.act)                          # (B, T, ffn)
                 x = ops.linear(hid, w["w2"], w["b2"], residual=x)

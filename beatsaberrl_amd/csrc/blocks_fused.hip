@@ -447,11 +447,12 @@ __device__ __forceinline__ void env_ring_load3(uint32_t voff, const void* sbase,
 // stage slots deep.  Stages are entered in PAIRS (every block has an even number of them): one wait + barrier admits
 // two stages and refills the two slots behind them, so all but those four slots may be in flight (AHEAD).  A loading
 // wave moves FPW ADJACENT fragments of every stage (eight waves: SF = 8 one each; 12: six waves two each; 16: two each;
-// four waves: 8: two each; 12: three each); image and ring are addressed by running byte offsets, no multiplies in the
-// loop.
+// four waves: 8: two each; 12: three each; 24: six each); image and ring are addressed by running byte offsets, no
+// multiplies in the loop.
 template <int SF_, int SLOTS_, int NW_ = 8> struct StageRing {
     static constexpr int NW = NW_, SF = SF_, SLOTS = SLOTS_, AHEAD = SLOTS - 4;
-    static constexpr int FPW = (SF + NW - 1) / NW <= 1 ? 1 : SF % 2 == 0 && SF / 2 <= NW ? 2 : 3, NLW = SF / FPW;
+    static constexpr int FPW = (SF + NW - 1) / NW <= 1 ? 1 : SF % 2 == 0 && SF / 2 <= NW ? 2 : SF % 3 == 0 && SF / 3 <= NW ? 3 : 6;
+    static constexpr int NLW = SF / FPW;               // FPW = 6: two transfers of three (the immediate offset ends at 4095)
     static constexpr uint32_t STAGE_BYTES = SF * 1024;
     static_assert(SLOTS >= 5 && FPW * NLW == SF && NLW <= NW && FPW * (AHEAD + 2) < 64, "fragment split; vmcnt is 6 bits");
     const uint4* ring;             // slot 0
@@ -464,7 +465,10 @@ template <int SF_, int SLOTS_, int NW_ = 8> struct StageRing {
 
     __device__ __forceinline__ void issue(uint32_t slot_off) {
         if (NLW == NW || loader) {
-            if constexpr (FPW == 3) env_ring_load3(voff, wsrc + src_off, wdst + slot_off);
+            if constexpr (FPW == 6) {
+                env_ring_load3(voff, wsrc + src_off, wdst + slot_off);
+                env_ring_load3(voff, wsrc + src_off + 3072, wdst + slot_off + 3072);
+            } else if constexpr (FPW == 3) env_ring_load3(voff, wsrc + src_off, wdst + slot_off);
             else if constexpr (FPW == 2) env_ring_load2(voff, wsrc + src_off, wdst + slot_off);
             else env_ring_load(voff, wsrc + src_off, wdst + slot_off);
         }
@@ -1000,10 +1004,13 @@ struct FfnArgs {
 // Eight waves, one workgroup per CU - or four waves, TWO workgroups per CU (d = 128 / 192, where two rings fit): the
 // waves of a workgroup walk the ring in lockstep, so all of them load and store their rows at the same time with
 // nothing to run meanwhile; a second, independent workgroup drifts out of phase and computes through it.
-template <int D, int NW> struct FfnRing : StageRing<Geo<D>::SF, NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : 6), NW> {};
+// d = 384: a wave's state (fp32 accumulator 192 registers, input fragments 96) wants the whole register file of a SIMD:
+// four waves, ONE workgroup per CU, 512 registers each; stages of 24 KB.
+template <int D, int NW> struct FfnRing : StageRing<Geo<D>::SF, NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : D == 192 ? 6 : 5), NW> {};
+template <int D, int NW> constexpr int ffn_wgs_per_cu() { return D == 384 ? 1 : 8 / NW; }
 
 template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_>
-__global__ __launch_bounds__(NW_ * 64, 8 / NW_) void ffn_rows_kernel(FfnArgs a) {
+__global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
     typedef FfnRing<D, NW_> R;
     constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
@@ -1199,9 +1206,9 @@ __global__ __launch_bounds__(256) void ffn_pack_frags_kernel(FfnPackArgs a) {
 }
 
 bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
-    if (d != 128 && d != 192 && d != 256) return false;
+    if (d != 128 && d != 192 && d != 256 && d != 384) return false;
     if (F < 64 || F % 32 != 0 || F > 16384 || (dtype != BSRL_F16 && dtype != BSRL_BF16)) return false;
-    const int slots = d == 128 ? 10 : d == 192 ? 7 : 6;
+    const int slots = d == 128 ? 10 : d == 192 ? 7 : d == 256 ? 6 : 5;
     return 2 * (F / 32) >= slots;
 }
 int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
@@ -1211,8 +1218,9 @@ template <int D, int NW> size_t ffn_dyn_bytes(int F) {
 template <typename DT, int D, int ACT, int NW>
 int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
     const size_t dyn = ffn_dyn_bytes<D, NW>(a.F);
-    if ((8 / NW) * (dyn + 1024) > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
-    const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32), slots = (int64_t)cus * (8 / NW);
+    constexpr int WGS = ffn_wgs_per_cu<D, NW>();
+    if (WGS * (dyn + 1024) > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
+    const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32), slots = (int64_t)cus * WGS;
     const dim3 grid((unsigned)(ntiles < slots ? ntiles : slots));
     auto launch = [&](auto kern) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
@@ -1225,14 +1233,16 @@ int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
 }
 template <typename DT, int D, int ACT>
 int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
-    if constexpr (D != 256) {
+    if constexpr (D == 384) return ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
+    else if constexpr (D != 256) {
         // two 4-wave workgroups per CU where two rings fit and the image is longer than the shorter ring
         if (a.total_stages >= FfnRing<D, 4>::SLOTS) {
             const int rc = ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
             if (rc != BSRL_UNSUPPORTED) return rc;
         }
     }
-    return ffn_launch_nw<DT, D, ACT, 8>(a, ln, cus, st);
+    if constexpr (D != 384) return ffn_launch_nw<DT, D, ACT, 8>(a, ln, cus, st);
+    return BSRL_UNSUPPORTED;
 }
 
 }  // namespace
@@ -1254,7 +1264,8 @@ extern "C" int bsrl_ffn_pack(const void* w0, const float* b0, const void* w2, co
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (d == 128) hipLaunchKernelGGL(ffn_pack_frags_kernel<128>, grid, dim3(256), 0, st, pa);
     else if (d == 192) hipLaunchKernelGGL(ffn_pack_frags_kernel<192>, grid, dim3(256), 0, st, pa);
-    else hipLaunchKernelGGL(ffn_pack_frags_kernel<256>, grid, dim3(256), 0, st, pa);
+    else if (d == 256) hipLaunchKernelGGL(ffn_pack_frags_kernel<256>, grid, dim3(256), 0, st, pa);
+    else hipLaunchKernelGGL(ffn_pack_frags_kernel<384>, grid, dim3(256), 0, st, pa);
     BSRL_CHECK_LAUNCH("bsrl_ffn_pack");
     return BSRL_OK;
 }
@@ -1289,9 +1300,12 @@ extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2,
     } else if (d == 192) {
         if (f16) rc = relu ? ffn_launch<F16, 192, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 192, BSRL_ACT_GELU>(a, ln, cus, st);
         else rc = relu ? ffn_launch<BF16, 192, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 192, BSRL_ACT_GELU>(a, ln, cus, st);
-    } else {
+    } else if (d == 256) {
         if (f16) rc = relu ? ffn_launch<F16, 256, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 256, BSRL_ACT_GELU>(a, ln, cus, st);
         else rc = relu ? ffn_launch<BF16, 256, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 256, BSRL_ACT_GELU>(a, ln, cus, st);
+    } else {
+        if (f16) rc = relu ? ffn_launch<F16, 384, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<F16, 384, BSRL_ACT_GELU>(a, ln, cus, st);
+        else rc = relu ? ffn_launch<BF16, 384, BSRL_ACT_RELU>(a, ln, cus, st) : ffn_launch<BF16, 384, BSRL_ACT_GELU>(a, ln, cus, st);
     }
     if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH("bsrl_ffn_packed");

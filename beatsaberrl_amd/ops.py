@@ -350,13 +350,13 @@ def ffn_fused_supported(d, F, dtype) -> bool:
 
 
 def ffn_fused_profitable(d, F, dtype) -> bool:
-    """Is the fused FFN kernel the faster route?  Measured on MI355X (fp16, 475k rows, FFN + next LayerNorm):
-    d = 128 (F = 512): 0.31 ms fused vs 0.31 + 0.06 ms for the two linears + LayerNorm; d = 192 (F = 768): 0.81 vs
-    0.54 + 0.09 (streaming / ring-buffered linears); d = 256: 4.0 vs 2.7 at 3.1M rows; d = 384: 44 vs 16.5 - past
-    d = 128 the per-workgroup row tile that fits in registers is too small for the weight stream, so the unfused
-    pair (hidden through HBM) wins."""
+    """Is the fused FFN kernel the faster route?  Measured on MI355X (fp16, FFN + next LayerNorm): the packed-image
+    kernel wins wherever it exists - 0.25 ms against 0.38 for two Linears + LayerNorm at d = 128 (F = 512, 475k rows),
+    0.39 against 0.62 at d = 192, 1.27 against 1.80 at d = 256 (1M rows), 10.3 against 11.7 at d = 384 (3.1M rows, GELU);
+    the kernel on the plain weights only at d = 128 (0.33 against 0.38 ms; 0.82 against 0.62 at d = 192, 44 against 11.7 at
+    d = 384: its per-workgroup row tile is too small for the weight stream)."""
     if ffn_pack_supported(d, F, dtype):
-        return True          # the packed-image kernel: 0.33 ms at d = 192 (F = 768), 0.2 ms at d = 128 for the same rows
+        return True
     return d <= 128 and ffn_fused_supported(d, F, dtype)
 
 
@@ -400,8 +400,8 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5,
     Returns (xo, ho) (ho None without LN), or None when unsupported.
     want_hidden (packed route only; None is returned where that route has no kernel): (xo, ho, hid) with hid (.., F) the
     activated hidden as the down-projection consumed it, for a backward (the reference's save mode).
-    packed: "auto" takes the packed-image kernel (bsrl_ffn_packed: d <= 256, weights streamed straight into LDS,
-    32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter."""
+    packed: "auto" takes the packed-image kernel (bsrl_ffn_packed: d in {128, 192, 256, 384}, weights streamed straight
+    into LDS, 32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter."""
     _need_cuda(x, h2, w0, w2)
     d = x.shape[-1]
     Fh = w0.shape[0]

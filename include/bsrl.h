@@ -141,9 +141,9 @@ int bsrl_ffn_fused(const void* x, const void* h2, const void* w0, const float* b
  * (d, F, dtype) combination has a kernel. */
 int bsrl_ffn_fused_supported(int64_t d, int64_t F, int dtype);
 /* The same operation (fp16_gemm.ffn_fused, fused_ffn.cu:551-619; same rounding points) from a
- * weight image in MFMA fragment order, for d in {128, 192, 256} and F a multiple of 32 with
- * F/16 >= 10 / 7 / 6 (d = 128 / 192 / 256): the weights stream straight into LDS and a wave owns
- * 32 rows.  bsrl_ffn_pack writes the image (bsrl_ffn_pack_size bytes, 16-byte aligned; 0 =
+ * weight image in MFMA fragment order, for d in {128, 192, 256, 384} and F a multiple of 32 with
+ * F/16 >= 10 / 7 / 6 / 5 (d = 128 / 192 / 256 / 384): the weights stream straight into LDS and a
+ * wave owns 32 rows.  bsrl_ffn_pack writes the image (bsrl_ffn_pack_size bytes, 16-byte aligned; 0 =
  * unsupported shape) from w0 (F, d) and w2 (d, F) in `dtype` and the fp32 biases - once per
  * weight update, like the 16-bit replicas the reference keeps (python/fp16_linear.py:150-192);
  * bsrl_ffn_packed is bsrl_ffn_fused with the image in place of w0, b0, w2, b2.  x, h2, xo, ho

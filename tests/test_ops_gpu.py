@@ -221,9 +221,9 @@ def test_linear_rows_are_batch_invariant():
 def test_ffn_fused(dtype, rows, d, Fh, act, with_ln, packed):
     """Closed form with the reference's rounding points (python/tests/test_fused_ffn.py:252-266):
     hidden rounded once, fp32 accumulate, out = round(x + (O + b2)), LN on the rounded out.  Both kernels: the one on
-    a packed weight image (d <= 256 with enough FFN stages; `packed="auto"`) and the one on the plain weights."""
+    a packed weight image (d = 128 / 192 / 256 / 384 with enough FFN stages; `packed="auto"`) and the one on the plain weights."""
     assert ops.ffn_fused_supported(d, Fh, dtype)
-    assert ops.ffn_pack_supported(d, Fh, dtype) == (d <= 256 and Fh >= 192)
+    assert ops.ffn_pack_supported(d, Fh, dtype) == (Fh >= 192)
     x = _rand(rows, d, dtype=dtype, seed=1)
     h2 = _rand(rows, d, dtype=dtype, seed=2)
     w0 = _rand(Fh, d, dtype=dtype, seed=3, scale=1 / math.sqrt(d))
