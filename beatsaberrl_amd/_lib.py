@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 13
+ABI_VERSION = 14
 CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
 CFG_NO_LATENCY = 2              # bsrl_cfg_desc.flags: small batches take the throughput forms too
 CFG_STATIC_MAX_ENVS = 16384     # BSRL_CFG_STATIC_MAX_ENVS: batch limit of bsrl_cfg_forward_static
@@ -55,6 +55,7 @@ SIGNATURES = {
                            _i32, _i32, _i32, _p]),
     "bsrl_linear_grouped": (_i32, [_p, _i64, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64,
                                    _i32, _i32, _i32, _i64, _i64, _p]),
+    "bsrl_mlp2": (_i32, [_p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _i64, _i64, _p]),
     "bsrl_attn_fwd": (_i32, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _p,
                              _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "bsrl_ffn_fused": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _f, _p, _p, _i64, _i64, _i64, _i32, _i32, _p]),

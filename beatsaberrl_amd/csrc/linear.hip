@@ -300,6 +300,24 @@ extern "C" int bsrl_linear_grouped(const void* x, int64_t ldx, const void* w, co
     return lin_dispatch(a, act, dtype, out_dtype, static_cast<hipStream_t>(stream), "bsrl_linear");
 }
 
+extern "C" int bsrl_mlp2(const void* x, int64_t ldx, const void* w1, const float* b1, int64_t K1, const void* w2,
+                         const float* b2, void* y, int64_t ldy, int64_t rows, int64_t d, int dtype, int64_t y_group_rows,
+                         int64_t y_group_stride, bsrl_stream stream) {
+    if (!x || !w1 || !b1 || !w2 || !b2 || !y) BSRL_FAIL(BSRL_EINVAL, "bsrl_mlp2: null pointer");
+    if (rows < 0 || K1 <= 0 || d <= 0 || K1 > (1 << 20) || d > (1 << 20))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_mlp2: bad shape rows=%lld K1=%lld d=%lld", (long long)rows, (long long)K1, (long long)d);
+    if (ldx < K1 || ldy < d) BSRL_FAIL(BSRL_EINVAL, "bsrl_mlp2: row stride smaller than row");
+    if (dtype != BSRL_F32 && dtype != BSRL_F16 && dtype != BSRL_BF16) BSRL_FAIL(BSRL_EINVAL, "bsrl_mlp2: bad dtype");
+    if (y_group_rows < 0 || (y_group_rows > 0 && (rows % y_group_rows != 0 || y_group_rows > (1 << 20) || y_group_stride < y_group_rows * ldy)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_mlp2: groups need rows %% group == 0 and group stride >= group * ldy");
+    if (dtype == BSRL_F32) return BSRL_UNSUPPORTED;
+    if (rows == 0) return BSRL_OK;
+    LinArgs l2{nullptr, 0, w2, b2, nullptr, 0, y, ldy, nullptr, 0, 0, rows, (int)d, (int)d, 0, (int)y_group_rows, y_group_stride, nullptr, 0};
+    if (!bsrl_mlp2_stream(l2, x, ldx, w1, b1, K1, dtype, static_cast<hipStream_t>(stream))) return BSRL_UNSUPPORTED;
+    BSRL_CHECK_LAUNCH("bsrl_mlp2");
+    return BSRL_OK;
+}
+
 extern "C" int bsrl_linear_gated(const void* x, int64_t ldx, const void* w, const void* gate, int64_t ldgate,
                                  void* y, int64_t ldy, int64_t rows, int64_t K, int64_t M, int dtype,
                                  bsrl_stream stream) {

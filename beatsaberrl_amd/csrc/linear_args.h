@@ -34,6 +34,11 @@ bool bsrl_linear_tiled(const LinArgs& a, int act, int dtype, hipStream_t st);
 // false when the shape is outside what it covers.
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st);
 
+// Two Linears with a ReLU between them in one launch (linear_stream.hip): x (rows, K1) -> relu(x W1^T + b1) -> l2 (its
+// w, bias, y, grouping; K = M = d); false when the shape is outside what it covers (K1 = 64, d = 128 / 192, 16-bit).
+bool bsrl_mlp2_stream(const LinArgs& l2, const void* x, int64_t ldx, const void* w1, const float* b1, int64_t K1, int dtype,
+                      hipStream_t st);
+
 // Ring-buffered 16-bit kernel for large row counts and K a multiple of 32 (linear_ring.hip): operands go from
 // global memory straight into an LDS ring; false when the shape is outside what it covers.
 bool bsrl_linear_ring(const LinArgs& a, int act, int dtype, hipStream_t st);

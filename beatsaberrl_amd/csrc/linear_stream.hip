@@ -177,6 +177,152 @@ __global__ __launch_bounds__(ST_THREADS) void linear_stream_kernel(LinArgs a, in
 }
 #undef ST_FETCH
 
+// ---- two Linears with a ReLU between them in one launch: y = (relu(x W1^T + b1)) W2^T + b2 ----------------------------
+// The policy's token encoders (python/policy.py:1224-1249: Linear(in, d) ReLU Linear(d, d), in <= 64 lanes, padded to 64)
+// as the streaming kernel twice over without the trip through HBM in between: both weights resident in LDS in fragment
+// order, a wave streams 32-row tiles of x, and the first Linear's rounded output - the same 16 x d row tile that
+// linear_stream_kernel would store - is read back from the wave's LDS tile as the second Linear's operand fragments.
+// Every step is the arithmetic of the two separate launches (fp32 accumulate from zero in ascending k, + bias,
+// ReLU, one rounding; fp32 accumulate, + bias, one rounding): the same bits.  Output rows may be grouped (LinArgs).
+struct Mlp2Args {
+    LinArgs l2;                  // the second Linear: w, bias, y / ldy / y_group / y_gstride, rows, K = M = d
+    const void* x; int64_t ldx;  // (rows, 32 KC1) 16-bit
+    const void* w1; const float* b1;      // (d, 32 KC1) 16-bit, (d) fp32
+};
+
+template <typename DT, int KC1, int KC, int MT>
+__global__ __launch_bounds__(ST_THREADS) void mlp2_stream_kernel(Mlp2Args a, int walkers) {
+    static_assert(MT * 16 == KC * 32, "the hidden width is the second Linear's K");
+    extern __shared__ __attribute__((aligned(16))) uint4 wl[];   // W1 [MT * KC1][64], W2 [MT * KC][64], b1, b2, 8 wave tiles
+    constexpr int KE = KC * 32, K1 = KC1 * 32;
+    constexpr int TP = KE + 8;                                    // wave tile row pitch (elements)
+    constexpr int PPR1 = K1 / 8;                                  // 16-byte pieces per x row
+    constexpr int NLD = (16 * PPR1 + WAVE - 1) / WAVE;
+    static_assert(16 * PPR1 == NLD * WAVE, "16 rows of x are whole wave loads");
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int walker = blockIdx.x;
+    uint4* wl2 = wl + MT * KC1 * 64;
+    {   // resident weights: fragment (mt, kc), lane l <- W[16 mt + l % 16][32 kc + 8 (l / 16) .. + 7]
+        const u16* w1 = static_cast<const u16*>(a.w1);
+        const u16* w2 = static_cast<const u16*>(a.l2.w);
+        for (int i = tid; i < MT * KC1 * 64; i += ST_THREADS) {
+            const int l = i & 63, f = i >> 6, mt = f / KC1, kc = f % KC1;
+            wl[i] = *reinterpret_cast<const uint4*>(w1 + (int64_t)(mt * 16 + (l & 15)) * K1 + kc * 32 + 8 * (l >> 4));
+        }
+        for (int i = tid; i < MT * KC * 64; i += ST_THREADS) {
+            const int l = i & 63, f = i >> 6, mt = f / KC, kc = f % KC;
+            wl2[i] = *reinterpret_cast<const uint4*>(w2 + (int64_t)(mt * 16 + (l & 15)) * KE + kc * 32 + 8 * (l >> 4));
+        }
+    }
+    float* bl1 = reinterpret_cast<float*>(wl2 + MT * KC * 64);
+    float* bl2 = bl1 + MT * 16;
+    u16* wt = reinterpret_cast<u16*>(bl2 + MT * 16) + wave * (16 * TP);
+    for (int i = tid; i < MT * 16; i += ST_THREADS) { bl1[i] = a.b1[i]; bl2[i] = a.l2.bias[i]; }
+    __syncthreads();                                              // the only barrier
+
+    const u16* x = static_cast<const u16*>(a.x);
+    u16* y = static_cast<u16*>(a.l2.y);
+    const int64_t rows = a.l2.rows, ntiles = (rows + ST_ROWS - 1) / ST_ROWS;
+    const int64_t stride = (int64_t)walkers * 8;
+    int64_t tile = (int64_t)walker * 8 + wave;
+    if (tile >= ntiles) return;
+    u32x4 pa[NLD], pb[NLD];
+#define M2_FETCH(t)                                                                                                   \
+    _Pragma("unroll") for (int it = 0; it < NLD; ++it) {                                                               \
+        const int p = it * WAVE + lane, r = p / PPR1, part = p % PPR1;                                                \
+        int64_t ra = (t) * ST_ROWS + r, rb = ra + 16;                                                                 \
+        ra = ra < rows ? ra : rows - 1;                                                                               \
+        rb = rb < rows ? rb : rows - 1;                                                                               \
+        pa[it] = *reinterpret_cast<const u32x4*>(x + ra * a.ldx + part * 8);                                          \
+        pb[it] = *reinterpret_cast<const u32x4*>(x + rb * a.ldx + part * 8);                                          \
+    }
+    M2_FETCH(tile)
+    for (; tile < ntiles; tile += stride) {
+        u32x4 hf[2][KC];                                          // the hidden rows as operand fragments
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            // x rows -> fragments through the wave tile
+            u32x4 xf[KC1];
+#pragma unroll
+            for (int it = 0; it < NLD; ++it) {
+                const int p = it * WAVE + lane;
+                *reinterpret_cast<u32x4*>(wt + (p / PPR1) * TP + (p % PPR1) * 8) = rt == 0 ? pa[it] : pb[it];
+            }
+#pragma unroll
+            for (int kc = 0; kc < KC1; ++kc) xf[kc] = *reinterpret_cast<const u32x4*>(wt + r16 * TP + kc * 32 + 8 * g);
+            // first Linear + ReLU, rounded, into the wave tile (row-major), two feature tiles at a time
+#pragma unroll
+            for (int mt = 0; mt < MT; mt += 2) {
+                f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kc = 0; kc < KC1; ++kc) {
+                    const s16x8 xv = __builtin_bit_cast(s16x8, xf[kc]);
+                    a0 = DT::mfma32(__builtin_bit_cast(s16x8, wl[(mt * KC1 + kc) * 64 + lane]), xv, a0);
+                    a1 = DT::mfma32(__builtin_bit_cast(s16x8, wl[((mt + 1) * KC1 + kc) * 64 + lane]), xv, a1);
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const f32x4 acc = h ? a1 : a0;
+                    const float4 bv = *reinterpret_cast<const float4*>(bl1 + (mt + h) * 16 + 4 * g);
+                    float o[4] = {acc[0] + bv.x, acc[1] + bv.y, acc[2] + bv.z, acc[3] + bv.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = keep_f32(apply_act16<BSRL_ACT_RELU>(o[e]));
+                    uint2 ov;
+                    ov.x = DT::pack2(o[0], o[1]);
+                    ov.y = DT::pack2(o[2], o[3]);
+                    *reinterpret_cast<uint2*>(wt + r16 * TP + (mt + h) * 16 + 4 * g) = ov;
+                }
+            }
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc) hf[rt][kc] = *reinterpret_cast<const u32x4*>(wt + r16 * TP + kc * 32 + 8 * g);
+        }
+        M2_FETCH(tile + stride)                                   // rows past the end clamp to the last row
+        // second Linear
+        f32x4 acc[MT][2];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) { acc[mt][0] = (f32x4){0.f, 0.f, 0.f, 0.f}; acc[mt][1] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const s16x8 x0 = __builtin_bit_cast(s16x8, hf[0][kc]), x1 = __builtin_bit_cast(s16x8, hf[1][kc]);
+#pragma unroll
+            for (int mt = 0; mt < MT; mt += 2) {
+                const s16x8 wf0 = __builtin_bit_cast(s16x8, wl2[(mt * KC + kc) * 64 + lane]);
+                const s16x8 wf1 = __builtin_bit_cast(s16x8, wl2[((mt + 1) * KC + kc) * 64 + lane]);
+                acc[mt][0] = DT::mfma32(wf0, x0, acc[mt][0]);
+                acc[mt][1] = DT::mfma32(wf0, x1, acc[mt][1]);
+                acc[mt + 1][0] = DT::mfma32(wf1, x0, acc[mt + 1][0]);
+                acc[mt + 1][1] = DT::mfma32(wf1, x1, acc[mt + 1][1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const float4 bv = *reinterpret_cast<const float4*>(bl2 + mt * 16 + 4 * g);
+                float o[4] = {acc[mt][rt][0] + bv.x, acc[mt][rt][1] + bv.y, acc[mt][rt][2] + bv.z, acc[mt][rt][3] + bv.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = keep_f32(o[e]);
+                uint2 ov;
+                ov.x = DT::pack2(o[0], o[1]);
+                ov.y = DT::pack2(o[2], o[3]);
+                *reinterpret_cast<uint2*>(wt + r16 * TP + mt * 16 + 4 * g) = ov;
+            }
+            constexpr int OPR = MT * 2;                           // 16-byte pieces per output row
+#pragma unroll 1
+            for (int c0 = 0; c0 < 16 * OPR; c0 += WAVE) {
+                const int c = c0 + lane;
+                const int r = c / OPR, pc = c % OPR;
+                const int64_t orow = tile * ST_ROWS + rt * 16 + r;
+                if (c < 16 * OPR && orow < rows)
+                    *reinterpret_cast<uint4*>(y + lin_yoff(a.l2, orow) + pc * 8) = *reinterpret_cast<const uint4*>(wt + r * TP + pc * 8);
+            }
+        }
+    }
+}
+#undef M2_FETCH
+
 int device_cus() {
     static const int cus = [] {
         int dev = 0, n = 0;
@@ -233,6 +379,23 @@ bool dispatch(const LinArgs& a, int act, hipStream_t st) {
     return by_k<DT, BSRL_ACT_NONE, 0>(a, st);
 }
 
+
+template <typename DT, int KC, int MT>
+bool mlp2_launch(const Mlp2Args& a, hipStream_t st) {
+    constexpr int KC1 = 2, TP = KC * 32 + 8;
+    const size_t lds = (size_t)MT * (KC1 + KC) * 1024 + (size_t)2 * MT * 16 * sizeof(float) + (size_t)8 * 16 * TP * sizeof(u16);
+    auto kern = mlp2_stream_kernel<DT, KC1, KC, MT>;
+    static const bool ready = [&] {
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess;
+    }();
+    if (!ready) { (void)hipGetLastError(); return false; }
+    const int64_t ntiles = (a.l2.rows + ST_ROWS - 1) / ST_ROWS;
+    int64_t walkers = device_cus();                               // one workgroup per CU (the resident weights fill its LDS)
+    const int64_t need = (ntiles + 7) / 8;
+    if (walkers > need) walkers = need;
+    hipLaunchKernelGGL(kern, dim3((unsigned)walkers), dim3(ST_THREADS), lds, st, a, (int)walkers);
+    return true;
+}
 }  // namespace
 
 bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st) {
@@ -244,4 +407,15 @@ bool bsrl_linear_stream(const LinArgs& a, int act, int dtype, hipStream_t st) {
     if (a.gate && (a.ldgate % 4 != 0 || !bsrl_aligned(a.gate, 8))) return false;
     if (a.bias && !bsrl_aligned(a.bias, 4)) return false;
     return dtype == BSRL_F16 ? dispatch<F16>(a, act, st) : dispatch<BF16>(a, act, st);
+}
+
+bool bsrl_mlp2_stream(const LinArgs& l2, const void* x, int64_t ldx, const void* w1, const float* b1, int64_t K1, int dtype,
+                      hipStream_t st) {
+    // 64 input lanes, d = 128 / 192, 16-bit in and out, 16-byte aligned rows, both biases present
+    if (K1 != 64 || l2.K != l2.M || (l2.M != 128 && l2.M != 192) || l2.out_f32 || l2.y2 || l2.res || l2.gate || !l2.bias || !b1) return false;
+    if (ldx % 8 != 0 || !bsrl_aligned(x, 16) || !bsrl_aligned(w1, 16) || !bsrl_aligned(l2.w, 16)) return false;
+    if (l2.ldy % 8 != 0 || l2.y_gstride % 8 != 0 || !bsrl_aligned(l2.y, 16) || l2.rows < 1 || l2.rows > 0x7fffffffLL) return false;
+    Mlp2Args a{l2, x, ldx, w1, b1};
+    if (dtype == BSRL_F16) return l2.M == 128 ? mlp2_launch<F16, 4, 8>(a, st) : mlp2_launch<F16, 6, 12>(a, st);
+    return l2.M == 128 ? mlp2_launch<BF16, 4, 8>(a, st) : mlp2_launch<BF16, 6, 12>(a, st);
 }

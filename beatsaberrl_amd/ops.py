@@ -238,6 +238,41 @@ def linear(x, w, bias=None, act=None, residual=None, out_dtype=None, split=None,
     return y if split is None else (y, y2)
 
 
+def mlp2_supported(K1, d, dtype) -> bool:
+    """Shapes bsrl_mlp2 covers: a 64-lane input, d = 128 / 192, 16-bit stream."""
+    return dtype in (torch.float16, torch.bfloat16) and K1 == 64 and d in (128, 192)
+
+
+def mlp2(x, w1, b1, w2, b2, out=None):
+    """relu(x w1^T + b1) w2^T + b2 in one launch (bsrl_mlp2; the hidden rows stay on the chip): bit for bit
+    linear(linear(x, w1, b1, act="relu"), w2, b2, out=out).  x (.., K1) contiguous, w1 (d, K1), w2 (d, d) in x's dtype,
+    b1 / b2 fp32; out: a (N, G, d) slice of a token stream that receives the rows (as in `linear`).  Returns None where
+    the shape has no kernel (the caller runs the two Linears)."""
+    _need_cuda(x, w1, w2, b1, b2)
+    K1, d = x.shape[-1], w2.shape[0]
+    if not mlp2_supported(K1, d, x.dtype):
+        return None
+    if not (x.is_contiguous() and w1.is_contiguous() and w2.is_contiguous()) or w1.dtype is not x.dtype or w2.dtype is not x.dtype:
+        raise TypeError("mlp2: x, w1, w2 must be contiguous in one dtype")
+    if tuple(w1.shape) != (d, K1) or tuple(w2.shape) != (d, d) or b1.numel() != d or b2.numel() != d:
+        raise TypeError(f"mlp2: expected w1 ({d}, {K1}), w2 ({d}, {d}), b1 / b2 ({d},)")
+    rows = x.numel() // K1
+    group, gstride = 0, 0
+    if out is None:
+        y = torch.empty(*x.shape[:-1], d, device=x.device, dtype=x.dtype)
+        ldy = d
+    else:
+        if out.dim() != 3 or out.shape[2] != d or out.stride(2) != 1 or out.dtype is not x.dtype or out.shape[0] * out.shape[1] != rows:
+            raise TypeError("mlp2: out must be a (N, G, d) view with unit last stride and N * G rows in x's dtype")
+        y = out
+        group, gstride = out.shape[1], out.stride(0)
+        ldy = out.stride(1) if group > 1 else d
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_mlp2(x.data_ptr(), K1, w1.data_ptr(), _ptr(_f32c(b1, "b1")), K1, w2.data_ptr(),
+                                   _ptr(_f32c(b2, "b2")), y.data_ptr(), ldy, rows, d, dt_code(x.dtype), group, gstride, _stream(x))
+    return y if _lib.check(rc, "bsrl_mlp2") else None
+
+
 def linear_gated(x, w, gate):
     """(x @ w.T) * [gate > 0]: the data gradient of a Linear masked by the ReLU before it, in one
     GEMM (reference fp16_gemm.dgrad_drelu, fp16_gemm.cu:479-518).  x (..., K), w (M, K) contiguous

@@ -81,6 +81,14 @@ def _seq(seq: nn.Sequential, x, out=None):
     receives the last Linear's rows directly.  x may be wider than the first Linear's input (rows
     zero-padded by the producer): the first weight's columns are then padded to match."""
     ms = list(seq)
+    if (len(ms) == 3 and isinstance(ms[0], nn.Linear) and isinstance(ms[1], nn.ReLU) and isinstance(ms[2], nn.Linear)
+            and x.shape[-1] >= ms[0].in_features and ms[0].bias is not None and ms[2].bias is not None
+            and ops.mlp2_supported(x.shape[-1], ms[2].out_features, x.dtype) and ms[0].out_features == ms[2].in_features == ms[2].out_features):
+        # Linear ReLU Linear on a 64-lane input: one launch, the hidden rows never written (same bits as the two below)
+        w1 = _fl._replica_padded(ms[0].weight, x.dtype, x.shape[-1]) if x.shape[-1] != ms[0].in_features else _fl._replica(ms[0].weight, x.dtype)
+        y = ops.mlp2(x.contiguous(), w1, _fl._bias32(ms[0].bias), _fl._replica(ms[2].weight, x.dtype), _fl._bias32(ms[2].bias), out=out)
+        if y is not None:
+            return y
     i = 0
     while i < len(ms):
         m = ms[i]

@@ -87,6 +87,15 @@ int bsrl_linear_grouped(const void* x, int64_t ldx, const void* w, const float* 
                         void* y2, int64_t ldy2, int64_t split,
                         int64_t rows, int64_t K, int64_t M, int act, int dtype, int out_dtype,
                         int64_t y_group_rows, int64_t y_group_stride, bsrl_stream stream);
+/* Two Linears with a ReLU between them in one launch: y = relu(x W1^T + b1) W2^T + b2 - a token encoder of the
+ * policy (python/policy.py:1224-1249, `_seq` / `_run` python/policy.py:76-145: Linear(in, d) ReLU Linear(d, d) through
+ * fp16_linear_relu and fp16_linear, python/fp16_linear.py:134-181), the hidden rows never written.  x (rows, K1) with
+ * row stride ldx, w1 (d, K1), w2 (d, d) in `dtype` (nn.Linear layout), b1 / b2 fp32 (d); y and its row grouping as
+ * in bsrl_linear_grouped.  Bit for bit what bsrl_linear(act = ReLU) followed by bsrl_linear_grouped gives.  16-bit
+ * dtypes, K1 = 64, d = 128 / 192, 16-byte aligned rows; BSRL_UNSUPPORTED otherwise (run the two Linears). */
+int bsrl_mlp2(const void* x, int64_t ldx, const void* w1, const float* b1, int64_t K1, const void* w2,
+              const float* b2, void* y, int64_t ldy, int64_t rows, int64_t d, int dtype,
+              int64_t y_group_rows, int64_t y_group_stride, bsrl_stream stream);
 
 /* ---- Short-sequence masked multi-head attention ----------------------------
  * Replaces fp16_gemm.attn29_fwd (small_attn.cu:515-536) and the SDPA / fp32

@@ -723,3 +723,35 @@ def test_softmax_expect_matches_float64(rows, n):
         ops.softmax_expect(logits.to(DEV).half(), centers.to(DEV))
     with pytest.raises(TypeError):
         ops.softmax_expect(logits.to(DEV), centers[:-1].to(DEV) if n > 1 else torch.zeros(2, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d", [128, 192])
+@pytest.mark.parametrize("rows,group", [(1, 0), (77, 0), (4099, 0), (24 * 700, 24), (2 * 9001, 2), (65536, 0)])
+def test_mlp2_is_the_two_linears_bit_for_bit(dtype, d, rows, group):
+    """bsrl_mlp2 (Linear ReLU Linear on a 64-lane input in one launch, hidden rows never written) against
+    linear(act="relu") followed by linear: the same bits, plain and into a token slice of a (B, T, d) stream; and
+    against the float64 closed form with the hidden rounded once (python/tests/test_fused_ffn.py:252-266 style)."""
+    x = _rand(rows, 64, dtype=dtype, seed=1)
+    x[:, 40:] = 0                                                 # the frontend pads the encoder inputs with zeros
+    w1 = _rand(d, 64, dtype=dtype, seed=2, scale=1 / math.sqrt(40))
+    w2 = _rand(d, d, dtype=dtype, seed=3, scale=1 / math.sqrt(d))
+    b1, b2 = _rand(d, seed=4) * 0.3, _rand(d, seed=5) * 0.3
+    assert ops.mlp2_supported(64, d, dtype) and not ops.mlp2_supported(40, d, dtype) and not ops.mlp2_supported(64, 256, dtype)
+    if group:
+        B, T = rows // group, group + 5
+        s1 = torch.full((B, T, d), 7.0, device=DEV, dtype=dtype)
+        s0 = s1.clone()
+        y1 = ops.mlp2(x, w1, b1, w2, b2, out=s1[:, 5:])
+        ops.linear(ops.linear(x, w1, b1, act="relu"), w2, b2, out=s0[:, 5:])
+        assert y1 is not None and torch.equal(s1, s0)
+        assert bool((s1[:, :5] == 7.0).all())                     # rows outside the slice untouched
+        got = s1[:, 5:].reshape(rows, d)
+    else:
+        got = ops.mlp2(x, w1, b1, w2, b2)
+        want = ops.linear(ops.linear(x, w1, b1, act="relu"), w2, b2)
+        assert got is not None and torch.equal(got, want)
+    hid = torch.relu(x.double() @ w1.double().t() + b1.double()).to(dtype).double()
+    ref = hid @ w2.double().t() + b2.double()
+    scale = ref.abs().max().item()
+    assert (got.double() - ref).abs().max().item() <= 1.5 * EPS16[dtype] * scale
