@@ -20,6 +20,7 @@ from __future__ import annotations
 
 import torch
 
+from . import fp16_linear as _fl
 from . import ops
 
 
@@ -188,16 +189,34 @@ class FusedFfnFn(torch.autograd.Function):
     forward and backward).  Shapes without the packed-image kernel always recompute."""
 
     @staticmethod
+    def _image(w0, b0, w2, b2, w0h, b0f, w2h, b2f):
+        """The packed kernel's weight image for the update path: one buffer per FFN (held on its first master
+        weight), repacked only when a master has changed - torch's in-place counters of the four masters (every
+        optimizer step and load moves them) and the global weights version make the key - instead of once per
+        forward call from the freshly cast copies."""
+        if not ops.ffn_pack_supported(w0h.shape[1], w0h.shape[0], w0h.dtype):
+            return None
+        key = (_fl._weights_version, w0._version, b0._version, w2._version, b2._version, w0h.dtype, str(w0h.device))
+        cache = getattr(w0, "_bsrl_ffn_image_train", None)
+        if cache is None:
+            cache = w0._bsrl_ffn_image_train = [None, None]
+        if cache[0] != key:
+            cache[1] = ops.ffn_pack_into(cache[1], w0h, b0f, w2h, b2f)
+            cache[0] = key
+        return cache[1]
+
+    @staticmethod
     def forward(ctx, x, h2, w0, b0, w2, b2, save_hidden=False):
         w0h, w2h = _w_for(w0, x.dtype), _w_for(w2, x.dtype)
         b0f, b2f = b0.detach().float().contiguous(), b2.detach().float().contiguous()
         xc, hc = x.contiguous(), h2.contiguous()
-        r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu", want_hidden=True) if save_hidden else None
+        img = FusedFfnFn._image(w0, b0, w2, b2, w0h, b0f, w2h, b2f)
+        r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu", want_hidden=True, image=img) if save_hidden else None
         hid = None
         if r is not None:
             hid = r[2]
         else:
-            r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu")
+            r = ops.ffn_fused(xc, hc, w0h, b0f, w2h, b2f, act="relu", image=img)
         if r is None:
             raise ops.Unsupported(f"fused FFN d={x.shape[-1]} F={w0.shape[0]} dtype={x.dtype}")
         ctx.has_hid = hid is not None

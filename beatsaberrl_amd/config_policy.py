@@ -121,6 +121,10 @@ class ConfigPolicy(nn.Module):
                 "out_w": c(blk.out_proj.weight), "out_b": f(blk.out_proj.bias),
                 "w0": c(blk.ffn[0].weight), "b0": f(blk.ffn[0].bias),
                 "w2": c(blk.ffn[2].weight), "b2": f(blk.ffn[2].bias)})
+            w = r["blk"][-1]
+            # the packed fused FFN's weight image lives with the replicas it was built from (one per weights version)
+            w["ffn_img"] = (ops.ffn_pack_into(None, w["w0"], w["b0"], w["w2"], w["b2"])
+                            if ops.ffn_pack_supported(self.d, self.ffn_dim, dt) else None)
         self._replica = (key, r)
         return r
 
@@ -311,7 +315,7 @@ class ConfigPolicy(nn.Module):
                 fused = ops.ffn_fused(x, h2, w["w0"], w["b0"], w["w2"], w["b2"], act=self.act,
                                       ln_w=nxt.weight.detach() if nxt is not None else None,
                                       ln_b=nxt.bias.detach() if nxt is not None else None,
-                                      eps=nxt.eps if nxt is not None else 1e-5)
+                                      eps=nxt.eps if nxt is not None else 1e-5, image=w["ffn_img"])
             if fused is not None:
                 x, h = fused
             else:

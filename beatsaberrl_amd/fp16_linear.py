@@ -226,6 +226,25 @@ def fused_ffn_ok(x, ffn, ln=None) -> bool:
     return ops.ffn_fused_profitable(ffn[0].in_features, ffn[0].out_features, x.dtype)
 
 
+def ffn_image(ffn, dtype):
+    """The packed fused FFN's weight image of a Linear-act-Linear Sequential, or None where the shape has no packed
+    kernel.  ONE buffer per module, rebuilt IN PLACE from the (in-place) replicas once per weights version: like the
+    replicas themselves (reference :367-375) its address never moves, so a captured graph that holds it follows every
+    refresh_fp16_caches / bump_weights_version."""
+    w0, w2 = ffn[0].weight, ffn[2].weight
+    if dtype is torch.float32 or not ops.ffn_pack_supported(ffn[0].in_features, ffn[0].out_features, dtype):
+        return None
+    cache = getattr(w0, "_bsrl_ffn_image", None)
+    if cache is None or cache[1] is not dtype or cache[2].device != w0.device:
+        cache = [-1, dtype, None]
+        w0._bsrl_ffn_image = cache
+    if cache[0] != _weights_version or cache[2] is None:
+        cache[2] = ops.ffn_pack_into(cache[2], _replica(w0, dtype), _bias32(ffn[0].bias), _replica(w2, dtype),
+                                     _bias32(ffn[2].bias))
+        cache[0] = _weights_version
+    return cache[2]
+
+
 def fused_ffn(x, h2, ffn, ln=None):
     """out = x + ffn(h2) [, LayerNorm_ln(out)] in one kernel (reference :1254-1275).
     Returns out, or (out, ln(out)) when ln is given."""
@@ -233,7 +252,7 @@ def fused_ffn(x, h2, ffn, ln=None):
     r = ops.ffn_fused(x.contiguous(), h2.contiguous(), _replica(ffn[0].weight, x.dtype), _bias32(ffn[0].bias),
                       _replica(ffn[2].weight, x.dtype), _bias32(ffn[2].bias), act=act,
                       ln_w=None if ln is None else ln.weight, ln_b=None if ln is None else ln.bias,
-                      eps=1e-5 if ln is None else ln.eps)
+                      eps=1e-5 if ln is None else ln.eps, image=ffn_image(ffn, x.dtype))
     if r is None:
         raise ops.Unsupported("fused_ffn: call fused_ffn_ok first")
     return r[0] if ln is None else r

@@ -399,44 +399,58 @@ def ffn_pack_supported(d, F, dtype) -> bool:
     return dtype in (torch.float16, torch.bfloat16) and _lib.load().bsrl_ffn_pack_size(d, F, dt_code(dtype)) > 0
 
 
-# weight images of ffn_fused's packed route, keyed by the identity and in-place version of the four tensors (the
-# 16-bit replicas are rewritten or replaced after every optimizer step: either changes the key); a few entries only
-_FFN_IMAGES: dict = {}
-_FFN_IMAGES_MAX = 64
-
-
-def ffn_pack(w0, b0, w2, b2):
-    """Weight image of the packed fused FFN (bsrl_ffn_pack) from w0 (F, d), w2 (d, F) in a 16-bit dtype and the fp32
-    biases; cached while the four tensors are unchanged."""
-    key = tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) for t in (w0, b0, w2, b2))
-    img = _FFN_IMAGES.get(key)
-    if img is not None:
-        return img
+def ffn_pack_into(img, w0, b0, w2, b2):
+    """(Re)build the packed fused FFN's weight image (bsrl_ffn_pack) from w0 (F, d), w2 (d, F) in a 16-bit dtype and
+    the fp32 biases INTO `img` (a uint8 buffer of bsrl_ffn_pack_size bytes; None: a new one is allocated) and return
+    it.  The owner of a stable image - a module whose forward a captured graph may replay - calls this once per weights
+    version with the same buffer, so the address the graph holds never moves and never goes stale."""
     Fh, d = w0.shape
     n = _lib.load().bsrl_ffn_pack_size(d, Fh, dt_code(w0.dtype))
     if n <= 0:
         raise Unsupported(f"ffn_pack d={d} F={Fh} dtype={w0.dtype}")
-    img = torch.empty(n, dtype=torch.uint8, device=w0.device)
+    if img is None or img.numel() != n or img.device != w0.device:
+        img = torch.empty(n, dtype=torch.uint8, device=w0.device)
     with torch.cuda.device(w0.device):
         rc = _lib.load().bsrl_ffn_pack(w0.data_ptr(), _f32c(b0, "b0").data_ptr(), w2.data_ptr(), _f32c(b2, "b2").data_ptr(),
                                        d, Fh, dt_code(w0.dtype), img.data_ptr(), _stream(w0))
     if not _lib.check(rc, "bsrl_ffn_pack"):
         raise Unsupported(f"ffn_pack d={d} F={Fh} dtype={w0.dtype}")
-    if len(_FFN_IMAGES) >= _FFN_IMAGES_MAX:
-        _FFN_IMAGES.clear()
+    return img
+
+
+# Weight images for EAGER callers that hand ffn_fused bare tensors (tests, ConfigPolicy's per-op route), keyed by the
+# identity and in-place version of the four tensors.  A refresh of the tensors changes the key and a NEW image is
+# built, and old entries are dropped one by one: nothing here is safe to hold in a captured graph - callers that
+# capture pass `image=` (fp16_linear.ffn_image keeps one per module at a stable address).
+_FFN_IMAGES: dict = {}
+_FFN_IMAGES_MAX = 64
+
+
+def ffn_pack(w0, b0, w2, b2):
+    """Weight image of the packed fused FFN for bare tensors; cached while the four tensors are unchanged."""
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape), t.dtype) for t in (w0, b0, w2, b2))
+    img = _FFN_IMAGES.get(key)
+    if img is not None:
+        return img
+    img = ffn_pack_into(None, w0, b0, w2, b2)
+    while len(_FFN_IMAGES) >= _FFN_IMAGES_MAX:
+        _FFN_IMAGES.pop(next(iter(_FFN_IMAGES)))          # oldest entry first
     # the key's data pointers stay valid only while the tensors live: hold them with the image
     _FFN_IMAGES[key] = img
     img._bsrl_sources = (w0, b0, w2, b2)
     return img
 
 
-def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5, packed="auto", want_hidden=False):
+def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5, packed="auto", want_hidden=False,
+              image=None):
     """xo = x + act(h2 w0^T + b0) w2^T + b2; ho = LN(xo) when ln_w is given.
     Returns (xo, ho) (ho None without LN), or None when unsupported.
     want_hidden (packed route only; None is returned where that route has no kernel): (xo, ho, hid) with hid (.., F) the
     activated hidden as the down-projection consumed it, for a backward (the reference's save mode).
     packed: "auto" takes the packed-image kernel (bsrl_ffn_packed: d in {128, 192, 256, 384}, weights streamed straight
-    into LDS, 32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter."""
+    into LDS, 32 rows per wave) where the shape has one, else the kernel on the plain weights; False forces the latter.
+    image: the caller's own weight image of (w0, b0, w2, b2) (ffn_pack_into) for the packed kernel - the form for
+    callers whose launches a graph replays; without it the image comes from the identity-keyed cache of ffn_pack."""
     _need_cuda(x, h2, w0, w2)
     d = x.shape[-1]
     Fh = w0.shape[0]
@@ -452,7 +466,9 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5,
     xo = torch.empty_like(x)
     ho = torch.empty_like(x) if ln_w is not None else None
     if packed and ffn_pack_supported(d, Fh, x.dtype):
-        img = ffn_pack(w0, _f32c(b0, "b0"), w2, _f32c(b2, "b2"))
+        img = image if image is not None else ffn_pack(w0, _f32c(b0, "b0"), w2, _f32c(b2, "b2"))
+        if img.numel() != _lib.load().bsrl_ffn_pack_size(d, Fh, dt_code(x.dtype)) or img.device != x.device:
+            raise RuntimeError("ffn_fused: image does not belong to this shape / dtype / device")
         hid = torch.empty(*x.shape[:-1], Fh, device=x.device, dtype=x.dtype) if want_hidden else None
         with torch.cuda.device(x.device):
             rc = _lib.load().bsrl_ffn_packed(img.data_ptr(), x.data_ptr(), h2.data_ptr(), _ptr(_f32c(ln_w, "ln_w")),

@@ -471,7 +471,7 @@ class NotePolicy(nn.Module):
         """Force every weight copy the kernels read up to date for the current weights version
         (python/policy.py:1448-1461): call after optimizer steps under a captured graph.  On the
         16-bit stream these are the replicas (the encoders' column-padded first-layer copies among
-        them) and the fused block image; on the fp32 stream only
+        them), the fused block image and, with `fused_ffn` on, each block FFN's packed image; on the fp32 stream only
         the concatenated q|k|v / k|v / head matrices (single Linears read the masters)."""
         dt = self.stream_dtype if self.fp16 else torch.float32
         if self.fused_blocks_ok(dt):
@@ -482,6 +482,9 @@ class NotePolicy(nn.Module):
                     _fl._replica(m.weight, dt)
             for enc in (self.saber_mlp, self.torso_mlp, self.leg_mlp, self.note_mlp):   # padded first-layer copies
                 _fl._replica_padded(enc[0].weight, dt, ops.FRONT_PITCH)
+            if self.fused_ffn != "off":                     # the per-op route's fused block FFNs read packed images
+                for blk in self.blocks:
+                    _fl.ffn_image(blk.ffn, dt)
         for blk in self.blocks:
             _fl.packed_halves([blk.q_proj, blk.k_proj, blk.v_proj], dt)
             _fl.packed_halves([blk.k_proj, blk.v_proj], dt)

@@ -264,6 +264,19 @@ def forward(p, spec: ConfigSpec, obs, n_valid=None, emulate=None,
     return out[:, :n_log].reshape(B, N_HEADS_OUT, spec.n_gears).contiguous(), out[:, n_log].contiguous()
 
 
+def round_operands(p, obs, dtype: str):
+    """The config's own 16-bit storage, with the arithmetic left in fp32: every weight MATRIX and the observations
+    rounded once to fp16 / bf16 and widened again (biases and LayerNorm affine stay fp32, as in every 16-bit stream
+    here and in the reference, python/fp16_linear.py:1-18).  `forward(*round_operands(...))` is then the reference's
+    own kernel-test idiom - a closed form "on the same fp16-rounded inputs" (python/tests/test_attn29.py:49-54,
+    python/tests/test_fp16_accum.py:84-89) - applied to the whole forward: what is left between it and a 16-bit
+    forward is the forward's own activation rounding, not the rounding of weights the config declares to BE 16-bit.
+    No arithmetic of the oracle changes: the same `forward` runs on other inputs."""
+    dt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    pr = {k: (v.to(dt).float() if v.dim() == 2 else v) for k, v in p.items()}
+    return pr, obs.to(dt).float()
+
+
 def top2_margin(logits: torch.Tensor) -> torch.Tensor:
     """(B, 29) gap between the best and second-best logit of every head."""
     t = logits.topk(2, dim=-1).values

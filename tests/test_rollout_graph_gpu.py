@@ -48,11 +48,14 @@ def _eager_work():
     (x @ x.t()).sum().item()            # unrelated kernels + a device sync between replays
 
 
-@pytest.mark.parametrize("fp16,blocks", [(True, "auto"), (True, "off"), (False, "off")])
-def test_replays_match_eager_steps_and_follow_weight_refreshes(fp16, blocks):
+@pytest.mark.parametrize("fp16,blocks,ffn", [(True, "auto", "off"), (True, "off", "off"), (False, "off", "off"),
+                                             (True, "off", "on")])
+def test_replays_match_eager_steps_and_follow_weight_refreshes(fp16, blocks, ffn):
+    """ffn = "on" with the block stack per op: the block FFNs run as the packed-image fused kernel, whose images the
+    captured graph holds by address - they must be rebuilt in place by refresh(), like the replicas."""
     torch.manual_seed(11)
     m = NotePolicy(embed=128, trunk_dim=256, n_blocks=3, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True,
-                   head_gears=tuple(7 if j == 4 else 5 for j in range(29))).to(DEV)
+                   head_gears=tuple(7 if j == 4 else 5 for j in range(29)), fused_ffn=ffn).to(DEV)
     m.fp16, m.fused_blocks = fp16, blocks
     env = _Env(_obs(37, 2))
     gr = GraphedRollout(m, env)
