@@ -29,6 +29,15 @@
 #include <mutex>
 #include <type_traits>
 
+#ifdef BSRL_TIMING
+// probe build only (never part of the library): time stamps of one wave of a few workgroups
+__device__ unsigned long long g_stamp[8 * 128];
+extern "C" int bsrl_dbg_stamps(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_stamp), sizeof(g_stamp)); }
+#define STAMP() do { if (st_on && st_i < 128) { g_stamp[st_base + st_i] = __builtin_amdgcn_s_memrealtime(); } ++st_i; } while (0)
+#else
+#define STAMP() do { } while (0)
+#endif
+
 namespace {
 
 constexpr int D = 128;            // model width
@@ -64,6 +73,7 @@ struct FwdArgs {
                                   // before it), written by cfg_pair_kernel
     const int32_t* n_packed;      // PACK: number of tiles in `pairs`
     int64_t B; int n_layers, F, s_begin, s_end, n_logits, final_ln, prop_dim, obj_dim;
+    int t_begin, t_end;           // MERGE: stage range of the token-0 tail (the last block's output projection, FFN and the readout)
     int cus;          // CUs of the device (PACK: the remainder split below)
     int ring_epw;     // RING: envs per workgroup (1..4): one per wave, the other waves only feed the weight ring
 };
@@ -160,6 +170,12 @@ enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
 // Envs per 16-row MFMA tile in the TAIL launch.  Measured: 8 (twice the waves in flight, twice the weight stream)
 // takes 30 us against 24 us with full tiles at B = 16384.
 constexpr int TAIL_ENVS = 16;
+// MERGE (the pruned form as ONE launch: every first launch on the direct-to-LDS pipeline): a workgroup runs the token-0
+// tail of the envs it parked ITSELF - no other workgroup is ever waited for.  Their ids queue up in an LDS ring of
+// TAIL_CAP entries; whenever a workgroup pass (4 waves x 16 envs) is full, and once more at the end for the rest,
+// the weight stream switches to the tail's stage range for one pass.  A head pass parks at most 32 envs per
+// workgroup (8 tiles x 4) onto fewer than 64 waiting ones, so 128 entries always suffice.
+constexpr int TAIL_WG_ENVS = 4 * TAIL_ENVS, TAIL_CAP = 128;
 constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 16 dwords of attention output
 
 // PACK (HEAD launch only): short envs share a 16-row tile under a block-diagonal key mask - two of at most 8 tokens
@@ -174,7 +190,10 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     static_assert(!RING || MODE == MODE_FULL, "the ring pipeline is the one-launch latency form");
     static_assert(!DMA || (!RING && MODE != MODE_TAIL), "the paired direct-to-LDS pipeline serves the throughput forms");
     static_assert(KRT == 1 || KRT == 2, "the softmax butterflies pair the row tiles");
+    constexpr bool MERGE = DMA && MODE == MODE_HEAD;
     __shared__ uint4 lds[(RING || DMA) ? 1 : 2][(RING || DMA) ? 64 : STAGE_U4];
+    __shared__ int tail_list[MERGE ? TAIL_CAP : 1];   // MERGE: envs whose token-0 row this workgroup has parked, oldest first
+    __shared__ int tail_wr;                           // MERGE: entries ever reserved in tail_list (monotonic)
     extern __shared__ float4 vlds4[];                 // every fp32 vector of the model, resident for the whole kernel
     const float* vlds = reinterpret_cast<const float*>(vlds4);
     // RING: the stage ring sits behind the vectors (1 KB aligned) in the dynamic region
@@ -186,9 +205,20 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     const float scale_l2e = 0.17677669529663688110f * 1.44269504088896340736f;      // log2(e) / sqrt(32)
     constexpr int ENVS_PER_TILE = MODE == MODE_TAIL ? TAIL_ENVS : 1;     // envs per 16-row MFMA tile
     constexpr int ENVS_PER_WG = 4 * KRT * ENVS_PER_TILE;
-    const int64_t n_units = PACK ? (int64_t)*a.n_packed : a.B;           // 16-row tiles (PACK) or envs to cover
-    const int64_t ntiles = RING ? (a.B + a.ring_epw - 1) / a.ring_epw : (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
+    // PACK: the tile count, written by the table kernel just before this launch (on whichever XCD ran it: a fabric round
+    // trip of ~2 us from here).  Requested first thing, consumed behind the prologue, which takes about as long.
+    int np_raw = 0;
+    if (PACK) asm volatile("global_load_dword %0, %1, off" : "=v"(np_raw) : "v"(a.n_packed));
 
+#ifdef BSRL_TIMING
+    const int st_wgs[8] = {0, 130, 255, 256, 258, 261, 262, 511};
+    int st_sel = -1;
+    for (int i = 0; i < 8; ++i) if ((int)blockIdx.x == st_wgs[i]) st_sel = i;
+    const bool st_on = tid == 0 && st_sel >= 0;
+    const int st_base = (st_sel < 0 ? 0 : st_sel) * 128;
+    int st_i = 0;
+    STAMP();
+#endif
     const uint4* img = a.frags;
     const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
     const int uwave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -204,10 +234,23 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     const uint32_t wdst = ring_base + uwave * 2048;
     uint32_t src_off = 0;                             // byte offset of stage pnext
     const uint32_t src_begin = (uint32_t)a.s_begin * STAGE_B, src_end = (uint32_t)a.s_end * STAGE_B;
+    // The stage sequence is a chain of segments (stage ranges).  seg_end closes the segment being fetched; the one
+    // after it is (nxt_begin, nxt_end).  Without MERGE there is one range, walked cyclically.  MERGE: the consumer
+    // names the successor at the start of every segment - the fetch runs at most DMA_SLOTS stages ahead of it and
+    // every segment is longer, so the successor is always known before the fetch reaches a segment's end.
+    const uint32_t tail_begin = (uint32_t)a.t_begin * STAGE_B, tail_end = (uint32_t)a.t_end * STAGE_B;
+    uint32_t seg_end = src_end, nxt_begin = src_begin, nxt_end = src_end;
     auto ring_issue_off = [&](uint32_t slot_off) __attribute__((always_inline)) {     // stage pnext -> the slot at slot_off
         ring_load2(lane * 16, wsrc + src_off, wdst + slot_off);
-        src_off = src_off + STAGE_B == src_end ? src_begin : src_off + STAGE_B;
+        src_off += STAGE_B;
+        if (MERGE) { if (src_off == seg_end) { src_off = nxt_begin; seg_end = nxt_end; } }
+        else src_off = src_off == src_end ? src_begin : src_off;
     };
+    // MERGE bookkeeping, all wave-uniform: t_rd = entries of tail_list consumed so far (monotonic), t_cnt = entries
+    // waiting as of the last decision, t_more_head = another head-type pass of this workgroup follows the current one
+    // (set by the pass loop), t_tail_next = the segment after the current one is a tail pass
+    int t_rd = 0, t_cnt = 0;
+    bool t_more_head = false, t_tail_next = false;
     // RING: called when the next stage is about to be consumed; on return it is readable in slot ring_cur
     uint32_t ring_off = (RING_SLOTS - 1) * STAGE_B;   // byte offset of slot ring_cur
     auto ring_advance = [&]() __attribute__((always_inline)) {
@@ -278,7 +321,9 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         for (int i = 0; i < DMA_SLOTS - 2; ++i) ring_issue_off(i * STAGE_B);
         const int nv4 = vec_floats(a.n_layers, a.F) / 4;
         for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
+        if (tid == 0) tail_wr = 0;
         lds_barrier();
+        STAMP();
     } else {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
         const int s0 = a.s_begin;
         const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
@@ -301,16 +346,38 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         lds_barrier();
     }
 
+    if (PACK) asm volatile("s_waitcnt vmcnt(0)" : "+v"(np_raw) :: "memory");
+    // 16-row tiles (PACK) or envs to cover; the loaded count is the same in every lane, and said to be so: the pass loop
+    // and (MERGE) the stage-fetch addresses derived from it must stay in scalar registers
+    const int64_t n_units = PACK ? (int64_t)__builtin_amdgcn_readfirstlane(np_raw) : a.B;
+    const int64_t ntiles = RING ? (a.B + a.ring_epw - 1) / a.ring_epw : (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
+
     // One pass of this wave over the weight stream with RT row tiles.  A generic lambda so that the packed first launch
     // can hold two bodies: two row tiles per wave for the bulk, ONE for the remainder tiles of the last round (below).
     // env0: the wave's first env (or first tile, PACK).
     // PACK: the table entries of the wave's NEXT pass ride along with this pass's own input loads (one wait for both) and
     // stay in scalar registers, so that a pass starts its key-count and observation loads without first waiting for
-    // its table entries (one L2 round trip per pass).  next0 < 0: no next pass of the bulk body.
+    // its table entries (one L2 round trip per pass).  next_wg0 = the first tile of the WORKGROUP's next bulk pass (the
+    // same in every wave, and visibly so to the compiler: what hangs on it must stay wave-uniform), < 0: none.
     int pre_pr[PACK ? KRT : 1][4];
     bool have_pre = false;
-    auto pass = [&](auto rt_tag, const int64_t env0, const int64_t next0) __attribute__((always_inline)) {
+    // tail_tag (MERGE): this pass is a token-0 tail pass of the workgroup's own parked envs, on the tail's stage range
+    auto pass = [&](auto rt_tag, auto tail_tag, const int64_t env0, const int64_t next_wg0) __attribute__((always_inline)) {
         constexpr int RT = decltype(rt_tag)::value;
+        constexpr bool TAILP = MODE == MODE_TAIL || decltype(tail_tag)::value;     // rows are envs (token 0 of each)
+        static_assert(!decltype(tail_tag)::value || (MERGE && RT == 1), "merged tail passes run one row tile per wave");
+        // MERGE: called right behind the first stage admission of a segment (its barrier has made every wave's
+        // reservations for this pass visible): what follows this segment?
+        auto merge_decide = [&]() __attribute__((always_inline)) {
+            if (!MERGE) return;
+            if (!decltype(tail_tag)::value) {
+                const int wr = __builtin_amdgcn_readfirstlane(__hip_atomic_load(&tail_wr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+                t_cnt = wr - t_rd;
+                t_tail_next = t_cnt >= TAIL_WG_ENVS || (!t_more_head && t_cnt > 0);
+            }
+            nxt_begin = t_tail_next ? tail_begin : src_begin;
+            nxt_end = t_tail_next ? tail_end : src_end;
+        };
         // every lambda below is force-inlined: one left out of line would take the residual registers by reference,
         // i.e. through scratch memory (seen with the bf16 instantiations, whose pack helper is larger)
         float kmask[RT][4];     // additive key mask for keys 4g..4g+3 of each env: 0 (attendable) or -inf
@@ -451,6 +518,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
             for (int st = 0; st < NT / 2; ++st) {
                 ADV(st);                    // 12 stages precede in the block (parity restarts even); TAIL starts here
+                if (decltype(tail_tag)::value && st == 0) merge_decide();
                 LOAD_STAGE(st & 1, wf);
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
@@ -459,6 +527,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
                         for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], of[rt][c].v, x[rt][2 * st + ntl]);
             }
+            if (decltype(tail_tag)::value) STAMP();
             norm_to_frags(lv + LV_LN2G, lv + LV_LN2B, true, hf);
             add_bias(lv + lv_b2(a.F));
             // Software-pipelined over 32-wide hidden chunks.  MFMA and VALU work only overlap when they
@@ -619,9 +688,10 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         };
 
         // ---- 29*K + 1 output projection (8 stages); rf[i] = operand fragments whose rows are envs,
-        //      row r16 of tile i being env env_base + i * 16 + r16 (stored when r16 < rows_valid) ----
-        auto heads = [&](auto& rf, int64_t env_base, int rows_valid, const float* fvp) __attribute__((always_inline)) {
+        //      row r16 being env lane_env (stored when lane_ok) ----
+        auto heads = [&](auto& rf, const int64_t lane_env, const bool lane_ok, const float* fvp) __attribute__((always_inline)) {
             constexpr int NR = sizeof(rf) / sizeof(rf[0]);
+            static_assert(NR == 1, "one operand tile per wave: row r16 is the env lane_env");
             // The outputs stay in registers until the last stage has been consumed: stores count in the same
             // in-order vmcnt queue as the weight prefetches, so a store issued inside the stage loop would make
             // the next stage's wait sit out an HBM write.
@@ -643,10 +713,11 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                     }
                 }
             }
+            if (decltype(tail_tag)::value) STAMP();
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
-                const int64_t env = env_base + i * 16 + r16;
-                if (r16 < rows_valid && env < a.B) {
+                const int64_t env = lane_env;
+                if (lane_ok) {
                     // a lane holds 4 consecutive outputs of its row: one 4-dword store (rows are only dword-aligned:
                     // the type says so and the compiler picks the widest store the target allows at that alignment)
                     typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -669,8 +740,9 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             }
         };
         const float* fv = vlds + V_LAYER0 + a.n_layers * lv_size(a.F);
+        STAMP();
 
-        if (MODE != MODE_TAIL) {
+        if constexpr (!TAILP) {
             // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
             Frag8 e[RT][KC];
             // PACK: the env of this lane's row r16 and the row's token index inside it (otherwise a tile is one env and
@@ -683,6 +755,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                 return env < a.B ? env : a.B - 1;
             };
             auto tok_at = [&](int rt) __attribute__((always_inline)) { return PACK ? ltok[PACK ? rt : 0] : r16; };
+            int n_park = 0;             // MERGE: token-0 rows this wave parks in this pass (wave-uniform)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 if (PACK) {
@@ -703,6 +776,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                         o = (sl >= 3 && e3 >= 0) ? 3 : o;
                         return o;
                     };
+                    if (env0 + rt < n_units) n_park += 1 + (e1 >= 0 ? 1 : 0) + (e2 >= 0 ? 1 : 0) + (e3 >= 0 ? 1 : 0);
                     const int orow = owner(r16 >> 2), okey = owner(g);
                     const int64_t le = orow == 0 ? e0 : orow == 1 ? e1 : orow == 2 ? e2 : e3;
                     lenv[PACK ? rt : 0] = le;
@@ -716,13 +790,22 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                     const int nvalid = a.n_valid ? a.n_valid[env] : T - 1;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) kmask[rt][i] = (4 * g + i) <= nvalid ? 0.f : -INFINITY;
+                    if (env0 + rt < a.B) n_park += 1;
                 }
             }
+            // MERGE: reserve this wave's entries of the workgroup's tail list now, so that the count of waiting envs is
+            // known to every wave behind the pass's first barrier (merge_decide), long before the stage fetch reaches
+            // the end of this segment
+            int t_pos = 0;
+            if (MERGE) {
+                if (lane == 0) t_pos = __hip_atomic_fetch_add(&tail_wr, n_park, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                t_pos = __builtin_amdgcn_readfirstlane(t_pos);
+            }
             int4 nxt[PACK ? RT : 1];
-            if (PACK && RT == KRT && next0 >= 0) {
+            if (PACK && RT == KRT && next_wg0 >= 0) {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    int64_t tix = next0 + rt; tix = tix < n_units ? tix : n_units - 1;
+                    int64_t tix = next_wg0 + (int64_t)wave * KRT + rt; tix = tix < n_units ? tix : n_units - 1;
                     nxt[PACK ? rt : 0] = a.pairs[tix];
                 }
             }
@@ -784,7 +867,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             // outstanding loads", i.e. drain the ring in mid-tile; after this it has nothing pending.
             if (RING || DMA) __builtin_amdgcn_s_waitcnt(0x0F70);
             if (PACK && RT == KRT) {
-                have_pre = next0 >= 0;
+                have_pre = next_wg0 >= 0;
                 if (have_pre) {
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
@@ -808,6 +891,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
             for (int st = 0; st < EMB_STAGES; ++st) {
                 ADVANCE(st & 1);
+                if (st == 0) merge_decide();
                 LOAD_STAGE(st & 1, wf);
 #pragma unroll
                 for (int c = 0; c < KC; ++c)
@@ -818,14 +902,30 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             }
             // ================= transformer blocks =================
             const int dense_layers = MODE == MODE_FULL ? a.n_layers : a.n_layers - 1;
+            STAMP();
             for (int l = 0; l < dense_layers; ++l) {
                 const float* lv = vlds + V_LAYER0 + l * lv_size(a.F);
                 attention(lv);
+                STAMP();
                 proj_and_ffn(lv);
+                STAMP();
             }
             if (MODE == MODE_HEAD) {
                 // last block: attention only, then park token 0 (lanes r16 == 0) for the TAIL launch
                 attention(vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F));
+                if (MERGE) {
+                    // the parked envs' ids -> the entries reserved at the start of the pass (lanes 0..15 speak for their
+                    // row; an env's place among the wave's entries is its rank among the parking lanes)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        const int64_t env = PACK ? lenv[PACK ? rt : 0] : env0 + rt;
+                        const bool parks = (PACK ? ((r16 & 3) == 0 && ltok[PACK ? rt : 0] == 0 && env0 + rt < n_units)
+                                                 : (r16 == 0 && env < a.B)) && g == 0;
+                        const uint64_t who = __ballot(parks);
+                        if (parks) tail_list[(t_pos + __popcll(who & ((1ull << lane) - 1))) & (TAIL_CAP - 1)] = (int)env;
+                        t_pos += __popcll(who);
+                    }
+                }
                 if (PACK ? (r16 & 3) == 0 : r16 == 0) {
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
@@ -841,6 +941,12 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                         }
                     }
                 }
+                // MERGE: the lanes rejoin HERE, in a block of their own.  Without it the join of the lane-dependent
+                // branches above is the head of the tail-pass loop that follows the pass, and the compiler's uniformity
+                // analysis then takes every value that loop carries - the stage-fetch offsets among them, which must
+                // be scalar operands of the transfer instructions - for lane-dependent.
+                if (MERGE) asm volatile("" ::: "memory");
+                STAMP();
             } else {
                 // ================= readout: token 0 of every env -> 29*K logits + value =================
                 Frag8 yf[RT][KC];
@@ -858,14 +964,31 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                             const uint32_t v = __shfl(yf[rt][c].w[w], 16 * g, WAVE);
                             if (r16 == rt) rf[0][c].w[w] = v;
                         }
-                heads(rf, env0, RT, fv);
+                heads(rf, env0 + r16, r16 < RT && env0 + r16 < a.B, fv);
             }
         } else {
             // ================= TAIL: rows are envs (token 0 of each) =================
             const float* lv = vlds + V_LAYER0 + (a.n_layers - 1) * lv_size(a.F);
+            int64_t tenv = env0 + r16;                     // this lane's row
+            bool tok = tenv < a.B;
+            if (decltype(tail_tag)::value) {
+                // MERGE: the next (at most) 64 envs of the workgroup's list, 16 to a wave.  Their rows were parked by
+                // this workgroup's own waves: once every wave's stores have completed (vmcnt) and every wave has said
+                // so (barrier), the rows and the list entries are readable - the waves of a workgroup share the CU's
+                // vector cache, and nothing else ever read these lines in this launch.
+                const int n = t_cnt < TAIL_WG_ENVS ? t_cnt : TAIL_WG_ENVS, base = t_rd;
+                t_rd += n; t_cnt -= n;
+                t_tail_next = !t_more_head && t_cnt > 0;
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                lds_barrier();
+                const int idx = wave * TAIL_ENVS + r16;
+                tok = idx < n;                             // rows past the list's end compute on the first env's row and store nothing
+                tenv = tail_list[(base + (tok ? idx : 0)) & (TAIL_CAP - 1)];
+            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                int64_t env = env0 + rt * TAIL_ENVS + r16; env = env < a.B ? env : a.B - 1;     // rows >= TAIL_ENVS: never stored
+                int64_t env = decltype(tail_tag)::value ? tenv : env0 + rt * TAIL_ENVS + r16;
+                env = env < a.B ? env : a.B - 1;           // rows >= TAIL_ENVS: never stored
 #pragma unroll
                 for (int i = 0; i < 4; ++i) kmask[rt][i] = 0.f;
                 const uint4* src = reinterpret_cast<const uint4*>(a.ws + (env * 4 + g) * WS_DWORDS);
@@ -874,10 +997,15 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
                 for (int c = 0; c < KC; ++c) of[rt][c].u = src[NT + c];
             }
+            // MERGE: the rows are waited for here, with the wait the compiler can see (as the tokenizer's loads are)
+            if (decltype(tail_tag)::value) __builtin_amdgcn_s_waitcnt(0x0F70);
+            STAMP();
             proj_and_ffn(lv);
+            STAMP();
             Frag8 yf[RT][KC];
             norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
-            heads(yf, env0, TAIL_ENVS, fv);
+            heads(yf, tenv, tok, fv);
+            STAMP();
         }
     };
     typedef std::integral_constant<int, KRT> rt_bulk;
@@ -891,28 +1019,64 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     int64_t n_bulk = ntiles;                 // workgroup passes of the bulk body
     int64_t rem_tile0 = 0; int rem_first_wg = 0, rem_passes = 0;
     if (PACK && KRT == 2 && a.cus > 0) {
-        const int64_t r = ntiles % a.cus;
-        const int64_t p2 = ntiles - r;
+        // (32-bit arithmetic: the packed tile count is an int32, and a 64-bit division is a ~200-instruction routine
+        // of which three sat between the prologue and the first pass)
+        const uint32_t nt32 = (uint32_t)ntiles;
+        const int64_t r = nt32 % (uint32_t)a.cus;
+        const int64_t p2 = nt32 - (uint32_t)r;
         const int64_t nrem = n_units - p2 * ENVS_PER_WG;                 // tiles left for one-tile passes
-        const int q = (int)((nrem + 3) / 4), fb = (int)(p2 % gridDim.x);
+        const int q = (int)(((uint32_t)nrem + 3u) / 4u), fb = (int)((uint32_t)p2 % gridDim.x);
         if (r > 0 && r <= 32 && p2 > 0 && fb + q <= (int)gridDim.x) { n_bulk = p2; rem_tile0 = p2 * ENVS_PER_WG; rem_first_wg = fb; rem_passes = q; }
     }
-    for (int64_t tile = blockIdx.x; tile < n_bulk; tile += gridDim.x) {
-        const int64_t env0 = RING ? tile * a.ring_epw + uwave : tile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE;
-        if (RING && (uwave >= a.ring_epw || env0 >= a.B)) {
-            // a wave without an env: it keeps its share of the weight ring moving (loads, waits, barriers - exactly one
-            // advance per stage, like the working waves) and reads no fragment, so the workgroup's LDS reads are those
-            // of its working waves only
-            for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
-            continue;
-        }
-        const int64_t ntile = tile + gridDim.x;
-        pass(rt_bulk(), env0, (PACK && ntile < n_bulk) ? ntile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE : -1);
-    }
-    if (PACK && KRT == 2) {
+    typedef std::integral_constant<int, 1> rt_one;
+    typedef std::false_type head_pass;
+    if constexpr (MERGE) {
+        // head-type passes (this workgroup's one-tile remainder pass first, if it has one, then its bulk passes), each
+        // followed by the tail passes it has made due: one whenever 64 envs wait, and the rest after the last head-type
+        // pass.  The remainder pass goes FIRST: the workgroups that get one are the younger of their CU's two, and a
+        // pass is a latency chain of 64 stages - run while the CU's other workgroup computes it costs the CU its
+        // arithmetic (half a bulk pass); run at the end, after that workgroup has left, it cost the whole chain
+        // (~18 us at the end of the launch, on 6 CUs of 256, at the headline batch).
         const int qi = (int)blockIdx.x - rem_first_wg;
-        if (qi >= 0 && qi < rem_passes) pass(std::integral_constant<int, 1>(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
+        bool rem_due = PACK && KRT == 2 && qi >= 0 && qi < rem_passes;
+        int64_t tile = blockIdx.x;
+        while (true) {
+            if (rem_due) {
+                rem_due = false;
+                t_more_head = tile < n_bulk;
+                // ... and at raised priority: this workgroup's chain of passes is one longer than every other's, so
+                // while it runs the extra one it goes first at the SIMDs' issue ports
+                __builtin_amdgcn_s_setprio(3);
+                pass(rt_one(), head_pass(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
+                __builtin_amdgcn_s_setprio(0);
+            } else if (tile < n_bulk) {
+                const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE;
+                const int64_t ntile = tile + gridDim.x;
+                t_more_head = ntile < n_bulk;
+                pass(rt_bulk(), head_pass(), env0, (PACK && ntile < n_bulk) ? ntile * ENVS_PER_WG : -1);
+                tile = ntile;
+            } else break;
+            while (t_tail_next) pass(rt_one(), std::integral_constant<bool, MERGE>(), 0, -1);
+        }
+    } else {
+        for (int64_t tile = blockIdx.x; tile < n_bulk; tile += gridDim.x) {
+            const int64_t env0 = RING ? tile * a.ring_epw + uwave : tile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE;
+            if (RING && (uwave >= a.ring_epw || env0 >= a.B)) {
+                // a wave without an env: it keeps its share of the weight ring moving (loads, waits, barriers - exactly one
+                // advance per stage, like the working waves) and reads no fragment, so the workgroup's LDS reads are those
+                // of its working waves only
+                for (int s_ = a.s_begin; s_ < a.s_end; ++s_) ring_advance();
+                continue;
+            }
+            const int64_t ntile = tile + gridDim.x;
+            pass(rt_bulk(), head_pass(), env0, (PACK && ntile < n_bulk) ? ntile * ENVS_PER_WG : -1);
+        }
+        if (PACK && KRT == 2) {
+            const int qi = (int)blockIdx.x - rem_first_wg;
+            if (qi >= 0 && qi < rem_passes) pass(rt_one(), head_pass(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
+        }
     }
+    STAMP();
     if (RING || DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
 }
@@ -1196,6 +1360,7 @@ int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStre
     }
     const int split = EMB_STAGES + (a.n_layers - 1) * ls + 3 * H;
     a.s_begin = 0; a.s_end = split;
+    a.t_begin = split; a.t_end = total;
     int rc;
     if (pack) {
         // the grid is sized for the unpacked tile count (the packed one is known on the device only); workgroups past
@@ -1211,7 +1376,7 @@ int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStre
     } else {
         rc = dma ? launch_one<DT, 2, ACT, MODE_HEAD, false, false, true>(a, cus, st) : launch_one<DT, 2, ACT, MODE_HEAD>(a, cus, st);
     }
-    if (rc != BSRL_OK) return rc;
+    if (rc != BSRL_OK || dma) return rc;           // on the direct-to-LDS pipeline the first launch runs the tail itself
     a.s_begin = split; a.s_end = total;
     return launch_one<DT, 1, ACT, MODE_TAIL>(a, cus, st);
 }
@@ -1280,7 +1445,7 @@ int cfg_forward_impl(const char* who, const bsrl_cfg_desc* d, const void* packed
     a.obs = obs; a.obs_ld = obs_ld; a.obs_f32 = obs_dtype == BSRL_F32;
     a.tok_vec = a.obs_f32 && d->obj_dim == 16 && d->prop_dim % 4 == 0 && obs_ld % 4 == 0 && bsrl_aligned(obs, 16);
     a.n_valid = n_valid; a.logits = logits; a.value = value; a.B = B;
-    a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0;
+    a.n_layers = d->n_layers; a.F = d->ffn; a.s_begin = 0; a.s_end = 0; a.t_begin = 0; a.t_end = 0;
     a.n_logits = 29 * d->n_gears; a.final_ln = d->final_ln; a.prop_dim = d->prop_dim; a.obj_dim = d->obj_dim;
     a.ws = static_cast<uint32_t*>(rows);
     a.ring_epw = 4; a.cus = 0;
