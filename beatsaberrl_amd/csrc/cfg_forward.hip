@@ -17,10 +17,19 @@
 // image by bsrl_cfg_pack, so a weight fragment is one 16-byte LDS read per lane.
 // The V projection swaps operand roles and so lands already transposed for P.V.
 //
-// Weights (~0.85 MB at 2 layers) stream from L2 through a 2-slot LDS ring in
-// 8 KB stages (8 fragments) shared by the workgroup's 4 waves: global loads are
-// issued three stages ahead into registers, written to LDS one stage ahead,
-// one barrier per stage.  HBM traffic is the obs in and the logits out.
+// Weights (~0.85 MB at 2 layers) stream from L2 in 8 KB stages (8 fragments) shared by the workgroup's 4 waves.
+// Three pipelines, chosen on the host by shape and batch (same output bits):
+//   * DMA  - the throughput forms' default: stages go straight from L2 into a 6-slot LDS ring
+//            (global_load_lds_dwordx4), admitted in pairs: one vmcnt wait + barrier per two stages;
+//   * RING - the latency form (B <= 4 per CU): the same transfers 13 stages ahead into a 14-slot ring, one env per wave;
+//   * register-staged (models whose vectors + two rings overflow a CU's LDS): global loads three stages ahead into
+//     registers, written to a 2-slot LDS ring one stage ahead, one barrier per stage.
+// HBM traffic is the obs in, the logits out and, in the pruned form, each env's parked token-0 row (768 B).
+//
+// Final-block query pruning runs as ONE launch on the DMA pipeline (MERGE): every workgroup parks the token-0 rows of
+// its own envs and, whenever 64 of them wait and once more at the end, switches its weight stream to the tail's stage
+// range and runs the last block's output projection, FFN and the readout on them itself - no workgroup ever waits
+// for another.  On the register-staged pipeline the tail is a second launch (MODE_TAIL).
 //
 // Replaces NotePolicy.forward_stacked (python/policy.py:1179-1344) for the
 // benchmark-config model; the weight image is the analogue of the reference's
@@ -28,15 +37,6 @@
 #include "bsrl_common.h"
 #include <mutex>
 #include <type_traits>
-
-#ifdef BSRL_TIMING
-// probe build only (never part of the library): time stamps of one wave of a few workgroups
-__device__ unsigned long long g_stamp[8 * 128];
-extern "C" int bsrl_dbg_stamps(unsigned long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_stamp), sizeof(g_stamp)); }
-#define STAMP() do { if (st_on && st_i < 128) { g_stamp[st_base + st_i] = __builtin_amdgcn_s_memrealtime(); } ++st_i; } while (0)
-#else
-#define STAMP() do { } while (0)
-#endif
 
 namespace {
 
@@ -164,8 +164,9 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 //   python/policy.py:533-539: exact, because masking is key-side only).  HEAD runs the
 //   tokenizer, blocks 0..L-2 and the last block's LN + QKV + attention, and parks the
 //   token-0 row of every env (fp32 residual + attention-output fragments) in the
-//   workspace; TAIL re-tiles those rows 16 envs per MFMA tile and runs the last block's
-//   output projection + FFN and the 29*K + 1 output projection on them.
+//   workspace; the tail re-tiles those rows 16 envs per MFMA tile and runs the last block's
+//   output projection + FFN and the 29*K + 1 output projection on them - inside the HEAD
+//   launch on the DMA pipeline (MERGE, below), as a launch of its own (MODE_TAIL) otherwise.
 enum { MODE_FULL = 0, MODE_HEAD = 1, MODE_TAIL = 2 };
 // Envs per 16-row MFMA tile in the TAIL launch.  Measured: 8 (twice the waves in flight, twice the weight stream)
 // takes 30 us against 24 us with full tiles at B = 16384.
@@ -184,9 +185,20 @@ constexpr int WS_DWORDS = 48;      // per (env, lane group): 32 fp32 residual + 
 // LayerNorm) is untouched by the row's position; the softmax sums and the P.V contraction see an env's keys a
 // multiple of 4 lanes / k slots further on: a key's place inside its lane group of 4 is unchanged, whole groups move,
 // and everything else a sum meets is an exact zero - an env's bits stay what they are alone in a tile.
-template <typename DT, int KRT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false>
+// INK (a PACK + MERGE variant, batches of at most INK_MAX_ENVS): no tile table in memory and no table kernel before the
+// launch.  Every workgroup classes the whole batch itself in its prologue (64 KB of key counts out of L2, beside the
+// weight ring's first stages) and keeps, in LDS, a 2-bit class code per env and the four classes' exclusive prefixes
+// over blocks of 64 envs; a tile's four slot entries are then SELECTED from those on the fly - lane i of the wave
+// answers "which env is the r-th of class c" for slot i by a binary search over the prefixes and a rank select in the
+// block's class mask - one pass ahead, while the pass's own observation loads are in flight.  The entries are
+// those cfg_pair_kernel writes (same classes, same stable order, same tile order).
+constexpr int INK_BLOCKS = 256, INK_MAX_ENVS = INK_BLOCKS * 64;
+constexpr int INK_WORDS = INK_BLOCKS * 4 + 4 * INK_BLOCKS + 4;           // class bit planes, prefixes, totals (dwords)
+constexpr size_t INK_BYTES = ((size_t)INK_WORDS * 4 + 255) & ~(size_t)255;
+template <typename DT, int KRT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false, bool INK = false>
 __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_kernel(FwdArgs a) {
     static_assert(!PACK || MODE == MODE_HEAD, "packing is a HEAD-launch variant");
+    static_assert(!INK || (PACK && DMA && MODE == MODE_HEAD && KRT == 2), "the in-kernel tile table is a variant of the packed one-launch form");
     static_assert(!RING || MODE == MODE_FULL, "the ring pipeline is the one-launch latency form");
     static_assert(!DMA || (!RING && MODE != MODE_TAIL), "the paired direct-to-LDS pipeline serves the throughput forms");
     static_assert(KRT == 1 || KRT == 2, "the softmax butterflies pair the row tiles");
@@ -208,17 +220,8 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
     // PACK: the tile count, written by the table kernel just before this launch (on whichever XCD ran it: a fabric round
     // trip of ~2 us from here).  Requested first thing, consumed behind the prologue, which takes about as long.
     int np_raw = 0;
-    if (PACK) asm volatile("global_load_dword %0, %1, off" : "=v"(np_raw) : "v"(a.n_packed));
+    if (PACK && !INK) asm volatile("global_load_dword %0, %1, off" : "=v"(np_raw) : "v"(a.n_packed));
 
-#ifdef BSRL_TIMING
-    const int st_wgs[8] = {0, 130, 255, 256, 258, 261, 262, 511};
-    int st_sel = -1;
-    for (int i = 0; i < 8; ++i) if ((int)blockIdx.x == st_wgs[i]) st_sel = i;
-    const bool st_on = tid == 0 && st_sel >= 0;
-    const int st_base = (st_sel < 0 ? 0 : st_sel) * 128;
-    int st_i = 0;
-    STAMP();
-#endif
     const uint4* img = a.frags;
     const uint32_t ring_base = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)const_cast<uint4*>(ring);
     const int uwave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -323,7 +326,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         for (int i = tid; i < nv4; i += 256) vlds4[i] = reinterpret_cast<const float4*>(a.vec)[i];
         if (tid == 0) tail_wr = 0;
         lds_barrier();
-        STAMP();
     } else {   // prologue: first stage -> LDS slot 0; the next two (TAIL: four) in flight (stage counts per mode are even)
         const int s0 = a.s_begin;
         const uint4 s0a = img[(int64_t)s0 * STAGE_U4 + tid], s0b = img[(int64_t)s0 * STAGE_U4 + tid + 256];
@@ -346,10 +348,119 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
         lds_barrier();
     }
 
-    if (PACK) asm volatile("s_waitcnt vmcnt(0)" : "+v"(np_raw) :: "memory");
+    if (PACK && !INK) asm volatile("s_waitcnt vmcnt(0)" : "+v"(np_raw) :: "memory");
+    // INK: class codes and prefixes of the whole batch -> LDS (behind the ring).  Classes as cfg_pair_kernel's: by key
+    // count n_valid >> 2 = 0 tiny, 1 mid, 2 host, 3 (or more, or negative) long; envs past the batch's end count as long
+    // ones behind every real env, which no select ever reaches.
+    uint32_t* const ink_code = reinterpret_cast<uint32_t*>(const_cast<uint4*>(ring) + DMA_SLOTS * STAGE_U4);   // [block][4]: 2 bits per env
+    uint32_t* const ink_pf = ink_code + INK_BLOCKS * 4;                                                       // [class][block]
+    uint32_t* const ink_tot = ink_pf + 4 * INK_BLOCKS;                                                        // [class]
+    int ink_tt = 0, ink_tm = 0, ink_th = 0, ink_first_quad = 0, ink_first_host = 0, ink_first_long = 0;
+    if constexpr (INK) {
+        // wave w classes envs [4096 w, 4096 w + 4096): sixteen coalesced 16-byte loads per lane, all in flight at once
+        // (one memory round trip), the four 2-bit codes of a load written as ONE byte into the code array - which is
+        // thereby in env order, 16 envs to a dword -, then lane l reads back block 64 w + l whole and counts its classes
+        const int nB = (int)a.B, nq_full = nB >> 2;                        // whole groups of four envs
+        const int4* nvq = reinterpret_cast<const int4*>(a.n_valid);        // 16-byte aligned (a condition of packing)
+        uint32_t tail_byte = 0xFFu;                                        // the codes of the last B % 4 envs (then ghosts)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int e = nq_full * 4 + k;
+            const uint32_t c = (uint32_t)a.n_valid[e < nB ? e : nB - 1] >> 2;
+            const uint32_t code = (e < nB && c < 3u) ? c : 3u;
+            tail_byte = (tail_byte & ~(3u << (2 * k))) | (code << (2 * k));
+        }
+        int4 v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = make_int4(0, 0, 0, 0);
+        if (nq_full > 0) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { const int q = (uwave * 16 + i) * 64 + lane; v[i] = nvq[q < nq_full ? q : nq_full - 1]; }
+        }
+        unsigned char* const cbytes = reinterpret_cast<unsigned char*>(ink_code);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int q = (uwave * 16 + i) * 64 + lane;
+            auto c2 = [](int nv) __attribute__((always_inline)) { const uint32_t c = (uint32_t)nv >> 2; return c < 3u ? c : 3u; };
+            uint32_t byte = c2(v[i].x) | (c2(v[i].y) << 2) | (c2(v[i].z) << 4) | (c2(v[i].w) << 6);
+            byte = q < nq_full ? byte : q == nq_full ? tail_byte : 0xFFu;
+            cbytes[q] = (unsigned char)byte;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                 // the wave's own bytes (the LDS serves a wave in order)
+        const int blk = uwave * 64 + lane;
+        const uint4 cw = reinterpret_cast<const uint4*>(ink_code)[blk];
+        const uint32_t cwd[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t n = 0;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) { const uint32_t x = cwd[d] ^ (0x55555555u * c); n += __popc(~(x | (x >> 1)) & 0x55555555u); }
+            ink_pf[c * INK_BLOCKS + blk] = n;
+        }
+        lds_barrier();
+        if (uwave == 0) {                                                  // counts -> exclusive prefixes, 4 blocks to a lane
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                uint4* row = reinterpret_cast<uint4*>(ink_pf + c * INK_BLOCKS);
+                const uint4 v = row[lane];
+                const uint32_t sum = v.x + v.y + v.z + v.w;
+                uint32_t incl = sum;
+#pragma unroll
+                for (int d = 1; d < WAVE; d <<= 1) { const uint32_t up = __shfl_up(incl, d, WAVE); if (lane >= d) incl += up; }
+                const uint32_t ex = incl - sum;
+                row[lane] = make_uint4(ex, ex + v.x, ex + v.x + v.y, ex + v.x + v.y + v.z);
+                if (lane == WAVE - 1) ink_tot[c] = incl;
+            }
+        }
+        lds_barrier();
+        ink_tt = __builtin_amdgcn_readfirstlane((int)ink_tot[0]);
+        ink_tm = __builtin_amdgcn_readfirstlane((int)ink_tot[1]);
+        ink_th = __builtin_amdgcn_readfirstlane((int)ink_tot[2]);
+        const int loose = ink_tt > ink_th ? ink_tt - ink_th : 0;           // tiny envs without a host
+        ink_first_quad = (ink_tm + 1) / 2;
+        ink_first_host = ink_first_quad + (loose + 3) / 4;
+        ink_first_long = ink_first_host + ink_th;
+    }
+    // INK: the four slot entries of the KRT consecutive tiles from t0 on (t0 the same in every lane), as cfg_pair_kernel
+    // would have written them: lane 4 rt + s answers for slot s of tile t0 + rt, the answers go to out[rt][s]
+    auto ink_entries = [&](const int t0, int (&out)[PACK ? KRT : 1][4]) __attribute__((always_inline)) {
+        const int n_all = ink_first_long + ((int)a.B - ink_tt - ink_tm - ink_th);
+        int t = t0 + ((lane >> 2) & (KRT - 1));
+        t = t < n_all ? t : n_all - 1;
+        const int sl = lane & 3;
+        int cls, rank; bool on;
+        if (t < ink_first_quad) { cls = 1; rank = 2 * t + (sl >> 1); on = (sl & 1) == 0 && rank < ink_tm; }
+        else if (t < ink_first_host) { cls = 0; rank = ink_th + 4 * (t - ink_first_quad) + sl; on = rank < ink_tt; }
+        else if (t < ink_first_long) { cls = sl == 3 ? 0 : 2; rank = t - ink_first_host; on = sl == 0 || (sl == 3 && rank < ink_tt); }
+        else { cls = 3; rank = t - ink_first_long; on = sl == 0; }
+        rank = on ? rank : 0;
+        const uint32_t* pf = ink_pf + cls * INK_BLOCKS;
+        int j = 0;                                                         // the last block that starts at or before the rank
+#pragma unroll
+        for (int step = INK_BLOCKS / 2; step > 0; step >>= 1) j += pf[j + step] <= (uint32_t)rank ? step : 0;
+        const uint32_t rr = (uint32_t)rank - pf[j];
+        // the block's codes (16 envs to a dword, 2 bits each) -> one bit per env of the class, at the even positions
+        const uint4 cw = reinterpret_cast<const uint4*>(ink_code)[j];
+        const uint32_t pat = 0x55555555u * (uint32_t)cls;
+        auto mask_of = [&](uint32_t w) __attribute__((always_inline)) { const uint32_t x = w ^ pat; return ~(x | (x >> 1)) & 0x55555555u; };
+        const uint32_t m0 = mask_of(cw.x), m1 = mask_of(cw.y), m2 = mask_of(cw.z), m3 = mask_of(cw.w);
+        const uint32_t s1 = __popc(m0), s2 = s1 + __popc(m1), s3 = s2 + __popc(m2);
+        const int dw = (rr >= s1 ? 1 : 0) + (rr >= s2 ? 1 : 0) + (rr >= s3 ? 1 : 0);
+        const uint32_t w = dw == 0 ? m0 : dw == 1 ? m1 : dw == 2 ? m2 : m3;
+        const uint32_t r2 = rr - (dw == 0 ? 0u : dw == 1 ? s1 : dw == 2 ? s2 : s3);
+        int pos = 0;                                                       // the r2-th set bit of w: the most bits below it that hold at most r2 ones
+#pragma unroll
+        for (int step = 16; step > 0; step >>= 1) pos += (uint32_t)__popc(w & ((1u << (pos + step)) - 1u)) <= r2 ? step : 0;
+        const int env = on ? j * 64 + dw * 16 + (pos >> 1) : -1;
+#pragma unroll
+        for (int rt = 0; rt < (PACK ? KRT : 1); ++rt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[rt][i] = __builtin_amdgcn_readlane(env, rt * 4 + i);
+    };
     // 16-row tiles (PACK) or envs to cover; the loaded count is the same in every lane, and said to be so: the pass loop
     // and (MERGE) the stage-fetch addresses derived from it must stay in scalar registers
-    const int64_t n_units = PACK ? (int64_t)__builtin_amdgcn_readfirstlane(np_raw) : a.B;
+    const int64_t n_units = INK ? (int64_t)(ink_first_long + ((int)a.B - ink_tt - ink_tm - ink_th))
+                                : PACK ? (int64_t)__builtin_amdgcn_readfirstlane(np_raw) : a.B;
     const int64_t ntiles = RING ? (a.B + a.ring_epw - 1) / a.ring_epw : (n_units + ENVS_PER_WG - 1) / ENVS_PER_WG;
 
     // One pass of this wave over the weight stream with RT row tiles.  A generic lambda so that the packed first launch
@@ -527,7 +638,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
 #pragma unroll
                         for (int rt = 0; rt < RT; ++rt) x[rt][2 * st + ntl] = DT::mfma32(wf[ntl * KC + c], of[rt][c].v, x[rt][2 * st + ntl]);
             }
-            if (decltype(tail_tag)::value) STAMP();
             norm_to_frags(lv + LV_LN2G, lv + LV_LN2B, true, hf);
             add_bias(lv + lv_b2(a.F));
             // Software-pipelined over 32-wide hidden chunks.  MFMA and VALU work only overlap when they
@@ -713,7 +823,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                     }
                 }
             }
-            if (decltype(tail_tag)::value) STAMP();
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
                 const int64_t env = lane_env;
@@ -740,7 +849,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             }
         };
         const float* fv = vlds + V_LAYER0 + a.n_layers * lv_size(a.F);
-        STAMP();
 
         if constexpr (!TAILP) {
             // ================= tokenizer: K = [obj 16 | prop <= 112], N = d =================
@@ -756,12 +864,16 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             };
             auto tok_at = [&](int rt) __attribute__((always_inline)) { return PACK ? ltok[PACK ? rt : 0] : r16; };
             int n_park = 0;             // MERGE: token-0 rows this wave parks in this pass (wave-uniform)
+            int now_pr[PACK ? KRT : 1][4];
+            if (INK && !(RT == KRT && have_pre)) ink_entries(__builtin_amdgcn_readfirstlane((int)env0), now_pr);   // no entries from the pass before: select them now
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 if (PACK) {
                     int e0, e1, e2, e3;
                     if (RT == KRT && have_pre) {
                         e0 = pre_pr[PACK ? rt : 0][0]; e1 = pre_pr[PACK ? rt : 0][1]; e2 = pre_pr[PACK ? rt : 0][2]; e3 = pre_pr[PACK ? rt : 0][3];
+                    } else if (INK) {
+                        e0 = now_pr[PACK ? rt : 0][0]; e1 = now_pr[PACK ? rt : 0][1]; e2 = now_pr[PACK ? rt : 0][2]; e3 = now_pr[PACK ? rt : 0][3];
                     } else {
                         int64_t tix = env0 + rt; tix = tix < n_units ? tix : n_units - 1;
                         const int4 pr = a.pairs[tix];
@@ -802,7 +914,7 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                 t_pos = __builtin_amdgcn_readfirstlane(t_pos);
             }
             int4 nxt[PACK ? RT : 1];
-            if (PACK && RT == KRT && next_wg0 >= 0) {
+            if (PACK && !INK && RT == KRT && next_wg0 >= 0) {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
                     int64_t tix = next_wg0 + (int64_t)wave * KRT + rt; tix = tix < n_units ? tix : n_units - 1;
@@ -865,8 +977,13 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             // (vmcnt(0); expcnt / lgkmcnt left at their maxima).  It does not know of the ring's loads, so wherever it
             // later met a value of its own still in flight - or reused such a register - it would wait for "all
             // outstanding loads", i.e. drain the ring in mid-tile; after this it has nothing pending.
+            // INK: the next pass's entries are selected HERE, between this pass's input loads and their wait
+            if (INK && RT == KRT) {
+                have_pre = next_wg0 >= 0;
+                if (have_pre) ink_entries((int)next_wg0 + uwave * KRT, pre_pr);
+            }
             if (RING || DMA) __builtin_amdgcn_s_waitcnt(0x0F70);
-            if (PACK && RT == KRT) {
+            if (PACK && !INK && RT == KRT) {
                 have_pre = next_wg0 >= 0;
                 if (have_pre) {
 #pragma unroll
@@ -902,13 +1019,10 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             }
             // ================= transformer blocks =================
             const int dense_layers = MODE == MODE_FULL ? a.n_layers : a.n_layers - 1;
-            STAMP();
             for (int l = 0; l < dense_layers; ++l) {
                 const float* lv = vlds + V_LAYER0 + l * lv_size(a.F);
                 attention(lv);
-                STAMP();
                 proj_and_ffn(lv);
-                STAMP();
             }
             if (MODE == MODE_HEAD) {
                 // last block: attention only, then park token 0 (lanes r16 == 0) for the TAIL launch
@@ -946,7 +1060,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                 // analysis then takes every value that loop carries - the stage-fetch offsets among them, which must
                 // be scalar operands of the transfer instructions - for lane-dependent.
                 if (MERGE) asm volatile("" ::: "memory");
-                STAMP();
             } else {
                 // ================= readout: token 0 of every env -> 29*K logits + value =================
                 Frag8 yf[RT][KC];
@@ -999,13 +1112,10 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             }
             // MERGE: the rows are waited for here, with the wait the compiler can see (as the tokenizer's loads are)
             if (decltype(tail_tag)::value) __builtin_amdgcn_s_waitcnt(0x0F70);
-            STAMP();
             proj_and_ffn(lv);
-            STAMP();
             Frag8 yf[RT][KC];
             norm_to_frags(fv + FV_LNG, fv + FV_LNB, a.final_ln != 0, yf);
             heads(yf, tenv, tok, fv);
-            STAMP();
         }
     };
     typedef std::integral_constant<int, KRT> rt_bulk;
@@ -1047,10 +1157,10 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
                 // ... and at raised priority: this workgroup's chain of passes is one longer than every other's, so
                 // while it runs the extra one it goes first at the SIMDs' issue ports
                 __builtin_amdgcn_s_setprio(3);
-                pass(rt_one(), head_pass(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
+                pass(rt_one(), head_pass(), rem_tile0 + (int64_t)qi * 4 + uwave, -1);
                 __builtin_amdgcn_s_setprio(0);
             } else if (tile < n_bulk) {
-                const int64_t env0 = tile * ENVS_PER_WG + (int64_t)wave * KRT * ENVS_PER_TILE;
+                const int64_t env0 = tile * ENVS_PER_WG + (int64_t)uwave * KRT * ENVS_PER_TILE;
                 const int64_t ntile = tile + gridDim.x;
                 t_more_head = ntile < n_bulk;
                 pass(rt_bulk(), head_pass(), env0, (PACK && ntile < n_bulk) ? ntile * ENVS_PER_WG : -1);
@@ -1076,7 +1186,6 @@ __global__ __launch_bounds__(256, (KRT <= 2 && !RING) ? 2 : 1) void cfg_forward_
             if (qi >= 0 && qi < rem_passes) pass(rt_one(), head_pass(), rem_tile0 + (int64_t)qi * 4 + wave, -1);
         }
     }
-    STAMP();
     if (RING || DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // no transfer into LDS may outlive the workgroup
     lds_barrier();   // every wave leaves together; no LDS slot is read after this point
 }
@@ -1330,10 +1439,11 @@ size_t dma_dyn_bytes(int n_layers, int F) {
 // two workgroups share a CU in the throughput forms: both rings must fit
 bool dma_fits(int n_layers, int F) { return 2 * (dma_dyn_bytes(n_layers, F) + 2048) <= LDS_PER_WG; }
 
-template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false>
+template <typename DT, int RT, int ACT, int MODE, bool PACK = false, bool RING = false, bool DMA = false, bool INK = false>
 int launch_one(const FwdArgs& a, int cus, hipStream_t st) {
-    const size_t dyn = RING ? ring_dyn_bytes(a.n_layers, a.F) : DMA ? dma_dyn_bytes(a.n_layers, a.F) : (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
-    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK, RING, DMA>;
+    const size_t dyn = RING ? ring_dyn_bytes(a.n_layers, a.F) : DMA ? dma_dyn_bytes(a.n_layers, a.F) + (INK ? INK_BYTES : 0)
+                            : (size_t)vec_floats(a.n_layers, a.F) * sizeof(float);
+    auto kern = cfg_forward_kernel<DT, RT, ACT, MODE, PACK, RING, DMA, INK>;
     if (dyn + sizeof(uint4) * 2 * STAGE_U4 > 64 * 1024) {       // beyond the default per-workgroup LDS window
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
             return BSRL_UNSUPPORTED;
@@ -1362,6 +1472,10 @@ int launch_all(FwdArgs a, bool pruned, bool pack, bool latency, int cus, hipStre
     a.s_begin = 0; a.s_end = split;
     a.t_begin = split; a.t_end = total;
     int rc;
+    if (pack && dma && a.B <= INK_MAX_ENVS && 2 * (dma_dyn_bytes(a.n_layers, a.F) + INK_BYTES + 2048) <= LDS_PER_WG) {
+        // the tile table lives in every workgroup's LDS: no table kernel (same grid sizing as below)
+        return launch_one<DT, 2, ACT, MODE_HEAD, true, false, true, true>(a, cus, st);
+    }
     if (pack) {
         // the grid is sized for the unpacked tile count (the packed one is known on the device only); workgroups past
         // the packed count leave after their prologue
