@@ -83,6 +83,9 @@ def main(argv=None):
     ap.add_argument("--fused-ffn", action="store_true", help="block FFNs forward as the fused kernel, which also writes the hidden for the backward")
     ap.add_argument("--fused-ffn-recompute", action="store_true", help="fused FFN forward that keeps no hidden: the backward recomputes it (less memory)")
     ap.add_argument("--no-step", action="store_true", help="forward + backward only (no clip, no optimizer)")
+    ap.add_argument("--update-values", default="rollout", choices=("rollout", "own"),
+                    help="rollout (default): the update forward also runs the rollout's fused forward and returns its "
+                         "logits / value bits; own: the per-op forward's values (no second forward)")
     args = ap.parse_args(argv)
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
@@ -96,6 +99,7 @@ def main(argv=None):
         policy.stream_dtype = torch.bfloat16 if args.bf16 else torch.float16
     if args.fused_ffn or args.fused_ffn_recompute:
         policy.fused_ffn = policy.arch["fused_ffn"] = "recompute" if args.fused_ffn_recompute else "on"
+    policy.update_values = args.update_values
     scale = 4096.0 if policy.fp16 else 1.0
     opt = torch.optim.Adam(policy.parameters(), lr=LR)
     print(f"gpu: {torch.cuda.get_device_name(0)}  torch {torch.__version__}  stream "

@@ -247,6 +247,19 @@ class Block(nn.Module):
         return r + (v,) if want_v else r
 
 
+class _ValuesOf(torch.autograd.Function):
+    """forward: `values`, bit for bit; backward: the incoming gradient goes to `graph` (same shape), the tensor whose
+    autograd graph stands in for the way `values` were computed."""
+
+    @staticmethod
+    def forward(ctx, graph, values):
+        return values.detach().clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, None
+
+
 def _block_train(self, x, attn_bias, n_queries=0, v0=None, want_v=False, fused_ffn=False):
     """Block.forward under autograd (update path): the same kernels in the same order as the per-op
     rollout route without the fused FFN, each paired with its backward; returns x_out (, v).
@@ -415,6 +428,14 @@ class NotePolicy(nn.Module):
         # value to ~2e-4 at the recipe shape).  True: the rollout takes the per-op route and the reference's critic op
         # order whatever the two switches say - same bits as the update forward, at the per-op route's speed.
         self.rollout_matches_update = False
+        # The same contract from the other side, at the fast routes' rollout speed: "rollout" = the update forward
+        # RETURNS the rollout forward's logits and value - it runs that forward too, grad-free, on the routes the
+        # rollout takes - and sends their gradients through its own per-op graph (a function that differs from the
+        # rollout's by 16-bit rounding, as any two 16-bit evaluations do).  Rollout and update outputs are then the
+        # same bits in every mode and PPO's first-epoch ratio is exactly 1, for one more (fused, ~3 ms at the recipe
+        # shape and 16384 envs) forward per update pass.  "own": the update returns its own per-op values (the gap
+        # bounded in the tests).  No effect on the fp32 stream, whose two forwards are the same ops.
+        self.update_values = "rollout"
         # sampling-call counter of the in-kernel Philox stream; on the device so that a captured
         # get_action_and_value draws fresh noise on every replay
         self.register_buffer("_sample_ctr", torch.zeros(1, dtype=torch.int64), persistent=False)
@@ -515,6 +536,13 @@ class NotePolicy(nn.Module):
         if obs.dim() != 2 or obs.shape[1] != OBS_DIM:
             raise RuntimeError(f"obs must be (B, {OBS_DIM}), got {tuple(obs.shape)}")
         if torch.is_grad_enabled():
+            if self.update_values not in ("rollout", "own"):
+                raise ValueError(f"update_values must be 'rollout' or 'own', got {self.update_values!r}")
+            if self.update_values == "rollout" and self.fp16 and not self.rollout_matches_update:
+                with torch.no_grad():
+                    r_out, r_value = self.forward_stacked(obs)       # the rollout's own routes, grad-free
+                out, value = self._forward_train(obs)
+                return _ValuesOf.apply(out, r_out), _ValuesOf.apply(value, r_value)
             return self._forward_train(obs)
         with contextlib.ExitStack() as modes:
             if self.fp16 and self.fp16_accum != "off":

@@ -41,6 +41,9 @@ def _policy(seed, **kw):
         for p in m.parameters():
             if p.dim() == 1:
                 p.add_(0.1 * torch.randn_like(p))
+    # these tests hold the update path's OWN forward and backward against the oracle: its own values, not the rollout's
+    # (the default "rollout" is covered by test_update_forward_returns_the_rollout_bits_on_the_default_routes)
+    m.update_values = "own"
     return m
 
 
@@ -155,35 +158,61 @@ def _group(name):
     return "encoder"
 
 
-def test_rollout_update_gap_on_the_default_routes_is_bounded_and_the_switch_closes_it():
-    """The reference holds rollout == update bitwise (python/tests/test_fp16_accum.py:146-160).  Here the DEFAULT
-    rollout (fused block stack + pooled critic) and the update forward differ by 16-bit rounding; this test bounds the
-    gap at the recipe shape with literal ceilings (measured at B = 4096: log-prob of the 29-head action 8.9e-3, i.e.
-    a first-epoch PPO ratio within 0.9 % of 1; logits 2.5e-3; value 1.5e-4), and shows that
-    `rollout_matches_update = True` restores the reference's contract: identical logits and value bits."""
+def test_update_forward_returns_the_rollout_bits_on_the_default_routes():
+    """The reference holds rollout == update bitwise in every mode (python/tests/test_fp16_accum.py:146-160,
+    tests/test_fused_ffn.py:471-495).  Here the DEFAULT rollout (fused block stack + pooled critic) is not the per-op
+    route the update differentiates, so the update forward also runs the rollout's forward and returns ITS logits and
+    value (`update_values = "rollout"`, the default): identical bits, gradients through the per-op graph.  With
+    `update_values = "own"` the update returns its per-op values and the gap is the 16-bit rounding between the two
+    routes, bounded here with literal ceilings (measured at B = 4096: log-prob of the 29-head action 8.9e-3, logits
+    2.5e-3, value 1.5e-4); `rollout_matches_update = True` closes it from the rollout's side (per-op rollout)."""
     torch.manual_seed(0)
     m = NotePolicy(embed=192, trunk_dim=384, n_blocks=6, n_heads=4, n_gears=5, ffn_mult=4, note_geo=True).to(DEV)
     m.fp16 = True
-    assert m.fused_blocks == "auto" and m.critic_pool and not m.rollout_matches_update
+    assert m.fused_blocks == "auto" and m.critic_pool and not m.rollout_matches_update and m.update_values == "rollout"
     od = _obs(4096, 0).to(DEV)
     with torch.no_grad():
         assert m.fused_blocks_ok(torch.float16)
         act, logp_r, _, v_r = m.get_action_and_value(od)
         lg_r, _ = m.forward_stacked(od)
+    # default: the update's outputs ARE the rollout's
     _, logp_u, _, v_u = m.get_action_and_value(od, action=act)
-    lg_u, _ = m.forward_stacked(od)
-    logp_u, v_u, lg_u = logp_u.detach(), v_u.detach(), lg_u.detach()
-    g_logp, g_lg, g_v = (logp_r - logp_u).abs().max().item(), (lg_r - lg_u).abs().max().item(), (v_r - v_u).abs().max().item()
-    print(f"\nrollout(default routes) vs update: |dlogp| {g_logp:.3e} (ratio off 1 by {(torch.exp(logp_u - logp_r) - 1).abs().max().item():.3e}), "
-          f"|dlogit| {g_lg:.3e}, |dvalue| {g_v:.3e}")
+    lg_u, v_u2 = m.forward_stacked(od)
+    assert lg_u.requires_grad and v_u.requires_grad
+    assert torch.equal(lg_u.detach(), lg_r) and torch.equal(v_u.detach(), v_r) and torch.equal(v_u2.detach(), v_r)
+    assert (logp_u.detach() - logp_r).abs().max().item() <= 5e-5     # same logits; kernel vs torch log-softmax summation
+    # ... and the gradients are the per-op graph's: the same loss differentiated with update_values = "own" gives
+    # gradients that agree to the rounding between the two forwards' values
+    def grads(mode):
+        m.update_values = mode
+        m.zero_grad(set_to_none=True)
+        lg, v = m.forward_stacked(od[:512])
+        (torch.log_softmax(lg, -1)[..., 0].sum() + v.sum()).backward()
+        return {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+    g_roll, g_own = grads("rollout"), grads("own")
+    assert g_roll.keys() == g_own.keys() and len(g_roll) > 50
+    gmax = max(g.norm().item() for g in g_own.values())
+    for n in g_roll:
+        # (k_proj.bias has a zero gradient in exact arithmetic - a softmax does not see a shift of all its keys -: its
+        # two rounding-noise vectors are compared on the scale of the model's gradients, like every near-zero one)
+        num, den = (g_roll[n] - g_own[n]).norm().item(), g_own[n].norm().item()
+        assert num <= 2e-2 * den + 1e-4 * gmax, (n, num, den, gmax)
+    # "own": the bounded gap
+    m.update_values = "own"
+    _, logp_o, _, v_o = m.get_action_and_value(od, action=act)
+    lg_o, _ = m.forward_stacked(od)
+    logp_o, v_o, lg_o = logp_o.detach(), v_o.detach(), lg_o.detach()
+    g_logp, g_lg, g_v = (logp_r - logp_o).abs().max().item(), (lg_r - lg_o).abs().max().item(), (v_r - v_o).abs().max().item()
+    print(f"\nrollout(default routes) vs the update's own values: |dlogp| {g_logp:.3e} (ratio off 1 by "
+          f"{(torch.exp(logp_o - logp_r) - 1).abs().max().item():.3e}), |dlogit| {g_lg:.3e}, |dvalue| {g_v:.3e}")
     assert 0 < g_logp <= 1.2e-2 and g_lg <= 3.5e-3 and g_v <= 3e-4
     m.rollout_matches_update = True
     with torch.no_grad():
         assert not m.fused_blocks_ok(torch.float16)
         lg_s, v_s = m.forward_stacked(od)
         _, logp_s, _, _ = m.get_action_and_value(od, action=act)
-    assert torch.equal(lg_s, lg_u) and torch.equal(v_s, v_u)
-    assert (logp_s - logp_u).abs().max().item() <= 5e-5        # same logits; kernel vs torch log-softmax summation
+    assert torch.equal(lg_s, lg_o) and torch.equal(v_s, v_o)
+    assert (logp_s - logp_o).abs().max().item() <= 5e-5
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
