@@ -123,25 +123,40 @@ def _replica_padded(w: torch.Tensor, dtype: torch.dtype, k_pad: int) -> torch.Te
     return cache[1]
 
 
-def packed_halves(ms, dtype=torch.float16):
+def packed_halves(ms, dtype=torch.float16, pad_rows=None, pad_bias=0.0):
     """(w_cat in `dtype`, b_cat fp32) for an ordered group of same-input Linears.  16-bit copies are refreshed per
     weights version (bump_weights_version), like every replica.  The fp32 "copy" is a plain concatenation of the
     masters: the reference's fp32 forward reads the masters themselves (python/policy.py:1371-1376), so it is also
-    rebuilt whenever torch's own in-place counters of the members move (any in-place edit, with or without a bump)."""
+    rebuilt whenever torch's own in-place counters of the members move (any in-place edit, with or without a bump).
+    pad_rows: every member's block is padded to that many output rows with zero weights and bias `pad_bias` - the
+    packed action heads with per-joint gear counts come out of ONE GEMM already in the (29, k_max) layout, the lanes past
+    a head's count holding the masked-logit constant exactly (0 + pad_bias in fp32), where the reference scatters the
+    ragged GEMM output over a constant fill (python/policy.py:1337-1344)."""
     key = ms[0].weight
     ident = tuple(id(m) for m in ms)                      # the members, not just the first one and the count
     table = getattr(key, "_bsrl_packed", None)
     if table is None:
         table = key._bsrl_packed = {}
-    cache = table.get((ident, dtype))
+    cache = table.get((ident, dtype, pad_rows))
     tv = tuple((m.weight._version, m.bias._version) for m in ms) if dtype is torch.float32 else None
+
+    def cat_w():
+        if pad_rows is None:
+            return torch.cat([m.weight.detach() for m in ms])
+        return torch.cat([torch.cat([m.weight.detach(), m.weight.new_zeros(pad_rows - m.out_features, m.in_features)])
+                          for m in ms])
+
+    def cat_b():
+        if pad_rows is None:
+            return torch.cat([m.bias.detach() for m in ms])
+        return torch.cat([torch.cat([m.bias.detach(), m.bias.new_full((pad_rows - m.out_features,), pad_bias)]) for m in ms])
+
     if cache is None or cache[1].device != key.device:
-        cache = [_weights_version, torch.cat([m.weight.detach() for m in ms]).to(dtype).contiguous(),
-                 torch.cat([m.bias.detach() for m in ms]).float().contiguous(), tv]
-        table[(ident, dtype)] = cache
+        cache = [_weights_version, cat_w().to(dtype).contiguous(), cat_b().float().contiguous(), tv]
+        table[(ident, dtype, pad_rows)] = cache
     elif cache[0] != _weights_version or cache[3] != tv:
-        cache[1].copy_(torch.cat([m.weight.detach() for m in ms]))
-        cache[2].copy_(torch.cat([m.bias.detach() for m in ms]))
+        cache[1].copy_(cat_w())
+        cache[2].copy_(cat_b())
         cache[0], cache[3] = _weights_version, tv
     return cache[1], cache[2]
 

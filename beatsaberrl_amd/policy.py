@@ -488,6 +488,14 @@ class NotePolicy(nn.Module):
             c[0] = _fl._weights_version
         return c[2]
 
+    def _heads_packed(self, dt):
+        """The 29 action heads as ONE packed (29 k_max, trunk_dim) matrix + fp32 bias (python/policy.py:1311-1335).  With
+        per-joint gear counts every head's block is padded to k_max rows - zero weights, the masked-logit constant as
+        bias - so the GEMM's output IS the (29, k_max) layout with its masked lanes (python/policy.py:1337-1344 scatters
+        over a constant fill instead)."""
+        ragged = self._gear_idx is not None
+        return _fl.packed_halves(list(self.heads), dt, pad_rows=self.k_max if ragged else None, pad_bias=MASKED_LOGIT)
+
     def refresh_fp16_caches(self):
         """Force every weight copy the kernels read up to date for the current weights version
         (python/policy.py:1448-1461): call after optimizer steps under a captured graph.  On the
@@ -510,7 +518,7 @@ class NotePolicy(nn.Module):
             _fl.packed_halves([blk.q_proj, blk.k_proj, blk.v_proj], dt)
             _fl.packed_halves([blk.k_proj, blk.v_proj], dt)
         _fl.packed_halves([self.critic_k, self.critic_v], dt)
-        _fl.packed_halves(list(self.heads), dt)
+        self._heads_packed(dt)
         if self.critic_pool:
             self._critic_pool_weights(dt)
 
@@ -603,15 +611,18 @@ class NotePolicy(nn.Module):
             with torch.cuda.stream(side):
                 attended = self._critic_attend(x_res, attn_bias)
         hfeat = self._trunk(lead.reshape(B, self.n_lead * d))
-        wh, bh = _fl.packed_halves(list(self.heads), dt)
-        out = ops.linear(hfeat, wh, bh, out_dtype=torch.float32)           # (B, sum n_j) fp32
+        wh, bh = self._heads_packed(dt)
+        out = ops.linear(hfeat, wh, bh, out_dtype=torch.float32)           # (B, 29 k_max) fp32, masked lanes included
         if side is not None:
             main.wait_stream(side)
+            # the pool's outputs were allocated on the side stream and are read on this one: tell the allocator, so that
+            # their blocks are not handed out again on the side stream while this stream's reads are still pending
+            for t in (attended if isinstance(attended, (tuple, list)) else (attended,)):
+                if torch.is_tensor(t):
+                    t.record_stream(main)
         else:
             attended = self._critic_attend(x_res, attn_bias)
         value = self._critic_value(attended, hfeat)
-        if self._gear_idx is not None:
-            out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
         return out.view(B, N_ACTION_HEADS, self.k_max), value
 
     def _forward_train(self, obs):
@@ -657,8 +668,14 @@ class NotePolicy(nn.Module):
             t = _lin_t(self.trunk_proj, z)
             hfeat = self.trunk_ln2(ChainFn.apply(self.trunk_ln1(t), t, False, self.trunk_fc1.weight, self.trunk_fc1.bias,
                                                  self.trunk_fc2.weight, self.trunk_fc2.bias))
-        out = LinearFn.apply(hfeat, torch.cat([m.weight for m in self.heads]), torch.cat([m.bias for m in self.heads]),
-                             None, None, True)
+        if self._gear_idx is None:
+            w_heads, b_heads = torch.cat([m.weight for m in self.heads]), torch.cat([m.bias for m in self.heads])
+        else:       # per-joint gear counts: every head padded to k_max rows (zero weights, the masked-logit constant as bias)
+            w_heads = torch.cat([torch.cat([m.weight, m.weight.new_zeros(self.k_max - m.out_features, m.in_features)])
+                                 for m in self.heads])
+            b_heads = torch.cat([torch.cat([m.bias, m.bias.new_full((self.k_max - m.out_features,), MASKED_LOGIT)])
+                                 for m in self.heads])
+        out = LinearFn.apply(hfeat, w_heads, b_heads, None, None, True)
         # critic (adapool_v1)
         hv = self.critic_ln(x_res)
         q = _lin_t(self.critic_q, hv[:, 2:3])
@@ -667,8 +684,6 @@ class NotePolicy(nn.Module):
         vlogits = _seq_t(self.critic_mlp, torch.cat([a, hfeat], dim=-1), out_f32=True)
         self._value_logits = vlogits
         value = torch.softmax(vlogits, dim=-1) @ self.value_centers
-        if self._gear_idx is not None:
-            out = out.new_full((B, N_ACTION_HEADS * self.k_max), MASKED_LOGIT).index_copy(1, self._gear_idx, out)
         return out.view(B, N_ACTION_HEADS, self.k_max), value
 
     def _trunk_v2_train(self, z):

@@ -226,7 +226,7 @@ int64_t bsrl_cfg_pack_size(const bsrl_cfg_desc* desc);
  * image (the analogue of fp16_linear.flat_refresh, fp16_linear.py:241-246). */
 int bsrl_cfg_pack(const bsrl_cfg_desc* desc, const bsrl_cfg_params* params,
                   void* packed, bsrl_stream stream);
-/* Bytes of scratch the pruned two-launch form of bsrl_cfg_forward needs for B envs
+/* Bytes of scratch the pruned form of bsrl_cfg_forward needs for B envs
  * (768 B per env for the parked rows + 16 B per env + 16 B for the tile table of
  * the packed launch), or 0 if the shape is unsupported. */
 int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
@@ -234,20 +234,27 @@ int64_t bsrl_cfg_workspace_size(const bsrl_cfg_desc* desc, int64_t B);
  * workspace == NULL (or smaller than bsrl_cfg_workspace_size): ONE persistent
  * kernel computes every token of every block.  With a workspace: final-block
  * query pruning, the reference's n_queries path (python/policy.py:533-539,
- * :1302-1305; exact, masking is key-side only) - launch 1 runs the tokenizer,
- * blocks 0..L-2 and the last block's attention and parks each env's token-0
- * row in the workspace, launch 2 runs the last block's output projection +
- * FFN and the heads on those rows, 16 envs per MFMA tile.  With n_valid given
- * and the full workspace, launch 1 also packs short envs into shared 16-row
- * tiles under a block-diagonal key mask: two of 5..8 tokens (n_valid 4..7) at
- * rows 0 / 8; one of at most 4 tokens (n_valid <= 3) at rows 12.. behind one of
- * 9..12 tokens, or four of them at rows 0 / 4 / 8 / 12 (a small kernel builds
- * the tile table on the stream first):
- * padded rows are what the reference computes and discards
- * (python/policy.py:1257-1260 masks them key-side), and an env's output bits
- * are the same packed or alone.  desc->flags = BSRL_CFG_NO_PACK keeps one env
- * per tile; a workspace of only 768 B per env, or an n_valid that is not
- * 16-byte aligned, does too. */
+ * :1302-1305; exact, masking is key-side only): the tokenizer, blocks 0..L-2
+ * and the last block's attention run on whole envs, each env's token-0 row is
+ * parked in the workspace, and the last block's output projection + FFN and
+ * the heads run on those rows, 16 envs per MFMA tile.  That is ONE launch:
+ * every workgroup runs the tail of the envs it parked itself, whenever 64 of
+ * them wait and once more at the end; no workgroup waits for another.  (Models
+ * whose weight ring cannot live in LDS twice per CU - vectors + 96 KB beyond
+ * 160 KB - run the tail as a second launch.)  With n_valid given and the full
+ * workspace, short envs share 16-row tiles under a block-diagonal key mask:
+ * two of 5..8 tokens (n_valid 4..7) at rows 0 / 8; one of at most 4 tokens
+ * (n_valid <= 3) at rows 12.. behind one of 9..12 tokens, or four of them at
+ * rows 0 / 4 / 8 / 12.  Up to 16384 envs every workgroup derives its tiles
+ * from the key counts itself (class prefixes in LDS); beyond, a small kernel
+ * builds the tile table in the workspace on the stream first.  Padded rows are
+ * what the reference computes and discards (python/policy.py:1257-1260 masks
+ * them key-side), and an env's output bits are the same packed or alone.
+ * desc->flags = BSRL_CFG_NO_PACK keeps one env per tile; a workspace of only
+ * 768 B per env, or an n_valid that is not 16-byte aligned, does too.
+ * Batches of at most 4 envs per CU take the latency form (one launch, no
+ * workspace use) unless BSRL_CFG_NO_LATENCY is set.  All forms give the same
+ * output bits. */
 int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
                      const void* obs, int64_t obs_ld, int obs_dtype,
                      const int32_t* n_valid, float* logits, float* value,
@@ -257,17 +264,23 @@ int bsrl_cfg_forward(const bsrl_cfg_desc* desc, const void* packed,
 /* bsrl_cfg_forward for callers that cannot allocate device memory: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
  * has no counterpart in the reference (whose ops allocate their outputs,
- * layer_norm.cu:545-547).  Same arguments and results as bsrl_cfg_forward in its
- * two-launch form with short envs sharing tiles, bit for bit, but the parked
- * rows and the tile table live in a device array built into the library
+ * layer_norm.cu:545-547).  Same arguments and results as bsrl_cfg_forward with a
+ * full workspace - the same kernels on the same launch shapes, so the same
+ * output bits - but the parked rows (and, beyond the in-kernel tile table's
+ * batch limit, the tile table) live in a device array built into the library
  * (BSRL_CFG_STATIC_MAX_ENVS * 784 + 16 bytes, held on every GPU the library is
  * used on until the process ends) instead of a caller workspace; the call
- * allocates and frees nothing.  B > BSRL_CFG_STATIC_MAX_ENVS is an error
- * (BSRL_EINVAL); ffn not a multiple of 64 returns BSRL_UNSUPPORTED.  Every call
- * on one GPU shares that GPU's array: calls that overlap in time on one GPU
- * (two streams, two threads) race - serialise them or use bsrl_cfg_forward
- * with one workspace per stream.  Nothing in the array has to be cleared
- * between calls. */
+ * allocates and frees nothing.  Batches of at most 4 envs per CU take the
+ * latency form here too, which uses no scratch at all.  B >
+ * BSRL_CFG_STATIC_MAX_ENVS is an error (BSRL_EINVAL); ffn not a multiple of 64
+ * returns BSRL_UNSUPPORTED.  Every call on one GPU shares that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race -
+ * serialise them or use bsrl_cfg_forward with one workspace per stream.
+ * Nothing in the array has to be cleared between calls.  The FIRST call on a
+ * device takes the array's address (hipGetSymbolAddress: the runtime loads
+ * the code object) and may raise a kernel's LDS limit (hipFuncSetAttribute):
+ * make it outside stream capture; later calls only launch and are capturable
+ * (tests/test_zz_no_alloc.py replays one from a graph). */
 #define BSRL_CFG_STATIC_MAX_ENVS 16384
 int bsrl_cfg_forward_static(const bsrl_cfg_desc* desc, const void* packed,
                             const void* obs, int64_t obs_ld, int obs_dtype,
