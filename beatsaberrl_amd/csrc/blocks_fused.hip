@@ -1006,13 +1006,14 @@ struct FfnArgs {
 // nothing to run meanwhile; a second, independent workgroup drifts out of phase and computes through it.
 // d = 384: a wave's state (fp32 accumulator 192 registers, input fragments 96) wants the whole register file of a SIMD:
 // four waves, ONE workgroup per CU, 512 registers each; stages of 24 KB.
-template <int D, int NW> struct FfnRing : StageRing<Geo<D>::SF, NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : D == 192 ? 6 : 5), NW> {};
+// (XS: one more slot where the vectors leave room for it - a stage more in flight behind the pair being consumed)
+template <int D, int NW, int XS = 0> struct FfnRing : StageRing<Geo<D>::SF, (NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : D == 192 ? 6 : 5)) + XS, NW> {};
 template <int D, int NW> constexpr int ffn_wgs_per_cu() { return D == 384 ? 1 : 8 / NW; }
 
-template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_>
+template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_, int XS>
 __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
-    typedef FfnRing<D, NW_> R;
+    typedef FfnRing<D, NW_, XS> R;
     constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
     extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
     float* vlds = reinterpret_cast<float*>(bvl4);
@@ -1047,7 +1048,36 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         const int64_t row0 = (tile * NW + wave) * 32;
         f32x4 x[2][NT];
         BFrag8 hf[2][KC];
-        {   // the tile's own loads: all issued, one wait the compiler can see (it does not know of the ring's transfers)
+        if constexpr (D == 384) {
+            // x and its accumulator first, h2 after them: with both raw inputs and the accumulator live at once the
+            // register allocator spills operand fragments, and reloads them from scratch in every chunk of the loop
+            // below (whose waits on those reloads drain the ring's transfers too)
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
+                const u16* xr = a.x + row * D;
+                uint2 rx[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) rx[nt] = *reinterpret_cast<const uint2*>(xr + 16 * nt + 4 * g);
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4 b = *reinterpret_cast<const float4*>(B2 + 16 * nt + 4 * g);
+                    x[rt][nt][0] = DT::to_f((u16)(rx[nt].x & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(rx[nt].x >> 16)) + b.y;
+                    x[rt][nt][2] = DT::to_f((u16)(rx[nt].y & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(rx[nt].y >> 16)) + b.w;
+                    asm("" : "+a"(x[rt][nt]));        // the accumulator lives in accumulation registers from here on
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
+                const u16* hr = a.h2 + row * D;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) hf[rt][nt >> 1].h[nt & 1] = *reinterpret_cast<const uint2*>(hr + 16 * nt + 4 * g);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        } else {   // the tile's own loads: all issued, one wait the compiler can see (it does not know of the ring's transfers)
             uint2 rx[2][NT], rh[2][NT];
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
@@ -1089,8 +1119,53 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 });
             });
         };
+        // PIPE (one wave per SIMD: nothing else runs while a wave waits): the fragment reads run NBUF - 1 fragments ahead
+        // of the MFMAs through a rotating set of NBUF registers quads, across stage boundaries too - before the two
+        // MFMAs of fragment i are issued, fragment i + NBUF - 1 is requested (behind the next stage's admission when it
+        // opens a stage), and a scheduling barrier keeps the request above the MFMAs.  SF is a multiple of NBUF, so a
+        // fragment's register set is the same in every stage.
+        constexpr bool PIPE = D == 384;
+        constexpr int NBUF = 4, SF = G::SF;
+        static_assert(!PIPE || SF % NBUF == 0, "rotating fragment registers");
+        s16x8 wr[NBUF];
+        // one stage: mm(i, fragment) per fragment; next: 0 = nothing follows in this tile, 1 = an odd stage (entered
+        // without a barrier), 2 = an even one (the pair admission, which reuses the slot of the stage being left: every
+        // wave's reads of it must have returned before the barrier)
+        auto stage = [&](int next, auto&& mm) __attribute__((always_inline)) {
+            static_for<0, SF>([&](auto i_) __attribute__((always_inline)) {
+                constexpr int i = decltype(i_)::value, n = i + NBUF - 1;
+                if constexpr (n < SF) wr[n % NBUF] = pipe.frag(n, lane);
+                else if (next) {
+                    if constexpr (n == SF) {
+                        if (next == 2) { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); advance(Even{}); }
+                        else advance(Odd{});
+                    }
+                    wr[n % NBUF] = pipe.frag(n - SF, lane);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                mm(i_, wr[i % NBUF]);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        auto up_init = [&](int ch) __attribute__((always_inline)) {
+#pragma unroll
+            for (int ntl = 0; ntl < 2; ++ntl) {
+                const float4 b = *reinterpret_cast<const float4*>(B1 + 32 * ch + 16 * ntl + 4 * g);
+                acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
+            }
+        };
+        auto up_mm = [&](auto i_, const s16x8& wf) __attribute__((always_inline)) {
+            constexpr int j = decltype(i_)::value / KB, ci = decltype(i_)::value % KB, half = j / 2, ntl = j % 2;
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) acc[ntl][rt] = DT::mfma32(wf, hf[rt][half * KB + ci].v, acc[ntl][rt]);
+        };
         advance(Even{});
-        up(0);
+        if (PIPE) {      // an odd stage follows W1(0): W1(1), or W2(0) when nch == 1
+#pragma unroll
+            for (int f = 0; f < NBUF - 1; ++f) wr[f] = pipe.frag(f, lane);
+            up_init(0); stage(1, up_mm);
+        }
+        else up(0);
         for (int ch = 0; ch < nch; ++ch) {
             BFrag8 hid[2];
 #pragma unroll
@@ -1115,17 +1190,27 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 }
             }
             // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
-            if (ch + 1 < nch) { advance(Odd{}); up(ch + 1); advance(Even{}); }
-            else advance(Odd{});
-            static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
-                constexpr int j = decltype(j_)::value;           // feature tiles [j * KB, +KB)
-                sub(j_, [&](const s16x8 (&w2)[KB]) __attribute__((always_inline)) {
+            if (PIPE) {
+                // the stage in the ring and its first NBUF - 1 fragments were requested by the stage before
+                if (ch + 1 < nch) { up_init(ch + 1); stage(2, up_mm); }                  // W1(ch + 1), then W2(ch): even
+                stage(ch + 1 < nch ? 1 : 0, [&](auto i_, const s16x8& w2) __attribute__((always_inline)) {   // W2(ch); an odd stage follows but the last
+                    constexpr int i = decltype(i_)::value;       // feature tile i
 #pragma unroll
-                    for (int i = 0; i < KB; ++i)
-#pragma unroll
-                        for (int rt = 0; rt < 2; ++rt) x[rt][j * KB + i] = DT::mfma32(w2[i], hid[rt].v, x[rt][j * KB + i]);
+                    for (int rt = 0; rt < 2; ++rt) x[rt][i] = DT::mfma32(w2, hid[rt].v, x[rt][i]);
                 });
-            });
+            } else {
+                if (ch + 1 < nch) { advance(Odd{}); up(ch + 1); advance(Even{}); }
+                else advance(Odd{});
+                static_for<0, NSUB>([&](auto j_) __attribute__((always_inline)) {
+                    constexpr int j = decltype(j_)::value;           // feature tiles [j * KB, +KB)
+                    sub(j_, [&](const s16x8 (&w2)[KB]) __attribute__((always_inline)) {
+#pragma unroll
+                        for (int i = 0; i < KB; ++i)
+#pragma unroll
+                            for (int rt = 0; rt < 2; ++rt) x[rt][j * KB + i] = DT::mfma32(w2[i], hid[rt].v, x[rt][j * KB + i]);
+                    });
+                });
+            }
         }
         // epilogue: round, store, optional LayerNorm on the rounded row
         float s[2] = {0.f, 0.f}, q[2] = {0.f, 0.f};
@@ -1212,12 +1297,12 @@ bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
     return 2 * (F / 32) >= slots;
 }
 int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
-template <int D, int NW> size_t ffn_dyn_bytes(int F) {
-    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW>::SLOTS * FfnRing<D, NW>::STAGE_BYTES;
+template <int D, int NW, int XS> size_t ffn_dyn_bytes(int F) {
+    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW, XS>::SLOTS * FfnRing<D, NW, XS>::STAGE_BYTES;
 }
-template <typename DT, int D, int ACT, int NW>
+template <typename DT, int D, int ACT, int NW, int XS = 0>
 int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
-    const size_t dyn = ffn_dyn_bytes<D, NW>(a.F);
+    const size_t dyn = ffn_dyn_bytes<D, NW, XS>(a.F);
     constexpr int WGS = ffn_wgs_per_cu<D, NW>();
     if (WGS * (dyn + 1024) > (size_t)LDS_BUDGET) return BSRL_UNSUPPORTED;
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32), slots = (int64_t)cus * WGS;
@@ -1228,13 +1313,19 @@ int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
         hipLaunchKernelGGL(kern, grid, dim3(NW * 64), dyn, st, a);
         return (int)BSRL_OK;
     };
-    if (a.hid) return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, true, NW>) : launch(ffn_rows_kernel<DT, D, ACT, false, true, NW>);
-    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW>);
+    if (a.hid) return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, true, NW, XS>) : launch(ffn_rows_kernel<DT, D, ACT, false, true, NW, XS>);
+    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW, XS>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW, XS>);
 }
 template <typename DT, int D, int ACT>
 int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
-    if constexpr (D == 384) return ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
-    else if constexpr (D != 256) {
+    if constexpr (D == 384) {
+        // six slots of 24 KB where the vectors fit beside them (F up to 2560) and the image is that long, else five
+        if (a.total_stages >= FfnRing<D, 4, 1>::SLOTS) {
+            const int rc = ffn_launch_nw<DT, D, ACT, 4, 1>(a, ln, cus, st);
+            if (rc != BSRL_UNSUPPORTED) return rc;
+        }
+        return ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
+    } else if constexpr (D != 256) {
         // two 4-wave workgroups per CU where two rings fit and the image is longer than the shorter ring
         if (a.total_stages >= FfnRing<D, 4>::SLOTS) {
             const int rc = ffn_launch_nw<DT, D, ACT, 4>(a, ln, cus, st);
