@@ -245,7 +245,7 @@ def main():
         d_, T_, F_ = spec.d, spec.T, spec.ffn
         saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the 15 unread tokens
         exec_flops = dense_flops - 2 * saved * B
-    # ... and, on the fused route, the 16-row tiles the first launch really runs: envs of 5..8 tokens go two to a
+    # ... and, on the fused route, the 16-row tiles the launch really runs: envs of 5..8 tokens go two to a
     # tile, of at most 4 tokens behind an env of 9..12 tokens or four to a tile (same output bits), so the per-tile
     # work is counted per tile
     tiles, issued_flops = None, None
@@ -266,8 +266,10 @@ def main():
     run_flops = issued_flops if issued_flops is not None else exec_flops
     achieved = run_flops / (dev_ms_avg * 1e-3) / 1e12
     peak = MFMA_PEAK_TFLOPS[dtype]
-    kname = ("cfg_pair_kernel + cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0, short envs share tiles)"
-             if tiles is not None else
+    kname = ("cfg_forward_kernel, ONE launch (tile table built in the kernel; final block pruned to token 0 and run by the "
+             "workgroup that parked the rows; short envs share tiles)" if tiles is not None and B <= 16384 else
+             "cfg_pair_kernel (tile table) + cfg_forward_kernel, one merged launch (final block pruned to token 0, short envs "
+             "share tiles)" if tiles is not None else
              "cfg_embed_kernel + blocks_kernel (final block pruned to token 0) + heads" if route == "blocks" else
              "cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
              "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else
