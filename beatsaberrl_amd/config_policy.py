@@ -11,8 +11,10 @@ whose last row is the value.
 
 Three routes, all entirely on the C-ABI kernels:
   * "ops":    one kernel per op (tokenizer, LayerNorm, packed QKV linear,
-              attention, out-proj + residual, LayerNorm, FFN up + act,
-              FFN down + residual, heads) - any supported shape and dtype;
+              attention, out-proj + residual, LayerNorm, FFN - one fused
+              kernel where the shape has one, else up + act and down +
+              residual -, heads; final block pruned to token 0) - any
+              supported shape and dtype;
   * "fused":  the whole forward in one persistent kernel reading a packed
               weight image (16-bit dtypes, T = 16 / d = 128);
   * "blocks": tokenizer kernel, then the whole block stack in one persistent
@@ -79,8 +81,8 @@ class ConfigPolicy(nn.Module):
         # straight into a deep LDS ring - the lowest latency per forward (B = 1: 33 us against 52); same output bits as
         # the throughput forms, so it is on by default.  False: the throughput forms at every batch size
         self.latency_form = True
-        # final-block query pruning on the fused route (the reference's n_queries path,
-        # python/policy.py:533-539): exact; False = one persistent kernel computing every token
+        # final-block query pruning on the fused and per-op routes (the reference's n_queries path,
+        # python/policy.py:533-539): exact; False = every token of the final block computed (fused: one persistent kernel)
         self.prune_final = True
         # fused route, pruned form, key counts given: envs of at most 8 tokens share 16-row tiles in twos, of at most 4 tokens ride behind a 9..12-token env or in fours (same bits)
         self.pack_short = True
@@ -304,9 +306,18 @@ class ConfigPolicy(nn.Module):
         for i, (blk, w) in enumerate(zip(self.blocks, r["blk"])):
             if h is None:
                 h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
-            qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                       # (B, T, 3d)
-            att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
-            x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                           # x + out(att)
+            if self.prune_final and i + 1 == len(self.blocks):
+                # Only token 0 of the final block is read (the reference's n_queries path, python/policy.py:533-539:
+                # exact, masking is key-side only): keys and values of every token, the query, the output projection,
+                # LN2 and the FFN of token 0 alone.  Row slices of the packed q|k|v weight are contiguous views.
+                kv = ops.linear(h, w["qkv_w"][d:], w["qkv_b"][d:])                            # (B, T, 2d)
+                q0 = ops.linear(h[:, 0], w["qkv_w"][:d], w["qkv_b"][:d])                      # (B, d), rows T*d apart
+                att = ops.attn_fwd(q0.view(B, 1, d), kv[..., :d], kv[..., d:], self.n_heads, n_valid=n_valid)
+                x = ops.linear(att.view(B, d), w["out_w"], w["out_b"], residual=x[:, 0]).view(B, 1, d)
+            else:
+                qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                   # (B, T, 3d)
+                att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
+                x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                       # x + out(att)
             h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)
             fused = h = None
             if dt is not torch.float32 and ops.ffn_fused_profitable(d, self.ffn_dim, dt):

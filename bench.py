@@ -239,11 +239,13 @@ def main():
     # (padding rows included: the reference computes and masks them).  Both are side notes of the roofline object;
     # its fraction is quoted on what the matrix pipe is really issued (below).
     dense_flops = cm.flops_per_env(spec) * B
-    pruned = (route == "fused" and m.prune_final) or route == "blocks"
+    pruned = (route in ("fused", "ops") and m.prune_final) or route == "blocks"
     exec_flops = dense_flops
     if pruned:
         d_, T_, F_ = spec.d, spec.T, spec.ffn
-        saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the 15 unread tokens
+        saved = (T_ - 1) * (d_ * d_ + 2 * d_ * F_)          # out-proj + FFN MACs of the T - 1 unread tokens
+        if route == "ops":
+            saved += (T_ - 1) * (d_ * d_ + 2 * T_ * d_)     # ... and their query projection, scores and weighted sums
         exec_flops = dense_flops - 2 * saved * B
     # ... and, on the fused route, the 16-row tiles the launch really runs: envs of 5..8 tokens go two to a
     # tile, of at most 4 tokens behind an env of 9..12 tokens or four to a tile (same output bits), so the per-tile
@@ -271,8 +273,9 @@ def main():
              "cfg_pair_kernel (tile table) + cfg_forward_kernel, one merged launch (final block pruned to token 0, short envs "
              "share tiles)" if tiles is not None else
              "cfg_embed_kernel + blocks_kernel (final block pruned to token 0) + heads" if route == "blocks" else
-             "cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned else
+             "cfg_forward_kernel HEAD + TAIL launches (final block pruned to token 0)" if pruned and route == "fused" else
              "cfg_forward_kernel FULL (one persistent launch)" if route == "fused" else
+             "launch train (per-op route; final block pruned to token 0)" if pruned else
              "launch train (per-op route)")
     traffic = None
     if tiles is not None and args.config == 1 and B == 16384:

@@ -121,6 +121,34 @@ def test_variants_ops_route(act, final_ln, dtype):
         _check16(lg, v, p, spec, obs, k, dtype, round_residual=True, ceil=ceil, margin=margin)
 
 
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-6), ("f16", 2.5e-3)])
+def test_ops_route_final_block_pruned_to_token0_matches_the_dense_form(dtype, tol):
+    """The per-op route computes only token 0 of the final block (keys / values of every token): exact in exact
+    arithmetic (the reference's n_queries path, python/policy.py:533-539).  fp32: the same numbers to rounding of a
+    different GEMM geometry; fp16: within the stream's own rounding, and against the oracle's pruned form."""
+    spec = cm.ConfigSpec(3, 128, 4, 256, 16, act="gelu", final_ln=True)
+    p, m = _build(spec, 31, dtype, "ops")
+    obs, k = cm.make_inputs(spec, 300, 32, "quarter_empty")
+    assert m.prune_final
+    lg, v = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    m.prune_final = False
+    lg_d, v_d = m.forward_stacked(obs.to(DEV), k.to(DEV))
+    scale = lg_d.abs().max().item()
+    assert (lg - lg_d).abs().max().item() <= tol * max(scale, 1.0), ((lg - lg_d).abs().max().item(), scale)
+    assert (v - v_d).abs().max().item() <= tol * max(v_d.abs().max().item(), 1.0)
+    r_p, rv_p = cm.forward(p, spec, obs, k, prune_final=True)
+    r_d, rv_d = cm.forward(p, spec, obs, k)
+    assert (r_p - r_d).abs().max().item() <= 2e-6 * max(r_d.abs().max().item(), 1.0)      # the oracle's own two forms agree
+    if dtype == "f32":
+        assert bool(((lg.cpu() - r_p).abs() <= 1e-5 * (r_p.abs() + r_p.abs().max())).all())
+    # no mask at all: the same
+    m.prune_final = True
+    lg2, _ = m.forward_stacked(obs.to(DEV), None)
+    m.prune_final = False
+    lg2_d, _ = m.forward_stacked(obs.to(DEV), None)
+    assert (lg2 - lg2_d).abs().max().item() <= tol * max(lg2_d.abs().max().item(), 1.0)
+
+
 def test_masked_slots_cannot_change_outputs_on_gpu():
     c = cm.CONFIGS[1]
     spec = c["spec"]
