@@ -86,6 +86,8 @@ class ConfigPolicy(nn.Module):
         self.prune_final = True
         # fused route, pruned form, key counts given: envs of at most 8 tokens share 16-row tiles in twos, of at most 4 tokens ride behind a 9..12-token env or in fours (same bits)
         self.pack_short = True
+        # per-op route: a block's output projection + LN2 + FFN as one kernel where the shape has one (d = 384)
+        self.fuse_block_tail = True
         self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
                      "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}
 
@@ -127,6 +129,9 @@ class ConfigPolicy(nn.Module):
             # the packed fused FFN's weight image lives with the replicas it was built from (one per weights version)
             w["ffn_img"] = (ops.ffn_pack_into(None, w["w0"], w["b0"], w["w2"], w["b2"])
                             if ops.ffn_pack_supported(self.d, self.ffn_dim, dt) else None)
+            # ... and the image of the one-kernel block tail (output projection + LN2 + FFN) where the shape has one
+            w["tail_img"] = (ops.proj_ffn_pack(w["out_w"], w["out_b"], w["w0"], w["b0"], w["w2"], w["b2"])
+                             if ops.proj_ffn_supported(self.d, self.ffn_dim, dt) else None)
         self._replica = (key, r)
         return r
 
@@ -317,6 +322,15 @@ class ConfigPolicy(nn.Module):
             else:
                 qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                   # (B, T, 3d)
                 att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
+                if w["tail_img"] is not None and self.fuse_block_tail:
+                    # output projection + residual, LN2, FFN (+ the next block's LN1) in one kernel
+                    nxt = self.blocks[i + 1].ln_attn if i + 1 < len(self.blocks) else None
+                    x, h = ops.proj_ffn_fused(att, x, w["tail_img"], self.ffn_dim, blk.ln_ffn.weight.detach(),
+                                              blk.ln_ffn.bias.detach(), blk.ln_ffn.eps, act=self.act,
+                                              ln_w=nxt.weight.detach() if nxt is not None else None,
+                                              ln_b=nxt.bias.detach() if nxt is not None else None,
+                                              eps=nxt.eps if nxt is not None else 1e-5)
+                    continue
                 x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                       # x + out(att)
             h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)
             fused = h = None

@@ -999,6 +999,9 @@ struct FfnArgs {
     const u16* x; const u16* h2; u16* xo; u16* ho; u16* hid;      // hid: (rows, F) activated hidden for a backward, or NULL
     const float* ln_w; const float* ln_b; float eps;
     int64_t rows; int F, total_stages;
+    // the attention-side tail in front of the FFN (PROJ instantiations): h2 is then the attention output, the image
+    // opens with d / 32 output-projection stages, vec continues with the projection bias
+    const float* ln2_w; const float* ln2_b; float eps2;
 };
 
 // Eight waves, one workgroup per CU - or four waves, TWO workgroups per CU (d = 128 / 192, where two rings fit): the
@@ -1010,20 +1013,28 @@ struct FfnArgs {
 template <int D, int NW, int XS = 0> struct FfnRing : StageRing<Geo<D>::SF, (NW == 8 ? (D == 128 ? 10 : D == 192 ? 7 : 6) : (D == 128 ? 8 : D == 192 ? 6 : 5)) + XS, NW> {};
 template <int D, int NW> constexpr int ffn_wgs_per_cu() { return D == 384 ? 1 : 8 / NW; }
 
-template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_, int XS>
+// PROJ (d = 384): the rest of the block's attention side in front of the FFN, in the same registers -
+//   x1 = x + att Wo^T + bo (rounded once),  h2 = LayerNorm(x1; ln2) (rounded once),  then the FFN of (x1, h2) as above -
+// what the output-projection kernel and the LayerNorm kernel between them would do through memory (three round trips
+// of the stream).  The projection runs as d / 32 more stages of the down-projection's form (the attention output's
+// operand fragments in place of the hidden chunk); the rounded x1 and h2 never leave the registers: a lane's four
+// features of an accumulator tile are half of an operand fragment of the up-projection.
+template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_, int XS, bool PROJ = false>
 __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
     typedef FfnRing<D, NW_, XS> R;
+    static_assert(!PROJ || (D == 384 && !SAVE), "the projection form exists for the register-pipelined d = 384 kernel");
     constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
     extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
     float* vlds = reinterpret_cast<float*>(bvl4);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
-    const int nvec = a.F + 3 * D;
+    const int nvec = a.F + (PROJ ? 6 : 3) * D;         // PROJ: ... | bo (d) | ln2_w (d) | ln2_b (d)
     const int ring_off_u4 = (nvec / 4 + 63) & ~63;
     const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
     const float* B1 = vlds; const float* B2 = vlds + a.F; const float* LNG = B2 + D; const float* LNB = LNG + D;
+    const float* BO = LNB + D; const float* LN2G = BO + D; const float* LN2B = LN2G + D;
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
 
     R pipe;
@@ -1041,6 +1052,9 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         pipe.start(ring, a.frags, a.total_stages, wave, lane);
         for (int i = tid; i < a.F + D; i += NW * 64) vlds[i] = a.vec[i];
         if (LN) for (int i = tid; i < D; i += NW * 64) { vlds[a.F + D + i] = a.ln_w[i]; vlds[a.F + 2 * D + i] = a.ln_b[i]; }
+        if (PROJ) for (int i = tid; i < D; i += NW * 64) {
+            vlds[a.F + 3 * D + i] = a.vec[a.F + D + i]; vlds[a.F + 4 * D + i] = a.ln2_w[i]; vlds[a.F + 5 * D + i] = a.ln2_b[i];
+        }
         blk_barrier();
     }
 
@@ -1062,7 +1076,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const float4 b = *reinterpret_cast<const float4*>(B2 + 16 * nt + 4 * g);
+                    const float4 b = *reinterpret_cast<const float4*>((PROJ ? BO : B2) + 16 * nt + 4 * g);
                     x[rt][nt][0] = DT::to_f((u16)(rx[nt].x & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(rx[nt].x >> 16)) + b.y;
                     x[rt][nt][2] = DT::to_f((u16)(rx[nt].y & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(rx[nt].y >> 16)) + b.w;
                     asm("" : "+a"(x[rt][nt]));        // the accumulator lives in accumulation registers from here on
@@ -1160,9 +1174,59 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
             for (int rt = 0; rt < 2; ++rt) acc[ntl][rt] = DT::mfma32(wf, hf[rt][half * KB + ci].v, acc[ntl][rt]);
         };
         advance(Even{});
-        if (PIPE) {      // an odd stage follows W1(0): W1(1), or W2(0) when nch == 1
+        if constexpr (PIPE) {      // an odd stage follows W1(0): W1(1), or W2(0) when nch == 1
 #pragma unroll
             for (int f = 0; f < NBUF - 1; ++f) wr[f] = pipe.frag(f, lane);
+            if constexpr (PROJ) {
+                // KC projection stages (even, odd, ...; KC is even, so W1(0) stays an even stage): stage c adds
+                // Wo[:, 32 c .. 32 c + 31] times the attention output's chunk c into every feature tile
+                static_for<0, KC>([&](auto c_) __attribute__((always_inline)) {
+                    constexpr int c = decltype(c_)::value;
+                    stage((c & 1) ? 2 : 1, [&](auto i_, const s16x8& wo) __attribute__((always_inline)) {
+                        constexpr int i = decltype(i_)::value;
+#pragma unroll
+                        for (int rt = 0; rt < 2; ++rt) x[rt][i] = DT::mfma32(wo, hf[rt][c].v, x[rt][i]);
+                    });
+                });
+                // W1(0) is admitted and its first fragments requested.  x1 rounded as the stream stores it, LayerNorm
+                // on the rounded row (one pass, as the epilogue below), h2 rounded into the operand fragments, and the
+                // FFN's accumulator x1 + b2
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    float s1 = 0.f, q1 = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const uint32_t lo = bpack2<DT>(x[rt][nt][0], x[rt][nt][1]), hi = bpack2<DT>(x[rt][nt][2], x[rt][nt][3]);
+                        f32x4 r;
+                        r[0] = DT::to_f((u16)(lo & 0xffff)); r[1] = DT::to_f((u16)(lo >> 16));
+                        r[2] = DT::to_f((u16)(hi & 0xffff)); r[3] = DT::to_f((u16)(hi >> 16));
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { s1 += r[i]; q1 = fmaf(r[i], r[i], q1); }
+                        asm("" : "+a"(r));
+                        x[rt][nt] = r;
+                        if ((nt & 3) == 3) __builtin_amdgcn_sched_barrier(0);      // keeps the accumulator's trips through the vector registers short
+                    }
+                    rows_reduce2(s1, q1, OpAdd());
+                    const float mean = s1 * (1.0f / D);
+                    const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q1 * (1.0f / D)), 0.f) + a.eps2);
+                    const float shift = -mean * rstd;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const float4 gm = *reinterpret_cast<const float4*>(LN2G + 16 * nt + 4 * g);
+                        const float4 bt = *reinterpret_cast<const float4*>(LN2B + 16 * nt + 4 * g);
+                        const float4 b2 = *reinterpret_cast<const float4*>(B2 + 16 * nt + 4 * g);
+                        f32x4 r = x[rt][nt];
+                        uint2 v;
+                        v.x = bpack2<DT>(fmaf(fmaf(r[0], rstd, shift), gm.x, bt.x), fmaf(fmaf(r[1], rstd, shift), gm.y, bt.y));
+                        v.y = bpack2<DT>(fmaf(fmaf(r[2], rstd, shift), gm.z, bt.z), fmaf(fmaf(r[3], rstd, shift), gm.w, bt.w));
+                        hf[rt][nt >> 1].h[nt & 1] = v;
+                        r[0] += b2.x; r[1] += b2.y; r[2] += b2.z; r[3] += b2.w;
+                        asm("" : "+a"(r));
+                        x[rt][nt] = r;
+                        if ((nt & 1) == 1) __builtin_amdgcn_sched_barrier(0);      // (the scheduler would hoist every vector read above the first use)
+                    }
+                }
+            }
             up_init(0); stage(1, up_mm);
         }
         else up(0);
@@ -1190,7 +1254,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 }
             }
             // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
-            if (PIPE) {
+            if constexpr (PIPE) {
                 // the stage in the ring and its first NBUF - 1 fragments were requested by the stage before
                 if (ch + 1 < nch) { up_init(ch + 1); stage(2, up_mm); }                  // W1(ch + 1), then W2(ch): even
                 stage(ch + 1 < nch ? 1 : 0, [&](auto i_, const s16x8& w2) __attribute__((always_inline)) {   // W2(ch); an odd stage follows but the last
@@ -1297,8 +1361,8 @@ bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
     return 2 * (F / 32) >= slots;
 }
 int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
-template <int D, int NW, int XS> size_t ffn_dyn_bytes(int F) {
-    return (size_t)(((F + 3 * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW, XS>::SLOTS * FfnRing<D, NW, XS>::STAGE_BYTES;
+template <int D, int NW, int XS> size_t ffn_dyn_bytes(int F, bool proj = false) {
+    return (size_t)(((F + (proj ? 6 : 3) * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW, XS>::SLOTS * FfnRing<D, NW, XS>::STAGE_BYTES;
 }
 template <typename DT, int D, int ACT, int NW, int XS = 0>
 int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
@@ -1336,7 +1400,107 @@ int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
     return BSRL_UNSUPPORTED;
 }
 
+// the projection form (d = 384): six ring slots where the longer vector block leaves room, else five
+template <typename DT, int ACT, int XS>
+int proj_ffn_launch_xs(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
+    constexpr int D = 384, NW = 4;
+    const size_t dyn = ffn_dyn_bytes<D, NW, XS>(a.F, true);
+    if (dyn + 1024 > (size_t)LDS_BUDGET || a.total_stages < FfnRing<D, NW, XS>::SLOTS) return BSRL_UNSUPPORTED;
+    const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
+    const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));
+    auto launch = [&](auto kern) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess)
+            return (int)BSRL_UNSUPPORTED;
+        hipLaunchKernelGGL(kern, grid, dim3(NW * 64), dyn, st, a);
+        return (int)BSRL_OK;
+    };
+    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW, XS, true>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW, XS, true>);
+}
+template <typename DT, int ACT>
+int proj_ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
+    const int rc = proj_ffn_launch_xs<DT, ACT, 1>(a, ln, cus, st);
+    return rc != BSRL_UNSUPPORTED ? rc : proj_ffn_launch_xs<DT, ACT, 0>(a, ln, cus, st);
+}
+
+struct ProjPackArgs { const u16* wo; const float* bo; void* frags; float* vec_bo; };
+// the d / 32 output-projection stages in front of the FFN stages: stage c, fragment i = rows [16 i, +16) of Wo, columns
+// [32 c, +32) in the operand order of a hidden chunk (the form of a W2 stage); one wave per fragment
+template <int D>
+__global__ __launch_bounds__(256) void proj_pack_frags_kernel(ProjPackArgs a) {
+    constexpr int SF = Geo<D>::SF, KC = Geo<D>::KC;
+    const int lane = threadIdx.x & 63, n16 = lane & 15, gg = lane >> 4;
+    const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= KC * SF) return;
+    const int c = f / SF, i = f % SF;
+    u16 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = a.wo[(int64_t)(16 * i + n16) * D + 32 * c + bperm_k(0, gg, j)];
+    uint4 o;
+    o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+    o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+    static_cast<uint4*>(a.frags)[(int64_t)f * 64 + lane] = o;
+    if (f == 0) for (int k = lane; k < D; k += 64) a.vec_bo[k] = a.bo[k];
+}
+bool proj_ffn_shape_ok(int64_t d, int64_t F, int dtype) { return d == 384 && ffn_packed_shape_ok(d, F, dtype); }
+int64_t proj_frag_bytes(int64_t d) { return (d / 32) * (d / 16) * 1024; }
+
 }  // namespace
+
+extern "C" int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int dtype) {
+    if (!proj_ffn_shape_ok(d, F, dtype)) return 0;
+    return proj_frag_bytes(d) + ffn_frag_bytes(d, F) + (F + 2 * d) * 4;
+}
+
+extern "C" int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w0, const float* b0, const void* w2,
+                                  const float* b2, int64_t d, int64_t F, int dtype, void* image, bsrl_stream stream) {
+    if (!wo || !bo || !w0 || !b0 || !w2 || !b2 || !image) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_pack: null pointer");
+    if (!proj_ffn_shape_ok(d, F, dtype)) return BSRL_UNSUPPORTED;
+    if (!bsrl_aligned(image, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_pack: image must be 16-byte aligned");
+    char* img = static_cast<char*>(image);
+    char* ffn_frags = img + proj_frag_bytes(d);
+    float* vec = reinterpret_cast<float*>(ffn_frags + ffn_frag_bytes(d, F));          // b0 (F) | b2 (d) | bo (d)
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ProjPackArgs pp{static_cast<const u16*>(wo), bo, image, vec + F + d};
+    const int64_t npf = (d / 32) * (d / 16);
+    hipLaunchKernelGGL(proj_pack_frags_kernel<384>, dim3((unsigned)((npf + 3) / 4)), dim3(256), 0, st, pp);
+    FfnPackArgs pa{static_cast<const u16*>(w0), b0, static_cast<const u16*>(w2), b2, ffn_frags, vec, (int)F};
+    const int64_t nfrags = 2 * (F / 32) * (d / 16);
+    hipLaunchKernelGGL(ffn_pack_frags_kernel<384>, dim3((unsigned)((nfrags + 3) / 4)), dim3(256), 0, st, pa);
+    BSRL_CHECK_LAUNCH("bsrl_proj_ffn_pack");
+    return BSRL_OK;
+}
+
+extern "C" int bsrl_proj_ffn_packed(const void* image, const void* att, const void* x, const float* ln2_w, const float* ln2_b,
+                                    float eps2, const float* ln_w, const float* ln_b, float eps, void* xo, void* ho,
+                                    int64_t rows, int64_t d, int64_t F, int act, int dtype, bsrl_stream stream) {
+    if (!image || !att || !x || !xo || !ln2_w || !ln2_b) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: null pointer");
+    if ((ln_w == nullptr) != (ho == nullptr) || (ln_w == nullptr) != (ln_b == nullptr))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: ln_w, ln_b and ho go together");
+    if (!proj_ffn_shape_ok(d, F, dtype) || (act != BSRL_ACT_RELU && act != BSRL_ACT_GELU)) return BSRL_UNSUPPORTED;
+    if (rows < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: rows < 0");
+    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(att, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: image must be 16-byte, rows 8-byte aligned");
+    if (rows == 0) return BSRL_OK;
+    FfnArgs a;
+    a.frags = static_cast<const uint2*>(image);
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + proj_frag_bytes(d) + ffn_frag_bytes(d, F));
+    a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(att);
+    a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho); a.hid = nullptr;
+    a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F;
+    a.total_stages = (int)(d / 32 + 2 * (F / 32));
+    a.ln2_w = ln2_w; a.ln2_b = ln2_b; a.eps2 = eps2;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    const bool relu = act == BSRL_ACT_RELU, ln = ln_w != nullptr;
+    int rc;
+    if (dtype == BSRL_F16) rc = relu ? proj_ffn_launch<F16, BSRL_ACT_RELU>(a, ln, cus, st) : proj_ffn_launch<F16, BSRL_ACT_GELU>(a, ln, cus, st);
+    else rc = relu ? proj_ffn_launch<BF16, BSRL_ACT_RELU>(a, ln, cus, st) : proj_ffn_launch<BF16, BSRL_ACT_GELU>(a, ln, cus, st);
+    if (rc != BSRL_OK) return rc;
+    BSRL_CHECK_LAUNCH("bsrl_proj_ffn_packed");
+    return BSRL_OK;
+}
 
 extern "C" int64_t bsrl_ffn_pack_size(int64_t d, int64_t F, int dtype) {
     if (!ffn_packed_shape_ok(d, F, dtype)) return 0;
@@ -1379,6 +1543,7 @@ extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2,
     a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(h2);
     a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho); a.hid = static_cast<u16*>(hid);
     a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F; a.total_stages = (int)(2 * (F / 32));
+    a.ln2_w = a.ln2_b = nullptr; a.eps2 = 0.f;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||

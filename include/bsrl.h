@@ -165,6 +165,24 @@ int bsrl_ffn_pack(const void* w0, const float* b0, const void* w2, const float* 
 int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const float* ln_w,
                     const float* ln_b, float eps, void* xo, void* ho, void* hid, int64_t rows,
                     int64_t d, int64_t F, int act, int dtype, bsrl_stream stream);
+/* The tail of a block from the attention output on, in one kernel (d = 384, where the per-op route
+ * runs the block as separate launches):
+ *   x1 = x + att Wo^T + bo            Block.forward's output projection + residual (python/policy.py:650-662)
+ *   h2 = LayerNorm(x1; ln2_w, ln2_b)  its ln_ffn (python/policy.py:663-672, layer_norm.cu:14-21)
+ *   xo = x1 + act(h2 W0^T + b0) W2^T + b2,  ho = LayerNorm(xo; ln_w, ln_b) if ln_w   (bsrl_ffn_packed)
+ * with the rounding points of the separate launches (x1, h2, hidden, xo, ho rounded once each; fp32
+ * accumulation and statistics), x1 and h2 never leaving the registers.  bsrl_proj_ffn_pack writes
+ * the image (bsrl_proj_ffn_pack_size bytes, 16-byte aligned; 0 = unsupported shape) from wo (d, d),
+ * w0 (F, d), w2 (d, F) in `dtype` and the fp32 biases.  att, x, xo, ho (rows, d) contiguous in
+ * `dtype`, 8-byte aligned; ln2_w / ln2_b required, ln_w / ln_b / ho together or all NULL. */
+int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int dtype);
+int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w0, const float* b0,
+                       const void* w2, const float* b2, int64_t d, int64_t F, int dtype,
+                       void* image, bsrl_stream stream);
+int bsrl_proj_ffn_packed(const void* image, const void* att, const void* x, const float* ln2_w,
+                         const float* ln2_b, float eps2, const float* ln_w, const float* ln_b,
+                         float eps, void* xo, void* ho, int64_t rows, int64_t d, int64_t F,
+                         int act, int dtype, bsrl_stream stream);
 
 /* ---- Config-model tokenizer -----------------------------------------------
  * The benchmark configs' "linear embedding": token 0 = Wp obs[:, :prop_dim] +

@@ -287,6 +287,55 @@ def test_ffn_fused_packed_image_follows_the_weights_and_large_row_counts():
     assert (a2.float() - ref2.float()).abs().max().item() <= 2 * EPS16[torch.float16] * scale
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,Fh", [(1, 1536), (77, 1536), (1000, 1536), (300, 192), (33000, 768)])
+@pytest.mark.parametrize("act,with_ln", [("relu", True), ("gelu", False), ("gelu", True)])
+def test_block_tail_in_one_kernel(dtype, rows, Fh, act, with_ln):
+    """Output projection + residual, LN2, FFN (+ next LN) as one kernel at d = 384: closed form with the rounding points
+    of the separate launches (x1, h2, hidden, xo, ho rounded once each; the reference's Block.forward,
+    python/policy.py:650-715, and its fused FFN test's idiom, python/tests/test_fused_ffn.py:252-306), and the error
+    class of the separate launches of this library on the same operands."""
+    d = 384
+    assert ops.proj_ffn_supported(d, Fh, dtype) and not ops.proj_ffn_supported(256, 1024, dtype)
+    x = _rand(rows, d, dtype=dtype, seed=1)
+    att = _rand(rows, d, dtype=dtype, seed=2)
+    wo = _rand(d, d, dtype=dtype, seed=9, scale=1 / math.sqrt(d))
+    w0 = _rand(Fh, d, dtype=dtype, seed=3, scale=1 / math.sqrt(d))
+    w2 = _rand(d, Fh, dtype=dtype, seed=4, scale=1 / math.sqrt(Fh))
+    bo, b0, b2 = _rand(d, seed=10) * 0.3, _rand(Fh, seed=5) * 0.3, _rand(d, seed=6) * 0.3
+    l2w, l2b = _rand(d, seed=11) * 0.2 + 1.0, _rand(d, seed=12) * 0.2
+    lw, lb = (_rand(d, seed=7) * 0.2 + 1.0, _rand(d, seed=8) * 0.2) if with_ln else (None, None)
+    img = ops.proj_ffn_pack(wo, bo, w0, b0, w2, b2)
+    xo, ho = ops.proj_ffn_fused(att, x, img, Fh, l2w, l2b, 1e-5, act=act, ln_w=lw, ln_b=lb)
+    # the separate launches
+    x1_u = ops.linear(att, wo, bo, residual=x)
+    h2_u = ops.ln_fwd(x1_u, l2w, l2b, 1e-5)
+    xo_u, ho_u = ops.ffn_fused(x1_u, h2_u, w0, b0, w2, b2, act=act, ln_w=lw, ln_b=lb)
+    # closed form in double with the same rounding points
+    x1 = (x.double() + att.double() @ wo.double().t() + bo.double()).to(dtype)
+    h2 = F.layer_norm(x1.double(), (d,), l2w.double(), l2b.double(), 1e-5).to(dtype)
+    pre = h2.double() @ w0.double().t() + b0.double()
+    hid = (torch.relu(pre) if act == "relu" else 0.5 * pre * (1 + torch.erf(pre / math.sqrt(2.0)))).to(dtype).double()
+    ref = x1.double() + hid @ w2.double().t() + b2.double()
+    scale = ref.abs().max().item()
+    e_new = (xo.double() - ref).norm() / ref.norm()
+    e_old = (xo_u.double() - ref).norm() / ref.norm()
+    # a one-ulp flip of x1 or h2 near a tie moves a whole row a little: the bound is on the error CLASS, and loosely on the maximum
+    assert e_new <= max(1.15 * e_old, 1e-3), (e_new.item(), e_old.item())
+    assert (xo.double() - ref).abs().max().item() <= 4 * EPS16[dtype] * scale
+    assert (xo.float() - xo_u.float()).abs().max().item() <= 4 * EPS16[dtype] * scale
+    if with_ln:
+        ln_ref = F.layer_norm(xo.float(), (d,), lw, lb, 1e-5)
+        assert (ho.float() - ln_ref).abs().max().item() <= 2 * EPS16[dtype] * (ln_ref.abs().max().item() + 1)
+    else:
+        assert ho is None
+    # a row's bits do not depend on the batch it sits in
+    if rows >= 300:
+        lo, hi = 130, 290
+        a, b = ops.proj_ffn_fused(att[lo:hi].contiguous(), x[lo:hi].contiguous(), img, Fh, l2w, l2b, 1e-5, act=act, ln_w=lw, ln_b=lb)
+        assert torch.equal(a, xo[lo:hi]) and (b is None or torch.equal(b, ho[lo:hi]))
+
+
 def test_ffn_fused_unsupported_shapes_say_so():
     assert not ops.ffn_fused_supported(160, 640, torch.float16)
     assert not ops.ffn_fused_supported(128, 500, torch.float16)
