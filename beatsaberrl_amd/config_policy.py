@@ -86,8 +86,10 @@ class ConfigPolicy(nn.Module):
         self.prune_final = True
         # fused route, pruned form, key counts given: envs of at most 8 tokens share 16-row tiles in twos, of at most 4 tokens ride behind a 9..12-token env or in fours (same bits)
         self.pack_short = True
-        # per-op route: a block's output projection + LN2 + FFN as one kernel where the shape has one (d = 384)
+        # per-op route: a block's output projection + LN2 + FFN as one kernel where the shape has one (d = 384), and the
+        # next block's LN1 + packed q|k|v projection behind it in the same launch
         self.fuse_block_tail = True
+        self.fuse_next_proj = True
         self.arch = {"n_layers": n_layers, "d": d, "n_heads": n_heads, "ffn": ffn, "T": T, "n_gears": n_gears,
                      "act": act, "final_ln": bool(final_ln), "prop_dim": prop_dim, "obj_dim": obj_dim}
 
@@ -129,9 +131,9 @@ class ConfigPolicy(nn.Module):
             # the packed fused FFN's weight image lives with the replicas it was built from (one per weights version)
             w["ffn_img"] = (ops.ffn_pack_into(None, w["w0"], w["b0"], w["w2"], w["b2"])
                             if ops.ffn_pack_supported(self.d, self.ffn_dim, dt) else None)
-            # ... and the image of the one-kernel block tail (output projection + LN2 + FFN) where the shape has one
-            w["tail_img"] = (ops.proj_ffn_pack(w["out_w"], w["out_b"], w["w0"], w["b0"], w["w2"], w["b2"])
-                             if ops.proj_ffn_supported(self.d, self.ffn_dim, dt) else None)
+            # ... and the images of the one-kernel block tail (output projection + LN2 + FFN + the next block's
+            # projection), built on first use per width of that projection
+            w["tail_img"] = {}
         self._replica = (key, r)
         return r
 
@@ -307,29 +309,48 @@ class ConfigPolicy(nn.Module):
         if obs.dtype not in (torch.float32, dt):
             obs = obs.float()
         x = self._tokens(obs, r, dt)                                                          # (B, T, d)
-        h = None                                                # LN1 of the block, when the previous block's FFN kernel wrote it
+        h = None                # LN1 of the block, when the previous block's kernel wrote it
+        proj = None             # the block's packed projection of h (q|k|v, or k|v for the pruned final block), likewise
+        L = len(self.blocks)
         for i, (blk, w) in enumerate(zip(self.blocks, r["blk"])):
-            if h is None:
-                h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
-            if self.prune_final and i + 1 == len(self.blocks):
+            pruned = self.prune_final and i + 1 == L
+            if proj is None:
+                if h is None:
+                    h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
+                # Row slices of the packed q|k|v weight are contiguous views: keys and values only for a pruned block
+                proj = ops.linear(h, w["qkv_w"][d:], w["qkv_b"][d:]) if pruned else ops.linear(h, w["qkv_w"], w["qkv_b"])
+            if pruned:
                 # Only token 0 of the final block is read (the reference's n_queries path, python/policy.py:533-539:
                 # exact, masking is key-side only): keys and values of every token, the query, the output projection,
-                # LN2 and the FFN of token 0 alone.  Row slices of the packed q|k|v weight are contiguous views.
-                kv = ops.linear(h, w["qkv_w"][d:], w["qkv_b"][d:])                            # (B, T, 2d)
+                # LN2 and the FFN of token 0 alone.
                 q0 = ops.linear(h[:, 0], w["qkv_w"][:d], w["qkv_b"][:d])                      # (B, d), rows T*d apart
-                att = ops.attn_fwd(q0.view(B, 1, d), kv[..., :d], kv[..., d:], self.n_heads, n_valid=n_valid)
+                att = ops.attn_fwd(q0.view(B, 1, d), proj[..., :d], proj[..., d:], self.n_heads, n_valid=n_valid)
                 x = ops.linear(att.view(B, d), w["out_w"], w["out_b"], residual=x[:, 0]).view(B, 1, d)
+                proj = None
             else:
-                qkv = ops.linear(h, w["qkv_w"], w["qkv_b"])                                   # (B, T, 3d)
-                att = ops.attn_fwd(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], self.n_heads, n_valid=n_valid)
-                if w["tail_img"] is not None and self.fuse_block_tail:
-                    # output projection + residual, LN2, FFN (+ the next block's LN1) in one kernel
-                    nxt = self.blocks[i + 1].ln_attn if i + 1 < len(self.blocks) else None
-                    x, h = ops.proj_ffn_fused(att, x, w["tail_img"], self.ffn_dim, blk.ln_ffn.weight.detach(),
-                                              blk.ln_ffn.bias.detach(), blk.ln_ffn.eps, act=self.act,
-                                              ln_w=nxt.weight.detach() if nxt is not None else None,
-                                              ln_b=nxt.bias.detach() if nxt is not None else None,
-                                              eps=nxt.eps if nxt is not None else 1e-5)
+                att = ops.attn_fwd(proj[..., :d], proj[..., d:2 * d], proj[..., 2 * d:], self.n_heads, n_valid=n_valid)
+                proj = None
+                if self.fuse_block_tail and ops.proj_ffn_supported(d, self.ffn_dim, dt):
+                    # output projection + residual, LN2, FFN, the next block's LN1 and its packed projection in one
+                    # kernel (k|v only, and LN1 written for the query row, when that block is the pruned final one)
+                    nblk = self.blocks[i + 1] if i + 1 < L else None
+                    nxt_pruned = self.prune_final and i + 2 == L
+                    lo = d if nxt_pruned else 0
+                    n_next = (3 * d - lo) if nblk is not None and self.fuse_next_proj else 0
+                    img = w["tail_img"].get(n_next)
+                    if img is None:
+                        wn = r["blk"][i + 1] if n_next else None
+                        img = w["tail_img"][n_next] = ops.proj_ffn_pack(
+                            w["out_w"], w["out_b"], w["w0"], w["b0"], w["w2"], w["b2"],
+                            wn["qkv_w"][lo:] if wn else None, wn["qkv_b"][lo:] if wn else None)
+                    res = ops.proj_ffn_fused(att, x, img, self.ffn_dim, blk.ln_ffn.weight.detach(), blk.ln_ffn.bias.detach(),
+                                             blk.ln_ffn.eps, act=self.act,
+                                             ln_w=nblk.ln_attn.weight.detach() if nblk is not None else None,
+                                             ln_b=nblk.ln_attn.bias.detach() if nblk is not None else None,
+                                             eps=nblk.ln_attn.eps if nblk is not None else 1e-5, n_next=n_next,
+                                             want_ho=nxt_pruned or n_next == 0)
+                    x, h = res[0], res[1]
+                    proj = res[2] if n_next else None
                     continue
                 x = ops.linear(att, w["out_w"], w["out_b"], residual=x)                       # x + out(att)
             h2 = ops.ln_fwd(x, blk.ln_ffn.weight, blk.ln_ffn.bias, blk.ln_ffn.eps)

@@ -1002,6 +1002,10 @@ struct FfnArgs {
     // the attention-side tail in front of the FFN (PROJ instantiations): h2 is then the attention output, the image
     // opens with d / 32 output-projection stages, vec continues with the projection bias
     const float* ln2_w; const float* ln2_b; float eps2;
+    // ... and a projection of the LayerNorm-ed output behind it (PROJ, with LN): qo (rows, 32 * nq) = ho Wn^T + bn, as nq
+    // more stages of the up-projection's form after the FFN stages (vec continues with bn); ho itself is stored only
+    // when the pointer is given
+    u16* qo; int nq;
 };
 
 // Eight waves, one workgroup per CU - or four waves, TWO workgroups per CU (d = 128 / 192, where two rings fit): the
@@ -1030,11 +1034,11 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g = lane >> 4;
-    const int nvec = a.F + (PROJ ? 6 : 3) * D;         // PROJ: ... | bo (d) | ln2_w (d) | ln2_b (d)
+    const int nvec = a.F + (PROJ ? 6 * D + 32 * a.nq : 3 * D);         // PROJ: ... | bo (d) | ln2_w (d) | ln2_b (d) | bn (32 nq)
     const int ring_off_u4 = (nvec / 4 + 63) & ~63;
     const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
     const float* B1 = vlds; const float* B2 = vlds + a.F; const float* LNG = B2 + D; const float* LNB = LNG + D;
-    const float* BO = LNB + D; const float* LN2G = BO + D; const float* LN2B = LN2G + D;
+    const float* BO = LNB + D; const float* LN2G = BO + D; const float* LN2B = LN2G + D; const float* BN = LN2B + D;
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
 
     R pipe;
@@ -1055,6 +1059,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         if (PROJ) for (int i = tid; i < D; i += NW * 64) {
             vlds[a.F + 3 * D + i] = a.vec[a.F + D + i]; vlds[a.F + 4 * D + i] = a.ln2_w[i]; vlds[a.F + 5 * D + i] = a.ln2_b[i];
         }
+        if (PROJ) for (int i = tid; i < 32 * a.nq; i += NW * 64) vlds[a.F + 6 * D + i] = a.vec[a.F + 2 * D + i];
         blk_barrier();
     }
 
@@ -1161,13 +1166,14 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
-        auto up_init = [&](int ch) __attribute__((always_inline)) {
+        auto acc_init = [&](const float* bias, int ch) __attribute__((always_inline)) {
 #pragma unroll
             for (int ntl = 0; ntl < 2; ++ntl) {
-                const float4 b = *reinterpret_cast<const float4*>(B1 + 32 * ch + 16 * ntl + 4 * g);
+                const float4 b = *reinterpret_cast<const float4*>(bias + 32 * ch + 16 * ntl + 4 * g);
                 acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
             }
         };
+        auto up_init = [&](int ch) __attribute__((always_inline)) { acc_init(B1, ch); };
         auto up_mm = [&](auto i_, const s16x8& wf) __attribute__((always_inline)) {
             constexpr int j = decltype(i_)::value / KB, ci = decltype(i_)::value % KB, half = j / 2, ntl = j % 2;
 #pragma unroll
@@ -1257,7 +1263,8 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
             if constexpr (PIPE) {
                 // the stage in the ring and its first NBUF - 1 fragments were requested by the stage before
                 if (ch + 1 < nch) { up_init(ch + 1); stage(2, up_mm); }                  // W1(ch + 1), then W2(ch): even
-                stage(ch + 1 < nch ? 1 : 0, [&](auto i_, const s16x8& w2) __attribute__((always_inline)) {   // W2(ch); an odd stage follows but the last
+                // W2(ch); an odd stage follows but the last, which ends the tile or (PROJ with a projection behind) is followed by an even one
+                stage(ch + 1 < nch ? 1 : (PROJ && a.nq > 0) ? 2 : 0, [&](auto i_, const s16x8& w2) __attribute__((always_inline)) {
                     constexpr int i = decltype(i_)::value;       // feature tile i
 #pragma unroll
                     for (int rt = 0; rt < 2; ++rt) x[rt][i] = DT::mfma32(w2, hid[rt].v, x[rt][i]);
@@ -1313,8 +1320,33 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                     uint2 v;
                     v.x = bpack2<DT>(fmaf(fmaf(x[rt][nt][0], rstd, shift), gm.x, bt.x), fmaf(fmaf(x[rt][nt][1], rstd, shift), gm.y, bt.y));
                     v.y = bpack2<DT>(fmaf(fmaf(x[rt][nt][2], rstd, shift), gm.z, bt.z), fmaf(fmaf(x[rt][nt][3], rstd, shift), gm.w, bt.w));
-                    if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                    if (row < a.rows && (!PROJ || a.ho)) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                    if constexpr (PROJ) hf[rt][nt >> 1].h[nt & 1] = v;       // operand fragments of the projection behind
                 }
+            }
+        }
+        if constexpr (PROJ && LN) {
+            // qo = ho Wn^T + bn: nq stages of 32 output columns in the up-projection's form (the first is admitted and its
+            // first fragments are in flight), each stored as it completes - a lane's four columns of a tile, 8 bytes
+            const int ldq = 32 * a.nq;
+            auto q_store = [&](int sq) __attribute__((always_inline)) {
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    const int64_t row = row0 + 16 * rt + r16;
+                    if (row < a.rows) {
+                        u16* qr = a.qo + row * ldq + 32 * sq + 4 * g;
+#pragma unroll
+                        for (int ntl = 0; ntl < 2; ++ntl) {
+                            uint2 v;
+                            v.x = bpack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]); v.y = bpack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
+                            *reinterpret_cast<uint2*>(qr + 16 * ntl) = v;
+                        }
+                    }
+                }
+            };
+            for (int sq = 0; sq < a.nq; sq += 2) {       // nq is even: an even stage, then an odd one
+                acc_init(BN, sq); stage(1, up_mm); q_store(sq);
+                acc_init(BN, sq + 1); stage(sq + 2 < a.nq ? 2 : 0, up_mm); q_store(sq + 1);
             }
         }
     }
@@ -1361,8 +1393,8 @@ bool ffn_packed_shape_ok(int64_t d, int64_t F, int dtype) {
     return 2 * (F / 32) >= slots;
 }
 int64_t ffn_frag_bytes(int64_t d, int64_t F) { return 2 * (F / 32) * (d / 16) * 1024; }
-template <int D, int NW, int XS> size_t ffn_dyn_bytes(int F, bool proj = false) {
-    return (size_t)(((F + (proj ? 6 : 3) * D) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW, XS>::SLOTS * FfnRing<D, NW, XS>::STAGE_BYTES;
+template <int D, int NW, int XS> size_t ffn_dyn_bytes(int F, bool proj = false, int nq = 0) {
+    return (size_t)(((F + (proj ? 6 * D + 32 * nq : 3 * D)) / 4 + 63) & ~63) * 16 + (size_t)FfnRing<D, NW, XS>::SLOTS * FfnRing<D, NW, XS>::STAGE_BYTES;
 }
 template <typename DT, int D, int ACT, int NW, int XS = 0>
 int ffn_launch_nw(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
@@ -1404,7 +1436,7 @@ int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
 template <typename DT, int ACT, int XS>
 int proj_ffn_launch_xs(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
     constexpr int D = 384, NW = 4;
-    const size_t dyn = ffn_dyn_bytes<D, NW, XS>(a.F, true);
+    const size_t dyn = ffn_dyn_bytes<D, NW, XS>(a.F, true, a.nq);
     if (dyn + 1024 > (size_t)LDS_BUDGET || a.total_stages < FfnRing<D, NW, XS>::SLOTS) return BSRL_UNSUPPORTED;
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
     const dim3 grid((unsigned)(ntiles < cus ? ntiles : cus));
@@ -1422,7 +1454,7 @@ int proj_ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
     return rc != BSRL_UNSUPPORTED ? rc : proj_ffn_launch_xs<DT, ACT, 0>(a, ln, cus, st);
 }
 
-struct ProjPackArgs { const u16* wo; const float* bo; void* frags; float* vec_bo; };
+struct ProjPackArgs { const u16* wo; const float* bo; void* frags; float* vec_bo; const u16* wn; const float* bn; void* nfrags; int nq; };
 // the d / 32 output-projection stages in front of the FFN stages: stage c, fragment i = rows [16 i, +16) of Wo, columns
 // [32 c, +32) in the operand order of a hidden chunk (the form of a W2 stage); one wave per fragment
 template <int D>
@@ -1441,28 +1473,56 @@ __global__ __launch_bounds__(256) void proj_pack_frags_kernel(ProjPackArgs a) {
     static_cast<uint4*>(a.frags)[(int64_t)f * 64 + lane] = o;
     if (f == 0) for (int k = lane; k < D; k += 64) a.vec_bo[k] = a.bo[k];
 }
-bool proj_ffn_shape_ok(int64_t d, int64_t F, int dtype) { return d == 384 && ffn_packed_shape_ok(d, F, dtype); }
+// the nq stages of the projection behind the FFN: stage s = rows [32 s, +32) of Wn in the form of a W1 stage
+template <int D>
+__global__ __launch_bounds__(256) void next_pack_frags_kernel(ProjPackArgs a) {
+    typedef Geo<D> G;
+    constexpr int SF = G::SF;
+    const int lane = threadIdx.x & 63, n16 = lane & 15, gg = lane >> 4;
+    const int f = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (f >= a.nq * SF) return;
+    const int sq = f / SF, i = f % SF;
+    const int burst = i / G::FB, rem = i % G::FB, ntl = rem / G::KB, c = burst * G::KB + rem % G::KB;
+    u16 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = a.wn[(int64_t)(32 * sq + 16 * ntl + n16) * D + bperm_k(c, gg, j)];
+    uint4 o;
+    o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+    o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+    static_cast<uint4*>(a.nfrags)[(int64_t)f * 64 + lane] = o;
+    if (f == 0) for (int k = lane; k < 32 * a.nq; k += 64) a.vec_bo[D + k] = a.bn[k];
+}
+bool proj_ffn_shape_ok(int64_t d, int64_t F, int64_t n_next, int dtype) {
+    return d == 384 && ffn_packed_shape_ok(d, F, dtype) && n_next >= 0 && n_next % 64 == 0 && n_next <= 3 * d;
+}
 int64_t proj_frag_bytes(int64_t d) { return (d / 32) * (d / 16) * 1024; }
 
 }  // namespace
 
-extern "C" int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int dtype) {
-    if (!proj_ffn_shape_ok(d, F, dtype)) return 0;
-    return proj_frag_bytes(d) + ffn_frag_bytes(d, F) + (F + 2 * d) * 4;
+extern "C" int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int64_t n_next, int dtype) {
+    if (!proj_ffn_shape_ok(d, F, n_next, dtype)) return 0;
+    return proj_frag_bytes(d) + ffn_frag_bytes(d, F) + (n_next / 32) * (d / 16) * 1024 + (F + 2 * d + n_next) * 4;
 }
 
 extern "C" int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w0, const float* b0, const void* w2,
-                                  const float* b2, int64_t d, int64_t F, int dtype, void* image, bsrl_stream stream) {
+                                  const float* b2, const void* wn, const float* bn, int64_t n_next, int64_t d, int64_t F,
+                                  int dtype, void* image, bsrl_stream stream) {
     if (!wo || !bo || !w0 || !b0 || !w2 || !b2 || !image) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_pack: null pointer");
-    if (!proj_ffn_shape_ok(d, F, dtype)) return BSRL_UNSUPPORTED;
+    if (!proj_ffn_shape_ok(d, F, n_next, dtype)) return BSRL_UNSUPPORTED;
+    if (n_next > 0 && (!wn || !bn)) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_pack: n_next > 0 needs wn and bn");
     if (!bsrl_aligned(image, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_pack: image must be 16-byte aligned");
     char* img = static_cast<char*>(image);
     char* ffn_frags = img + proj_frag_bytes(d);
-    float* vec = reinterpret_cast<float*>(ffn_frags + ffn_frag_bytes(d, F));          // b0 (F) | b2 (d) | bo (d)
+    char* next_frags = ffn_frags + ffn_frag_bytes(d, F);
+    float* vec = reinterpret_cast<float*>(next_frags + (n_next / 32) * (d / 16) * 1024);      // b0 (F) | b2 (d) | bo (d) | bn (n_next)
     hipStream_t st = static_cast<hipStream_t>(stream);
-    ProjPackArgs pp{static_cast<const u16*>(wo), bo, image, vec + F + d};
+    ProjPackArgs pp{static_cast<const u16*>(wo), bo, image, vec + F + d, static_cast<const u16*>(wn), bn, next_frags, (int)(n_next / 32)};
     const int64_t npf = (d / 32) * (d / 16);
     hipLaunchKernelGGL(proj_pack_frags_kernel<384>, dim3((unsigned)((npf + 3) / 4)), dim3(256), 0, st, pp);
+    if (n_next > 0) {
+        const int64_t nnf = (n_next / 32) * (d / 16);
+        hipLaunchKernelGGL(next_pack_frags_kernel<384>, dim3((unsigned)((nnf + 3) / 4)), dim3(256), 0, st, pp);
+    }
     FfnPackArgs pa{static_cast<const u16*>(w0), b0, static_cast<const u16*>(w2), b2, ffn_frags, vec, (int)F};
     const int64_t nfrags = 2 * (F / 32) * (d / 16);
     hipLaunchKernelGGL(ffn_pack_frags_kernel<384>, dim3((unsigned)((nfrags + 3) / 4)), dim3(256), 0, st, pa);
@@ -1472,23 +1532,30 @@ extern "C" int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w
 
 extern "C" int bsrl_proj_ffn_packed(const void* image, const void* att, const void* x, const float* ln2_w, const float* ln2_b,
                                     float eps2, const float* ln_w, const float* ln_b, float eps, void* xo, void* ho,
-                                    int64_t rows, int64_t d, int64_t F, int act, int dtype, bsrl_stream stream) {
+                                    void* qo, int64_t n_next, int64_t rows, int64_t d, int64_t F, int act, int dtype,
+                                    bsrl_stream stream) {
     if (!image || !att || !x || !xo || !ln2_w || !ln2_b) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: null pointer");
-    if ((ln_w == nullptr) != (ho == nullptr) || (ln_w == nullptr) != (ln_b == nullptr))
-        BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: ln_w, ln_b and ho go together");
-    if (!proj_ffn_shape_ok(d, F, dtype) || (act != BSRL_ACT_RELU && act != BSRL_ACT_GELU)) return BSRL_UNSUPPORTED;
+    if ((ln_w == nullptr) != (ln_b == nullptr)) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: ln_w and ln_b go together");
+    if (n_next == 0 && (ln_w == nullptr) != (ho == nullptr))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: without a projection behind, ln_w / ln_b and ho go together");
+    if (n_next > 0 && (!ln_w || !qo)) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: n_next > 0 needs ln_w, ln_b and qo");
+    if (ho && !ln_w) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: ho needs ln_w and ln_b");
+    if (!proj_ffn_shape_ok(d, F, n_next, dtype) || (act != BSRL_ACT_RELU && act != BSRL_ACT_GELU)) return BSRL_UNSUPPORTED;
     if (rows < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: rows < 0");
-    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(att, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)))
+    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(att, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)) ||
+        (qo && !bsrl_aligned(qo, 8)))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: image must be 16-byte, rows 8-byte aligned");
     if (rows == 0) return BSRL_OK;
     FfnArgs a;
     a.frags = static_cast<const uint2*>(image);
-    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + proj_frag_bytes(d) + ffn_frag_bytes(d, F));
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + proj_frag_bytes(d) + ffn_frag_bytes(d, F) +
+                                           (n_next / 32) * (d / 16) * 1024);
     a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(att);
     a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho); a.hid = nullptr;
     a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F;
-    a.total_stages = (int)(d / 32 + 2 * (F / 32));
+    a.total_stages = (int)(d / 32 + 2 * (F / 32) + n_next / 32);
     a.ln2_w = ln2_w; a.ln2_b = ln2_b; a.eps2 = eps2;
+    a.qo = static_cast<u16*>(qo); a.nq = (int)(n_next / 32);
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -1543,7 +1610,7 @@ extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2,
     a.x = static_cast<const u16*>(x); a.h2 = static_cast<const u16*>(h2);
     a.xo = static_cast<u16*>(xo); a.ho = static_cast<u16*>(ho); a.hid = static_cast<u16*>(hid);
     a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = (int)F; a.total_stages = (int)(2 * (F / 32));
-    a.ln2_w = a.ln2_b = nullptr; a.eps2 = 0.f;
+    a.ln2_w = a.ln2_b = nullptr; a.eps2 = 0.f; a.qo = nullptr; a.nq = 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess ||

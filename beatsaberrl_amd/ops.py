@@ -489,52 +489,60 @@ def ffn_fused(x, h2, w0, b0, w2, b2, act="relu", ln_w=None, ln_b=None, eps=1e-5,
     return xo, ho
 
 
-def proj_ffn_supported(d, F, dtype) -> bool:
-    """True where the block tail (output projection + LN2 + FFN) has a one-kernel form (bsrl_proj_ffn_packed)."""
-    return dtype is not torch.float32 and _lib.load().bsrl_proj_ffn_pack_size(d, F, dt_code(dtype)) > 0
+def proj_ffn_supported(d, F, dtype, n_next=0) -> bool:
+    """True where the block tail (output projection + LN2 + FFN, optionally the next block's packed projection of
+    n_next columns behind it) has a one-kernel form (bsrl_proj_ffn_packed)."""
+    return dtype is not torch.float32 and _lib.load().bsrl_proj_ffn_pack_size(d, F, n_next, dt_code(dtype)) > 0
 
 
-def proj_ffn_pack(wo, bo, w0, b0, w2, b2):
-    """Weight image of proj_ffn_fused (bsrl_proj_ffn_pack) from wo (d, d), w0 (F, d), w2 (d, F) in a 16-bit dtype and
-    the fp32 biases; rebuild once per weights version."""
-    _need_cuda(wo, w0, w2)
+def proj_ffn_pack(wo, bo, w0, b0, w2, b2, wn=None, bn=None):
+    """Weight image of proj_ffn_fused (bsrl_proj_ffn_pack) from wo (d, d), w0 (F, d), w2 (d, F), optionally wn
+    (n_next, d) - the projection applied to the LayerNorm-ed output, e.g. the next block's packed q|k|v - in a 16-bit
+    dtype and the fp32 biases; rebuild once per weights version."""
+    _need_cuda(wo, w0, w2, wn)
     Fh, d = w0.shape
-    n = _lib.load().bsrl_proj_ffn_pack_size(d, Fh, dt_code(w0.dtype))
-    if n <= 0 or tuple(wo.shape) != (d, d) or tuple(w2.shape) != (d, Fh) or not (wo.is_contiguous() and w0.is_contiguous() and w2.is_contiguous()):
-        raise Unsupported(f"proj_ffn_pack d={d} F={Fh} dtype={w0.dtype}")
+    n_next = 0 if wn is None else wn.shape[0]
+    n = _lib.load().bsrl_proj_ffn_pack_size(d, Fh, n_next, dt_code(w0.dtype))
+    if n <= 0 or tuple(wo.shape) != (d, d) or tuple(w2.shape) != (d, Fh) or not (wo.is_contiguous() and w0.is_contiguous() and w2.is_contiguous()) \
+            or (wn is not None and (wn.shape[1] != d or not wn.is_contiguous() or wn.dtype is not w0.dtype or bn is None or bn.numel() != n_next)):
+        raise Unsupported(f"proj_ffn_pack d={d} F={Fh} n_next={n_next} dtype={w0.dtype}")
     img = torch.empty(n, dtype=torch.uint8, device=w0.device)
     with torch.cuda.device(w0.device):
         rc = _lib.load().bsrl_proj_ffn_pack(wo.data_ptr(), _f32c(bo, "bo").data_ptr(), w0.data_ptr(), _f32c(b0, "b0").data_ptr(),
-                                            w2.data_ptr(), _f32c(b2, "b2").data_ptr(), d, Fh, dt_code(w0.dtype), img.data_ptr(),
-                                            _stream(w0))
+                                            w2.data_ptr(), _f32c(b2, "b2").data_ptr(), _ptr(wn), _ptr(_f32c(bn, "bn")), n_next,
+                                            d, Fh, dt_code(w0.dtype), img.data_ptr(), _stream(w0))
     if not _lib.check(rc, "bsrl_proj_ffn_pack"):
-        raise Unsupported(f"proj_ffn_pack d={d} F={Fh} dtype={w0.dtype}")
+        raise Unsupported(f"proj_ffn_pack d={d} F={Fh} n_next={n_next} dtype={w0.dtype}")
     return img
 
 
-def proj_ffn_fused(att, x, image, F, ln2_w, ln2_b, eps2=1e-5, act="relu", ln_w=None, ln_b=None, eps=1e-5):
+def proj_ffn_fused(att, x, image, F, ln2_w, ln2_b, eps2=1e-5, act="relu", ln_w=None, ln_b=None, eps=1e-5, n_next=0,
+                   want_ho=True):
     """The tail of a block from the attention output on: x1 = x + att Wo^T + bo, h2 = LN(x1; ln2), xo = x1 +
     act(h2 W0^T + b0) W2^T + b2, ho = LN(xo; ln) when ln_w is given - one kernel, x1 and h2 in registers.  att, x
-    (.., d) contiguous; image from proj_ffn_pack; F the hidden width.  Returns (xo, ho) (ho None without LN)."""
+    (.., d) contiguous; image from proj_ffn_pack; F the hidden width.  n_next > 0 (the image was packed with wn): also
+    qo (.., n_next) = ho Wn^T + bn from the same launch; want_ho=False then leaves ho unwritten.
+    Returns (xo, ho) or (xo, ho, qo) (ho None where not written)."""
     _need_cuda(att, x, image)
     d = x.shape[-1]
     if not (x.is_contiguous() and att.is_contiguous()) or att.shape != x.shape or att.dtype is not x.dtype:
         raise RuntimeError("proj_ffn_fused: att and x contiguous, one shape, one dtype")
-    if image.numel() != _lib.load().bsrl_proj_ffn_pack_size(d, F, dt_code(x.dtype)) or image.device != x.device:
+    if image.numel() != _lib.load().bsrl_proj_ffn_pack_size(d, F, n_next, dt_code(x.dtype)) or image.device != x.device:
         raise RuntimeError("proj_ffn_fused: image does not belong to this shape / dtype / device")
-    if ln2_w.numel() != d or ln2_b.numel() != d or (ln_w is None) != (ln_b is None):
-        raise RuntimeError(f"proj_ffn_fused: ln2_w / ln2_b of {d} elements; ln_w and ln_b come together")
+    if ln2_w.numel() != d or ln2_b.numel() != d or (ln_w is None) != (ln_b is None) or (n_next > 0 and ln_w is None):
+        raise RuntimeError(f"proj_ffn_fused: ln2_w / ln2_b of {d} elements; ln_w and ln_b come together, and with n_next")
     rows = x.numel() // d
     xo = torch.empty_like(x)
-    ho = torch.empty_like(x) if ln_w is not None else None
+    ho = torch.empty_like(x) if ln_w is not None and (want_ho or n_next == 0) else None
+    qo = torch.empty(*x.shape[:-1], n_next, device=x.device, dtype=x.dtype) if n_next > 0 else None
     with torch.cuda.device(x.device):
         rc = _lib.load().bsrl_proj_ffn_packed(image.data_ptr(), att.data_ptr(), x.data_ptr(), _f32c(ln2_w, "ln2_w").data_ptr(),
                                               _f32c(ln2_b, "ln2_b").data_ptr(), float(eps2), _ptr(_f32c(ln_w, "ln_w")),
-                                              _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), rows, d, F,
-                                              _ACT[act], dt_code(x.dtype), _stream(x))
+                                              _ptr(_f32c(ln_b, "ln_b")), float(eps), xo.data_ptr(), _ptr(ho), _ptr(qo), n_next,
+                                              rows, d, F, _ACT[act], dt_code(x.dtype), _stream(x))
     if not _lib.check(rc, "bsrl_proj_ffn_packed"):
-        raise Unsupported(f"proj_ffn_fused d={d} F={F} dtype={x.dtype}")
-    return xo, ho
+        raise Unsupported(f"proj_ffn_fused d={d} F={F} n_next={n_next} dtype={x.dtype}")
+    return (xo, ho, qo) if n_next > 0 else (xo, ho)
 
 
 def cfg_embed(obs, wp, bp, wo, bo, T, dtype):

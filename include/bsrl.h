@@ -171,18 +171,24 @@ int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const floa
  *   h2 = LayerNorm(x1; ln2_w, ln2_b)  its ln_ffn (python/policy.py:663-672, layer_norm.cu:14-21)
  *   xo = x1 + act(h2 W0^T + b0) W2^T + b2,  ho = LayerNorm(xo; ln_w, ln_b) if ln_w   (bsrl_ffn_packed)
  * with the rounding points of the separate launches (x1, h2, hidden, xo, ho rounded once each; fp32
- * accumulation and statistics), x1 and h2 never leaving the registers.  bsrl_proj_ffn_pack writes
- * the image (bsrl_proj_ffn_pack_size bytes, 16-byte aligned; 0 = unsupported shape) from wo (d, d),
- * w0 (F, d), w2 (d, F) in `dtype` and the fp32 biases.  att, x, xo, ho (rows, d) contiguous in
- * `dtype`, 8-byte aligned; ln2_w / ln2_b required, ln_w / ln_b / ho together or all NULL. */
-int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int dtype);
+ * accumulation and statistics), x1 and h2 never leaving the registers.  With n_next > 0 (a multiple
+ * of 64, at most 3 d) the NEXT block's packed projection comes out of the same launch:
+ *   qo = ho Wn^T + bn                 the q|k|v Linears of Block.forward (python/policy.py:541-560)
+ * (rows, n_next), rounded once, ho's fragments taken from the registers; ho itself is then written only
+ * if the pointer is given.  bsrl_proj_ffn_pack writes the image (bsrl_proj_ffn_pack_size bytes,
+ * 16-byte aligned; 0 = unsupported shape) from wo (d, d), w0 (F, d), w2 (d, F), wn (n_next, d; NULL
+ * when n_next = 0) in `dtype` and the fp32 biases.  att, x, xo, ho (rows, d), qo (rows, n_next)
+ * contiguous in `dtype`, 8-byte aligned; ln2_w / ln2_b required; ln_w / ln_b together; without a
+ * projection behind, ho goes with them. */
+int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int64_t n_next, int dtype);
 int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w0, const float* b0,
-                       const void* w2, const float* b2, int64_t d, int64_t F, int dtype,
-                       void* image, bsrl_stream stream);
+                       const void* w2, const float* b2, const void* wn, const float* bn,
+                       int64_t n_next, int64_t d, int64_t F, int dtype, void* image,
+                       bsrl_stream stream);
 int bsrl_proj_ffn_packed(const void* image, const void* att, const void* x, const float* ln2_w,
                          const float* ln2_b, float eps2, const float* ln_w, const float* ln_b,
-                         float eps, void* xo, void* ho, int64_t rows, int64_t d, int64_t F,
-                         int act, int dtype, bsrl_stream stream);
+                         float eps, void* xo, void* ho, void* qo, int64_t n_next, int64_t rows,
+                         int64_t d, int64_t F, int act, int dtype, bsrl_stream stream);
 
 /* ---- Config-model tokenizer -----------------------------------------------
  * The benchmark configs' "linear embedding": token 0 = Wp obs[:, :prop_dim] +

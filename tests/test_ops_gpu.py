@@ -334,6 +334,24 @@ def test_block_tail_in_one_kernel(dtype, rows, Fh, act, with_ln):
         lo, hi = 130, 290
         a, b = ops.proj_ffn_fused(att[lo:hi].contiguous(), x[lo:hi].contiguous(), img, Fh, l2w, l2b, 1e-5, act=act, ln_w=lw, ln_b=lb)
         assert torch.equal(a, xo[lo:hi]) and (b is None or torch.equal(b, ho[lo:hi]))
+    # ... with a projection of the LayerNorm-ed output behind it (the next block's packed q|k|v, or its k|v alone): xo and
+    # ho keep their bits, qo is the Linear of the SAME ho to one rounding (another accumulation order: <= 1 ulp, mostly equal)
+    if with_ln:
+        for n_next, want_ho in ((1152, False), (768, True)):
+            assert ops.proj_ffn_supported(d, Fh, dtype, n_next) and not ops.proj_ffn_supported(d, Fh, dtype, 96)
+            wn = _rand(n_next, d, dtype=dtype, seed=13, scale=1 / math.sqrt(d))
+            bn = _rand(n_next, seed=14) * 0.3
+            img_n = ops.proj_ffn_pack(wo, bo, w0, b0, w2, b2, wn, bn)
+            xo_n, ho_n, qo = ops.proj_ffn_fused(att, x, img_n, Fh, l2w, l2b, 1e-5, act=act, ln_w=lw, ln_b=lb, n_next=n_next,
+                                                want_ho=want_ho)
+            assert torch.equal(xo_n, xo) and qo.shape == (rows, n_next)
+            assert (ho_n is None) == (not want_ho) and (ho_n is None or torch.equal(ho_n, ho))
+            q_ref = ho.double() @ wn.double().t() + bn.double()
+            q_lin = ops.linear(ho, wn, bn)
+            qs = q_ref.abs().max().item()
+            assert (qo.double() - q_ref).abs().max().item() <= 1.01 * EPS16[dtype] * qs
+            assert (qo.float() - q_lin.float()).abs().max().item() <= 2 * EPS16[dtype] * qs
+            assert (qo == q_lin).float().mean().item() > 0.98
 
 
 def test_ffn_fused_unsupported_shapes_say_so():
