@@ -58,7 +58,7 @@ def main(argv=None):
         variants = {
             "persistent kernel, latency form (1 launch)": dict(route="fused", prune=False, latency=True),
             "persistent kernel (1 launch)": dict(route="fused", prune=False),
-            "fused, final block pruned (2 launches)": dict(route="fused", prune=True),
+            "fused, final block pruned (1 launch)": dict(route="fused", prune=True),
             "per-op route (multi-kernel)": dict(route="ops", prune=False),
         }
         for name, v in variants.items():
