@@ -1039,6 +1039,13 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
     const uint4* ring = reinterpret_cast<const uint4*>(bvl4) + ring_off_u4;
     const float* B1 = vlds; const float* B2 = vlds + a.F; const float* LNG = B2 + D; const float* LNB = LNG + D;
     const float* BO = LNB + D; const float* LN2G = BO + D; const float* LN2B = LN2G + D; const float* BN = LN2B + D;
+    // WIDE (d = 384): the weight rows of an accumulator-tile PAIR are ordered so that a lane's four features of tile
+    // 2p and its four of tile 2p + 1 are EIGHT CONSECUTIVE features, 32 p + 8 g + 0..7 (A row m of tile i is feature
+    // 32 (i / 2) + 8 (m / 4) + 4 (i % 2) + m % 4): rows come in and leave in 16-byte pieces, 64 contiguous bytes per
+    // row and instruction instead of 32, and both an input row's and a LayerNorm output's operand fragment hold their k
+    // values in natural order.  foff(nt): first feature of the lane's four in tile nt.
+    constexpr bool WIDE = D == 384;
+    auto foff = [&](int nt) __attribute__((always_inline)) { return WIDE ? 32 * (nt >> 1) + 8 * g + 4 * (nt & 1) : 16 * nt + 4 * g; };
     const int64_t ntiles = (a.rows + NW * 32 - 1) / (NW * 32);
 
     R pipe;
@@ -1077,11 +1084,14 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 const u16* xr = a.x + row * D;
                 uint2 rx[NT];
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) rx[nt] = *reinterpret_cast<const uint2*>(xr + 16 * nt + 4 * g);
+                for (int p = 0; p < NT / 2; ++p) {
+                    const uint4 r4 = *reinterpret_cast<const uint4*>(xr + 32 * p + 8 * g);
+                    rx[2 * p] = make_uint2(r4.x, r4.y); rx[2 * p + 1] = make_uint2(r4.z, r4.w);
+                }
                 __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const float4 b = *reinterpret_cast<const float4*>((PROJ ? BO : B2) + 16 * nt + 4 * g);
+                    const float4 b = *reinterpret_cast<const float4*>((PROJ ? BO : B2) + foff(nt));
                     x[rt][nt][0] = DT::to_f((u16)(rx[nt].x & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(rx[nt].x >> 16)) + b.y;
                     x[rt][nt][2] = DT::to_f((u16)(rx[nt].y & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(rx[nt].y >> 16)) + b.w;
                     asm("" : "+a"(x[rt][nt]));        // the accumulator lives in accumulation registers from here on
@@ -1093,7 +1103,10 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
                 const u16* hr = a.h2 + row * D;
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) hf[rt][nt >> 1].h[nt & 1] = *reinterpret_cast<const uint2*>(hr + 16 * nt + 4 * g);
+                for (int c = 0; c < KC; ++c) {
+                    const uint4 r4 = *reinterpret_cast<const uint4*>(hr + 32 * c + 8 * g);
+                    hf[rt][c].h[0] = make_uint2(r4.x, r4.y); hf[rt][c].h[1] = make_uint2(r4.z, r4.w);
+                }
             }
             __builtin_amdgcn_s_waitcnt(0x0F70);
         } else {   // the tile's own loads: all issued, one wait the compiler can see (it does not know of the ring's transfers)
@@ -1166,14 +1179,15 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
-        auto acc_init = [&](const float* bias, int ch) __attribute__((always_inline)) {
+        // (wide: the stage's 32 columns in the paired order above - a lane's four of tile 0 and four of tile 1 adjacent)
+        auto acc_init = [&](const float* bias, int ch, bool wide) __attribute__((always_inline)) {
 #pragma unroll
             for (int ntl = 0; ntl < 2; ++ntl) {
-                const float4 b = *reinterpret_cast<const float4*>(bias + 32 * ch + 16 * ntl + 4 * g);
+                const float4 b = *reinterpret_cast<const float4*>(bias + 32 * ch + (wide ? 8 * g + 4 * ntl : 16 * ntl + 4 * g));
                 acc[ntl][0] = (f32x4){b.x, b.y, b.z, b.w}; acc[ntl][1] = acc[ntl][0];
             }
         };
-        auto up_init = [&](int ch) __attribute__((always_inline)) { acc_init(B1, ch); };
+        auto up_init = [&](int ch) __attribute__((always_inline)) { acc_init(B1, ch, false); };
         auto up_mm = [&](auto i_, const s16x8& wf) __attribute__((always_inline)) {
             constexpr int j = decltype(i_)::value / KB, ci = decltype(i_)::value % KB, half = j / 2, ntl = j % 2;
 #pragma unroll
@@ -1218,9 +1232,9 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                     const float shift = -mean * rstd;
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
-                        const float4 gm = *reinterpret_cast<const float4*>(LN2G + 16 * nt + 4 * g);
-                        const float4 bt = *reinterpret_cast<const float4*>(LN2B + 16 * nt + 4 * g);
-                        const float4 b2 = *reinterpret_cast<const float4*>(B2 + 16 * nt + 4 * g);
+                        const float4 gm = *reinterpret_cast<const float4*>(LN2G + foff(nt));
+                        const float4 bt = *reinterpret_cast<const float4*>(LN2B + foff(nt));
+                        const float4 b2 = *reinterpret_cast<const float4*>(B2 + foff(nt));
                         f32x4 r = x[rt][nt];
                         uint2 v;
                         v.x = bpack2<DT>(fmaf(fmaf(r[0], rstd, shift), gm.x, bt.x), fmaf(fmaf(r[1], rstd, shift), gm.y, bt.y));
@@ -1289,11 +1303,15 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         for (int rt = 0; rt < 2; ++rt) {
             const int64_t row = row0 + 16 * rt + r16;
             u16* o = a.xo + row * D;
+            uint2 vprev = make_uint2(0, 0);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 uint2 v;
                 v.x = bpack2<DT>(x[rt][nt][0], x[rt][nt][1]); v.y = bpack2<DT>(x[rt][nt][2], x[rt][nt][3]);
-                if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                if constexpr (WIDE) {
+                    if (nt & 1) { if (row < a.rows) *reinterpret_cast<uint4*>(o + 32 * (nt >> 1) + 8 * g) = make_uint4(vprev.x, vprev.y, v.x, v.y); }
+                    else vprev = v;
+                } else if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
                 if (LN) {
                     x[rt][nt][0] = DT::to_f((u16)(v.x & 0xffff)); x[rt][nt][1] = DT::to_f((u16)(v.x >> 16));
                     x[rt][nt][2] = DT::to_f((u16)(v.y & 0xffff)); x[rt][nt][3] = DT::to_f((u16)(v.y >> 16));
@@ -1313,40 +1331,42 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 const float mean = s[rt] * (1.0f / D);
                 const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, q[rt] * (1.0f / D)), 0.f) + a.eps);
                 const float shift = -mean * rstd;
+                uint2 hprev = make_uint2(0, 0);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
-                    const float4 gm = *reinterpret_cast<const float4*>(LNG + 16 * nt + 4 * g);
-                    const float4 bt = *reinterpret_cast<const float4*>(LNB + 16 * nt + 4 * g);
+                    const float4 gm = *reinterpret_cast<const float4*>(LNG + foff(nt));
+                    const float4 bt = *reinterpret_cast<const float4*>(LNB + foff(nt));
                     uint2 v;
                     v.x = bpack2<DT>(fmaf(fmaf(x[rt][nt][0], rstd, shift), gm.x, bt.x), fmaf(fmaf(x[rt][nt][1], rstd, shift), gm.y, bt.y));
                     v.y = bpack2<DT>(fmaf(fmaf(x[rt][nt][2], rstd, shift), gm.z, bt.z), fmaf(fmaf(x[rt][nt][3], rstd, shift), gm.w, bt.w));
-                    if (row < a.rows && (!PROJ || a.ho)) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
+                    if constexpr (WIDE) {
+                        if (nt & 1) {
+                            if (row < a.rows && (!PROJ || a.ho)) *reinterpret_cast<uint4*>(o + 32 * (nt >> 1) + 8 * g) = make_uint4(hprev.x, hprev.y, v.x, v.y);
+                        } else hprev = v;
+                    } else if (row < a.rows && (!PROJ || a.ho)) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
                     if constexpr (PROJ) hf[rt][nt >> 1].h[nt & 1] = v;       // operand fragments of the projection behind
                 }
             }
         }
         if constexpr (PROJ && LN) {
             // qo = ho Wn^T + bn: nq stages of 32 output columns in the up-projection's form (the first is admitted and its
-            // first fragments are in flight), each stored as it completes - a lane's four columns of a tile, 8 bytes
+            // first fragments are in flight), each stored as it completes
             const int ldq = 32 * a.nq;
             auto q_store = [&](int sq) __attribute__((always_inline)) {
 #pragma unroll
                 for (int rt = 0; rt < 2; ++rt) {
                     const int64_t row = row0 + 16 * rt + r16;
-                    if (row < a.rows) {
-                        u16* qr = a.qo + row * ldq + 32 * sq + 4 * g;
-#pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl) {
-                            uint2 v;
-                            v.x = bpack2<DT>(acc[ntl][rt][0], acc[ntl][rt][1]); v.y = bpack2<DT>(acc[ntl][rt][2], acc[ntl][rt][3]);
-                            *reinterpret_cast<uint2*>(qr + 16 * ntl) = v;
-                        }
+                    if (row < a.rows) {       // the stage's columns in the paired order: 16 bytes per lane
+                        uint4 v;
+                        v.x = bpack2<DT>(acc[0][rt][0], acc[0][rt][1]); v.y = bpack2<DT>(acc[0][rt][2], acc[0][rt][3]);
+                        v.z = bpack2<DT>(acc[1][rt][0], acc[1][rt][1]); v.w = bpack2<DT>(acc[1][rt][2], acc[1][rt][3]);
+                        *reinterpret_cast<uint4*>(a.qo + row * ldq + 32 * sq + 8 * g) = v;
                     }
                 }
             };
             for (int sq = 0; sq < a.nq; sq += 2) {       // nq is even: an even stage, then an odd one
-                acc_init(BN, sq); stage(1, up_mm); q_store(sq);
-                acc_init(BN, sq + 1); stage(sq + 2 < a.nq ? 2 : 0, up_mm); q_store(sq + 1);
+                acc_init(BN, sq, true); stage(1, up_mm); q_store(sq);
+                acc_init(BN, sq + 1, true); stage(sq + 2 < a.nq ? 2 : 0, up_mm); q_store(sq + 1);
             }
         }
     }
@@ -1371,14 +1391,17 @@ __global__ __launch_bounds__(256) void ffn_pack_frags_kernel(FfnPackArgs a) {
     else if (s3 == 2 * nch - 1) { upw = false; ch = nch - 1; }
     else { upw = ((s3 - 1) & 1) == 0; ch = (s3 - 1) / 2 + (upw ? 1 : 0); }
     const u16* src; int ld, n, kbase = 0, c = 0;
+    // d = 384 (the kernel's WIDE order): feature tiles' rows paired - A row m of tile i is feature
+    // 32 (i / 2) + 8 (m / 4) + 4 (i % 2) + m % 4 -, and the k values of an INPUT-feature chunk in natural order
+    constexpr bool WIDE = D == 384;
     if (upw) {
         const int burst = i / G::FB, rem = i % G::FB, ntl = rem / G::KB;
         c = burst * G::KB + rem % G::KB;
         src = a.w0; ld = D; n = 32 * ch + 16 * ntl + n16;
-    } else { src = a.w2; ld = a.F; n = 16 * i + n16; kbase = 32 * ch; }
+    } else { src = a.w2; ld = a.F; n = WIDE ? 32 * (i >> 1) + 8 * (n16 >> 2) + 4 * (i & 1) + (n16 & 3) : 16 * i + n16; kbase = 32 * ch; }
     u16 v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + bperm_k(c, gg, j)];
+    for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)n * ld + kbase + (WIDE && upw ? 32 * c + 8 * gg + j : bperm_k(c, gg, j))];
     uint4 o;
     o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
     o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
@@ -1466,7 +1489,8 @@ __global__ __launch_bounds__(256) void proj_pack_frags_kernel(ProjPackArgs a) {
     const int c = f / SF, i = f % SF;
     u16 v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = a.wo[(int64_t)(16 * i + n16) * D + 32 * c + bperm_k(0, gg, j)];
+    for (int j = 0; j < 8; ++j)       // rows in the paired order, the attention output's k values in natural order
+        v[j] = a.wo[(int64_t)(32 * (i >> 1) + 8 * (n16 >> 2) + 4 * (i & 1) + (n16 & 3)) * D + 32 * c + 8 * gg + j];
     uint4 o;
     o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
     o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
@@ -1485,7 +1509,8 @@ __global__ __launch_bounds__(256) void next_pack_frags_kernel(ProjPackArgs a) {
     const int burst = i / G::FB, rem = i % G::FB, ntl = rem / G::KB, c = burst * G::KB + rem % G::KB;
     u16 v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = a.wn[(int64_t)(32 * sq + 16 * ntl + n16) * D + bperm_k(c, gg, j)];
+    for (int j = 0; j < 8; ++j)       // the stage's 32 columns in the paired order, k natural
+        v[j] = a.wn[(int64_t)(32 * sq + 8 * (n16 >> 2) + 4 * ntl + (n16 & 3)) * D + 32 * c + 8 * gg + j];
     uint4 o;
     o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
     o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
@@ -1545,6 +1570,8 @@ extern "C" int bsrl_proj_ffn_packed(const void* image, const void* att, const vo
     if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(att, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)) ||
         (qo && !bsrl_aligned(qo, 8)))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: image must be 16-byte, rows 8-byte aligned");
+    if (!bsrl_aligned(x, 16) || !bsrl_aligned(att, 16) || !bsrl_aligned(xo, 16) || (ho && !bsrl_aligned(ho, 16)) || (qo && !bsrl_aligned(qo, 16)))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_proj_ffn_packed: rows must be 16-byte aligned");
     if (rows == 0) return BSRL_OK;
     FfnArgs a;
     a.frags = static_cast<const uint2*>(image);
@@ -1603,6 +1630,8 @@ extern "C" int bsrl_ffn_packed(const void* image, const void* x, const void* h2,
     if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 8) || !bsrl_aligned(h2, 8) || !bsrl_aligned(xo, 8) || (ho && !bsrl_aligned(ho, 8)) ||
         (hid && !bsrl_aligned(hid, 8)))
         BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: image must be 16-byte, rows 8-byte aligned");
+    if (d == 384 && (!bsrl_aligned(x, 16) || !bsrl_aligned(h2, 16) || !bsrl_aligned(xo, 16) || (ho && !bsrl_aligned(ho, 16))))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_ffn_packed: at d = 384 rows must be 16-byte aligned (they move in 16-byte pieces)");
     if (rows == 0) return BSRL_OK;
     FfnArgs a;
     a.frags = static_cast<const uint2*>(image);

@@ -156,7 +156,7 @@ int bsrl_ffn_fused_supported(int64_t d, int64_t F, int dtype);
  * unsupported shape) from w0 (F, d) and w2 (d, F) in `dtype` and the fp32 biases - once per
  * weight update, like the 16-bit replicas the reference keeps (python/fp16_linear.py:150-192);
  * bsrl_ffn_packed is bsrl_ffn_fused with the image in place of w0, b0, w2, b2.  x, h2, xo, ho
- * (rows, d) contiguous in `dtype`, 8-byte aligned.  hid, if not NULL, receives the activated
+ * (rows, d) contiguous in `dtype`, 8-byte aligned (d = 384: 16-byte).  hid, if not NULL, receives the activated
  * hidden (rows, F) in `dtype` exactly as the down-projection consumed it - what the reference's
  * kernel returns for the backward (fused_ffn.cu:551-619, `hid`; its ReLU mask is hid > 0). */
 int64_t bsrl_ffn_pack_size(int64_t d, int64_t F, int dtype);
@@ -178,7 +178,7 @@ int bsrl_ffn_packed(const void* image, const void* x, const void* h2, const floa
  * if the pointer is given.  bsrl_proj_ffn_pack writes the image (bsrl_proj_ffn_pack_size bytes,
  * 16-byte aligned; 0 = unsupported shape) from wo (d, d), w0 (F, d), w2 (d, F), wn (n_next, d; NULL
  * when n_next = 0) in `dtype` and the fp32 biases.  att, x, xo, ho (rows, d), qo (rows, n_next)
- * contiguous in `dtype`, 8-byte aligned; ln2_w / ln2_b required; ln_w / ln_b together; without a
+ * contiguous in `dtype`, 16-byte aligned; ln2_w / ln2_b required; ln_w / ln_b together; without a
  * projection behind, ho goes with them. */
 int64_t bsrl_proj_ffn_pack_size(int64_t d, int64_t F, int64_t n_next, int dtype);
 int bsrl_proj_ffn_pack(const void* wo, const float* bo, const void* w0, const float* b0,
