@@ -8,7 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbsrl_hip.so")
-ABI_VERSION = 16
+ABI_VERSION = 17
 CFG_NO_PACK = 1                 # bsrl_cfg_desc.flags: one env per tile in the fused forward
 CFG_NO_LATENCY = 2              # bsrl_cfg_desc.flags: small batches take the throughput forms too
 CFG_STATIC_MAX_ENVS = 16384     # BSRL_CFG_STATIC_MAX_ENVS: batch limit of bsrl_cfg_forward_static
@@ -63,6 +63,9 @@ SIGNATURES = {
     "bsrl_ffn_pack_size": (_i64, [_i64, _i64, _i32]),
     "bsrl_ffn_pack": (_i32, [_p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
     "bsrl_ffn_packed": (_i32, [_p, _p, _p, _p, _p, _f, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p]),
+    "bsrl_ln_proj_pack_size": (_i64, [_i64, _i64, _i32]),
+    "bsrl_ln_proj_pack": (_i32, [_p, _p, _i64, _i64, _i32, _p, _p]),
+    "bsrl_ln_proj_packed": (_i32, [_p, _p, _p, _p, _f, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "bsrl_proj_ffn_pack_size": (_i64, [_i64, _i64, _i64, _i32]),
     "bsrl_proj_ffn_pack": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p, _p]),
     "bsrl_proj_ffn_packed": (_i32, [_p, _p, _p, _p, _p, _f, _p, _p, _f, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _i32, _p]),

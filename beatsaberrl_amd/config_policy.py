@@ -315,10 +315,19 @@ class ConfigPolicy(nn.Module):
         for i, (blk, w) in enumerate(zip(self.blocks, r["blk"])):
             pruned = self.prune_final and i + 1 == L
             if proj is None:
-                if h is None:
-                    h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
                 # Row slices of the packed q|k|v weight are contiguous views: keys and values only for a pruned block
-                proj = ops.linear(h, w["qkv_w"][d:], w["qkv_b"][d:]) if pruned else ops.linear(h, w["qkv_w"], w["qkv_b"])
+                lo = d if pruned else 0
+                if h is None and self.fuse_block_tail and self.fuse_next_proj and ops.ln_proj_supported(d, 3 * d - lo, dt):
+                    # LN1 + the packed projection in one kernel (LN1 itself written only for the pruned block's query row)
+                    img = w["tail_img"].get(("lead", lo))
+                    if img is None:
+                        img = w["tail_img"][("lead", lo)] = ops.ln_proj_pack(w["qkv_w"][lo:], w["qkv_b"][lo:])
+                    h, proj = ops.ln_proj_fused(x, img, 3 * d - lo, blk.ln_attn.weight.detach(), blk.ln_attn.bias.detach(),
+                                                blk.ln_attn.eps, want_ho=pruned)
+                else:
+                    if h is None:
+                        h = ops.ln_fwd(x, blk.ln_attn.weight, blk.ln_attn.bias, blk.ln_attn.eps)
+                    proj = ops.linear(h, w["qkv_w"][lo:], w["qkv_b"][lo:])
             if pruned:
                 # Only token 0 of the final block is read (the reference's n_queries path, python/policy.py:533-539:
                 # exact, masking is key-side only): keys and values of every token, the query, the output projection,

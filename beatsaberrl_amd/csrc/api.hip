@@ -11,5 +11,5 @@ void bsrl_set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
-extern "C" int bsrl_version(void) { return 16; }
+extern "C" int bsrl_version(void) { return 17; }
 extern "C" const char* bsrl_last_error(void) { return g_err; }

@@ -1023,11 +1023,14 @@ template <int D, int NW> constexpr int ffn_wgs_per_cu() { return D == 384 ? 1 : 
 // of the stream).  The projection runs as d / 32 more stages of the down-projection's form (the attention output's
 // operand fragments in place of the hidden chunk); the rounded x1 and h2 never leave the registers: a lane's four
 // features of an accumulator tile are half of an operand fragment of the up-projection.
-template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_, int XS, bool PROJ = false>
+// LEAD (a PROJ instantiation with LN): nothing but the last phase - qo = LayerNorm(x) Wn^T + bn; the image holds the nq
+// projection stages only (F = 0), h2 is not read, xo is not written.
+template <typename DT, int D, int ACT, bool LN, bool SAVE, int NW_, int XS, bool PROJ = false, bool LEAD = false>
 __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows_kernel(FfnArgs a) {
     typedef Geo<D> G;
     typedef FfnRing<D, NW_, XS> R;
     static_assert(!PROJ || (D == 384 && !SAVE), "the projection form exists for the register-pipelined d = 384 kernel");
+    static_assert(!LEAD || (PROJ && LN), "the lead form is the projection form's last phase");
     constexpr int NW = R::NW, NT = G::NT, KC = G::KC, NB = G::NB, KB = G::KB, NSUB = 2 * NB;
     extern __shared__ float4 bvl4[];          // b0 (F) | b2 (d) | ln_w (d) | ln_b (d), then the stage ring (1 KB aligned)
     float* vlds = reinterpret_cast<float*>(bvl4);
@@ -1098,6 +1101,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (!LEAD)
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
@@ -1197,7 +1201,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         if constexpr (PIPE) {      // an odd stage follows W1(0): W1(1), or W2(0) when nch == 1
 #pragma unroll
             for (int f = 0; f < NBUF - 1; ++f) wr[f] = pipe.frag(f, lane);
-            if constexpr (PROJ) {
+            if constexpr (PROJ && !LEAD) {
                 // KC projection stages (even, odd, ...; KC is even, so W1(0) stays an even stage): stage c adds
                 // Wo[:, 32 c .. 32 c + 31] times the attention output's chunk c into every feature tile
                 static_for<0, KC>([&](auto c_) __attribute__((always_inline)) {
@@ -1247,7 +1251,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                     }
                 }
             }
-            up_init(0); stage(1, up_mm);
+            if constexpr (!LEAD) { up_init(0); stage(1, up_mm); }
         }
         else up(0);
         for (int ch = 0; ch < nch; ++ch) {
@@ -1309,7 +1313,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                 uint2 v;
                 v.x = bpack2<DT>(x[rt][nt][0], x[rt][nt][1]); v.y = bpack2<DT>(x[rt][nt][2], x[rt][nt][3]);
                 if constexpr (WIDE) {
-                    if (nt & 1) { if (row < a.rows) *reinterpret_cast<uint4*>(o + 32 * (nt >> 1) + 8 * g) = make_uint4(vprev.x, vprev.y, v.x, v.y); }
+                    if (nt & 1) { if (row < a.rows && !LEAD) *reinterpret_cast<uint4*>(o + 32 * (nt >> 1) + 8 * g) = make_uint4(vprev.x, vprev.y, v.x, v.y); }
                     else vprev = v;
                 } else if (row < a.rows) *reinterpret_cast<uint2*>(o + 16 * nt + 4 * g) = v;
                 if (LN) {
@@ -1456,7 +1460,7 @@ int ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
 }
 
 // the projection form (d = 384): six ring slots where the longer vector block leaves room, else five
-template <typename DT, int ACT, int XS>
+template <typename DT, int ACT, int XS, bool LEAD = false>
 int proj_ffn_launch_xs(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
     constexpr int D = 384, NW = 4;
     const size_t dyn = ffn_dyn_bytes<D, NW, XS>(a.F, true, a.nq);
@@ -1469,7 +1473,8 @@ int proj_ffn_launch_xs(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
         hipLaunchKernelGGL(kern, grid, dim3(NW * 64), dyn, st, a);
         return (int)BSRL_OK;
     };
-    return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW, XS, true>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW, XS, true>);
+    if constexpr (LEAD) return launch(ffn_rows_kernel<DT, D, ACT, true, false, NW, XS, true, true>);
+    else return ln ? launch(ffn_rows_kernel<DT, D, ACT, true, false, NW, XS, true>) : launch(ffn_rows_kernel<DT, D, ACT, false, false, NW, XS, true>);
 }
 template <typename DT, int ACT>
 int proj_ffn_launch(const FfnArgs& a, bool ln, int cus, hipStream_t st) {
@@ -1516,6 +1521,8 @@ __global__ __launch_bounds__(256) void next_pack_frags_kernel(ProjPackArgs a) {
     o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
     static_cast<uint4*>(a.nfrags)[(int64_t)f * 64 + lane] = o;
     if (f == 0) for (int k = lane; k < 32 * a.nq; k += 64) a.vec_bo[D + k] = a.bn[k];
+    // an image without the stages in front (no output projection): the kernel's b2 | bo are zeros
+    if (f == 0 && a.wo == nullptr) for (int k = lane; k < 2 * D; k += 64) a.vec_bo[k - D] = 0.f;
 }
 bool proj_ffn_shape_ok(int64_t d, int64_t F, int64_t n_next, int dtype) {
     return d == 384 && ffn_packed_shape_ok(d, F, dtype) && n_next >= 0 && n_next % 64 == 0 && n_next <= 3 * d;
@@ -1593,6 +1600,63 @@ extern "C" int bsrl_proj_ffn_packed(const void* image, const void* att, const vo
     else rc = relu ? proj_ffn_launch<BF16, BSRL_ACT_RELU>(a, ln, cus, st) : proj_ffn_launch<BF16, BSRL_ACT_GELU>(a, ln, cus, st);
     if (rc != BSRL_OK) return rc;
     BSRL_CHECK_LAUNCH("bsrl_proj_ffn_packed");
+    return BSRL_OK;
+}
+
+// LayerNorm + packed projection alone: the block-tail kernel with nothing in front of its last phase
+namespace {
+bool ln_proj_shape_ok(int64_t d, int64_t n_next, int dtype) {
+    return d == 384 && (dtype == BSRL_F16 || dtype == BSRL_BF16) && n_next >= 6 * 32 && n_next % 64 == 0 && n_next <= 3 * d;
+}
+}  // namespace
+
+extern "C" int64_t bsrl_ln_proj_pack_size(int64_t d, int64_t n_next, int dtype) {
+    if (!ln_proj_shape_ok(d, n_next, dtype)) return 0;
+    return (n_next / 32) * (d / 16) * 1024 + (2 * d + n_next) * 4;
+}
+
+extern "C" int bsrl_ln_proj_pack(const void* wn, const float* bn, int64_t n_next, int64_t d, int dtype, void* image,
+                                 bsrl_stream stream) {
+    if (!wn || !bn || !image) BSRL_FAIL(BSRL_EINVAL, "bsrl_ln_proj_pack: null pointer");
+    if (!ln_proj_shape_ok(d, n_next, dtype)) return BSRL_UNSUPPORTED;
+    if (!bsrl_aligned(image, 16)) BSRL_FAIL(BSRL_EINVAL, "bsrl_ln_proj_pack: image must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float* vec = reinterpret_cast<float*>(static_cast<char*>(image) + (n_next / 32) * (d / 16) * 1024);   // zeros (2 d: the kernel's b2 | bo) | bn
+    ProjPackArgs pp{nullptr, nullptr, nullptr, vec + d, static_cast<const u16*>(wn), bn, image, (int)(n_next / 32)};
+    const int64_t nnf = (n_next / 32) * (d / 16);
+    hipLaunchKernelGGL(next_pack_frags_kernel<384>, dim3((unsigned)((nnf + 3) / 4)), dim3(256), 0, st, pp);
+    BSRL_CHECK_LAUNCH("bsrl_ln_proj_pack");
+    return BSRL_OK;
+}
+
+extern "C" int bsrl_ln_proj_packed(const void* image, const void* x, const float* ln_w, const float* ln_b, float eps,
+                                   void* ho, void* qo, int64_t n_next, int64_t rows, int64_t d, int dtype, bsrl_stream stream) {
+    if (!image || !x || !ln_w || !ln_b || !qo) BSRL_FAIL(BSRL_EINVAL, "bsrl_ln_proj_packed: null pointer");
+    if (!ln_proj_shape_ok(d, n_next, dtype)) return BSRL_UNSUPPORTED;
+    if (rows < 0) BSRL_FAIL(BSRL_EINVAL, "bsrl_ln_proj_packed: rows < 0");
+    if (!bsrl_aligned(image, 16) || !bsrl_aligned(x, 16) || (ho && !bsrl_aligned(ho, 16)) || !bsrl_aligned(qo, 16))
+        BSRL_FAIL(BSRL_EINVAL, "bsrl_ln_proj_packed: image and rows must be 16-byte aligned");
+    if (rows == 0) return BSRL_OK;
+    FfnArgs a;
+    a.frags = static_cast<const uint2*>(image);
+    a.vec = reinterpret_cast<const float*>(static_cast<const char*>(image) + (n_next / 32) * (d / 16) * 1024);
+    a.x = static_cast<const u16*>(x); a.h2 = a.x;
+    a.xo = nullptr; a.ho = static_cast<u16*>(ho); a.hid = nullptr;
+    a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps; a.rows = rows; a.F = 0;
+    a.total_stages = (int)(n_next / 32);
+    a.ln2_w = ln_w; a.ln2_b = ln_b; a.eps2 = eps;
+    a.qo = static_cast<u16*>(qo); a.nq = (int)(n_next / 32);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    int rc = dtype == BSRL_F16 ? proj_ffn_launch_xs<F16, BSRL_ACT_RELU, 1, true>(a, true, cus, st)
+                               : proj_ffn_launch_xs<BF16, BSRL_ACT_RELU, 1, true>(a, true, cus, st);
+    if (rc == BSRL_UNSUPPORTED)
+        rc = dtype == BSRL_F16 ? proj_ffn_launch_xs<F16, BSRL_ACT_RELU, 0, true>(a, true, cus, st)
+                               : proj_ffn_launch_xs<BF16, BSRL_ACT_RELU, 0, true>(a, true, cus, st);
+    if (rc != BSRL_OK) return rc;
+    BSRL_CHECK_LAUNCH("bsrl_ln_proj_packed");
     return BSRL_OK;
 }
 

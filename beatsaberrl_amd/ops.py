@@ -545,6 +545,48 @@ def proj_ffn_fused(att, x, image, F, ln2_w, ln2_b, eps2=1e-5, act="relu", ln_w=N
     return (xo, ho, qo) if n_next > 0 else (xo, ho)
 
 
+def ln_proj_supported(d, n_next, dtype) -> bool:
+    """True where LayerNorm + a packed projection of n_next columns has a one-kernel form (bsrl_ln_proj_packed)."""
+    return dtype is not torch.float32 and _lib.load().bsrl_ln_proj_pack_size(d, n_next, dt_code(dtype)) > 0
+
+
+def ln_proj_pack(wn, bn):
+    """Weight image of ln_proj_fused (bsrl_ln_proj_pack) from wn (n_next, d) in a 16-bit dtype and bn fp32."""
+    _need_cuda(wn, bn)
+    n_next, d = wn.shape
+    n = _lib.load().bsrl_ln_proj_pack_size(d, n_next, dt_code(wn.dtype))
+    if n <= 0 or not wn.is_contiguous() or bn.numel() != n_next:
+        raise Unsupported(f"ln_proj_pack d={d} n_next={n_next} dtype={wn.dtype}")
+    img = torch.empty(n, dtype=torch.uint8, device=wn.device)
+    with torch.cuda.device(wn.device):
+        rc = _lib.load().bsrl_ln_proj_pack(wn.data_ptr(), _f32c(bn, "bn").data_ptr(), n_next, d, dt_code(wn.dtype), img.data_ptr(),
+                                           _stream(wn))
+    if not _lib.check(rc, "bsrl_ln_proj_pack"):
+        raise Unsupported(f"ln_proj_pack d={d} n_next={n_next} dtype={wn.dtype}")
+    return img
+
+
+def ln_proj_fused(x, image, n_next, ln_w, ln_b, eps=1e-5, want_ho=False):
+    """qo (.., n_next) = LayerNorm(x; ln_w, ln_b) Wn^T + bn in one kernel (image from ln_proj_pack); x (.., d)
+    contiguous.  Returns (ho, qo): ho = the LayerNorm output when want_ho, else None."""
+    _need_cuda(x, image)
+    d = x.shape[-1]
+    if not x.is_contiguous() or ln_w.numel() != d or ln_b.numel() != d:
+        raise RuntimeError(f"ln_proj_fused: x contiguous, ln_w / ln_b of {d} elements")
+    if image.numel() != _lib.load().bsrl_ln_proj_pack_size(d, n_next, dt_code(x.dtype)) or image.device != x.device:
+        raise RuntimeError("ln_proj_fused: image does not belong to this shape / dtype / device")
+    rows = x.numel() // d
+    ho = torch.empty_like(x) if want_ho else None
+    qo = torch.empty(*x.shape[:-1], n_next, device=x.device, dtype=x.dtype)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bsrl_ln_proj_packed(image.data_ptr(), x.data_ptr(), _f32c(ln_w, "ln_w").data_ptr(),
+                                             _f32c(ln_b, "ln_b").data_ptr(), float(eps), _ptr(ho), qo.data_ptr(), n_next, rows, d,
+                                             dt_code(x.dtype), _stream(x))
+    if not _lib.check(rc, "bsrl_ln_proj_packed"):
+        raise Unsupported(f"ln_proj_fused d={d} n_next={n_next} dtype={x.dtype}")
+    return ho, qo
+
+
 def cfg_embed(obs, wp, bp, wo, bo, T, dtype):
     """Config-model tokenizer: obs (B, obs_dim) fp32 or `dtype` -> tokens (B, T, d)."""
     _need_cuda(obs, wp, wo)

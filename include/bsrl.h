@@ -189,6 +189,19 @@ int bsrl_proj_ffn_packed(const void* image, const void* att, const void* x, cons
                          const float* ln2_b, float eps2, const float* ln_w, const float* ln_b,
                          float eps, void* xo, void* ho, void* qo, int64_t n_next, int64_t rows,
                          int64_t d, int64_t F, int act, int dtype, bsrl_stream stream);
+/* The last phase of that kernel alone, for the first block of a stack (d = 384):
+ *   ho = LayerNorm(x; ln_w, ln_b)     Block.forward's ln_attn (python/policy.py:541, layer_norm.cu:14-21)
+ *   qo = ho Wn^T + bn                 its packed q|k|v Linears (python/policy.py:541-560)
+ * one launch, ho's fragments taken from the registers (ho itself written only if the pointer is
+ * given).  n_next a multiple of 64 in [192, 3 d]; image (bsrl_ln_proj_pack_size bytes, 16-byte
+ * aligned; 0 = unsupported) from wn (n_next, d) in `dtype` and bn fp32.  x, ho (rows, d), qo
+ * (rows, n_next) contiguous in `dtype`, 16-byte aligned. */
+int64_t bsrl_ln_proj_pack_size(int64_t d, int64_t n_next, int dtype);
+int bsrl_ln_proj_pack(const void* wn, const float* bn, int64_t n_next, int64_t d, int dtype,
+                      void* image, bsrl_stream stream);
+int bsrl_ln_proj_packed(const void* image, const void* x, const float* ln_w, const float* ln_b,
+                        float eps, void* ho, void* qo, int64_t n_next, int64_t rows, int64_t d,
+                        int dtype, bsrl_stream stream);
 
 /* ---- Config-model tokenizer -----------------------------------------------
  * The benchmark configs' "linear embedding": token 0 = Wp obs[:, :prop_dim] +

@@ -354,6 +354,36 @@ def test_block_tail_in_one_kernel(dtype, rows, Fh, act, with_ln):
             assert (qo == q_lin).float().mean().item() > 0.98
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,n_next,want_ho", [(1, 1152, False), (77, 1152, True), (1000, 768, True), (33000, 1152, False)])
+def test_layernorm_and_packed_projection_in_one_kernel(dtype, rows, n_next, want_ho):
+    """LN1 + the packed q|k|v Linears of a block (python/policy.py:541-560) as one launch at d = 384: the LayerNorm output
+    has ln_fwd's rounding (one flip per thousands of values at most: the statistics are summed in another order), the
+    projection is the Linear of that output to one rounding."""
+    d = 384
+    assert ops.ln_proj_supported(d, n_next, dtype) and not ops.ln_proj_supported(256, 768, dtype) and not ops.ln_proj_supported(d, 96, dtype)
+    x = _rand(rows, d, dtype=dtype, seed=1)
+    wn = _rand(n_next, d, dtype=dtype, seed=2, scale=1 / math.sqrt(d))
+    bn = _rand(n_next, seed=3) * 0.3
+    lw, lb = _rand(d, seed=4) * 0.2 + 1.0, _rand(d, seed=5) * 0.2
+    img = ops.ln_proj_pack(wn, bn)
+    ho, qo = ops.ln_proj_fused(x, img, n_next, lw, lb, 1e-5, want_ho=want_ho)
+    h_ref = ops.ln_fwd(x, lw, lb, 1e-5)
+    assert (ho is None) == (not want_ho)
+    if want_ho:
+        assert (ho.float() - h_ref.float()).abs().max().item() <= 1.01 * EPS16[dtype] * h_ref.float().abs().max().item()
+        assert (ho == h_ref).float().mean().item() > 0.995
+        q_ref = ho.double() @ wn.double().t() + bn.double()
+        assert (qo.double() - q_ref).abs().max().item() <= 1.01 * EPS16[dtype] * q_ref.abs().max().item()
+    q_lin = ops.linear(h_ref, wn, bn)
+    qs = q_lin.float().abs().max().item()
+    assert (qo.float() - q_lin.float()).abs().max().item() <= 4 * EPS16[dtype] * qs
+    if rows >= 1000:
+        lo, hi = 130, 290
+        _, b = ops.ln_proj_fused(x[lo:hi].contiguous(), img, n_next, lw, lb, 1e-5)
+        assert torch.equal(b, qo[lo:hi])
+
+
 def test_ffn_fused_unsupported_shapes_say_so():
     assert not ops.ffn_fused_supported(160, 640, torch.float16)
     assert not ops.ffn_fused_supported(128, 500, torch.float16)
