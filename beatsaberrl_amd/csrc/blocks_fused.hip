@@ -1078,28 +1078,16 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         f32x4 x[2][NT];
         BFrag8 hf[2][KC];
         if constexpr (D == 384) {
-            // x and its accumulator first, h2 after them: with both raw inputs and the accumulator live at once the
-            // register allocator spills operand fragments, and reloads them from scratch in every chunk of the loop
-            // below (whose waits on those reloads drain the ring's transfers too)
+            // every load of the tile issued at once - x row tile 0, x row tile 1, then h2 -, and the compiler's own waits
+            // (it counts its loads, not the ring's transfers, which only makes them stricter) let each conversion start
+            // as its rows land: one memory latency per tile, not one per array
+            uint4 rx[2][NT / 2];
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 int64_t row = row0 + 16 * rt + r16; row = row < a.rows ? row : a.rows - 1;
                 const u16* xr = a.x + row * D;
-                uint2 rx[NT];
 #pragma unroll
-                for (int p = 0; p < NT / 2; ++p) {
-                    const uint4 r4 = *reinterpret_cast<const uint4*>(xr + 32 * p + 8 * g);
-                    rx[2 * p] = make_uint2(r4.x, r4.y); rx[2 * p + 1] = make_uint2(r4.z, r4.w);
-                }
-                __builtin_amdgcn_s_waitcnt(0x0F70);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const float4 b = *reinterpret_cast<const float4*>((PROJ ? BO : B2) + foff(nt));
-                    x[rt][nt][0] = DT::to_f((u16)(rx[nt].x & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(rx[nt].x >> 16)) + b.y;
-                    x[rt][nt][2] = DT::to_f((u16)(rx[nt].y & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(rx[nt].y >> 16)) + b.w;
-                    asm("" : "+a"(x[rt][nt]));        // the accumulator lives in accumulation registers from here on
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                for (int p = 0; p < NT / 2; ++p) rx[rt][p] = *reinterpret_cast<const uint4*>(xr + 32 * p + 8 * g);
             }
             if constexpr (!LEAD)
 #pragma unroll
@@ -1112,7 +1100,19 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                     hf[rt][c].h[0] = make_uint2(r4.x, r4.y); hf[rt][c].h[1] = make_uint2(r4.z, r4.w);
                 }
             }
-            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const float4 b = *reinterpret_cast<const float4*>((PROJ ? BO : B2) + foff(nt));
+                    const uint32_t lo = (nt & 1) ? rx[rt][nt >> 1].z : rx[rt][nt >> 1].x, hi = (nt & 1) ? rx[rt][nt >> 1].w : rx[rt][nt >> 1].y;
+                    x[rt][nt][0] = DT::to_f((u16)(lo & 0xffff)) + b.x; x[rt][nt][1] = DT::to_f((u16)(lo >> 16)) + b.y;
+                    x[rt][nt][2] = DT::to_f((u16)(hi & 0xffff)) + b.z; x[rt][nt][3] = DT::to_f((u16)(hi >> 16)) + b.w;
+                    asm("" : "+a"(x[rt][nt]));        // the accumulator lives in accumulation registers from here on
+                    if ((nt & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         } else {   // the tile's own loads: all issued, one wait the compiler can see (it does not know of the ring's transfers)
             uint2 rx[2][NT], rh[2][NT];
 #pragma unroll
