@@ -535,6 +535,8 @@ def proj_ffn_fused(att, x, image, F, ln2_w, ln2_b, eps2=1e-5, act="relu", ln_w=N
     xo = torch.empty_like(x)
     ho = torch.empty_like(x) if ln_w is not None and (want_ho or n_next == 0) else None
     qo = torch.empty(*x.shape[:-1], n_next, device=x.device, dtype=x.dtype) if n_next > 0 else None
+    if rows == 0:                      # nothing to launch (an empty tensor has no address to hand over)
+        return (xo, ho, qo) if n_next > 0 else (xo, ho)
     with torch.cuda.device(x.device):
         rc = _lib.load().bsrl_proj_ffn_packed(image.data_ptr(), att.data_ptr(), x.data_ptr(), _f32c(ln2_w, "ln2_w").data_ptr(),
                                               _f32c(ln2_b, "ln2_b").data_ptr(), float(eps2), _ptr(_f32c(ln_w, "ln_w")),
@@ -578,6 +580,8 @@ def ln_proj_fused(x, image, n_next, ln_w, ln_b, eps=1e-5, want_ho=False):
     rows = x.numel() // d
     ho = torch.empty_like(x) if want_ho else None
     qo = torch.empty(*x.shape[:-1], n_next, device=x.device, dtype=x.dtype)
+    if rows == 0:
+        return ho, qo
     with torch.cuda.device(x.device):
         rc = _lib.load().bsrl_ln_proj_packed(image.data_ptr(), x.data_ptr(), _f32c(ln_w, "ln_w").data_ptr(),
                                              _f32c(ln_b, "ln_b").data_ptr(), float(eps), _ptr(ho), qo.data_ptr(), n_next, rows, d,

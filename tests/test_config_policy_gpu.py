@@ -149,6 +149,38 @@ def test_ops_route_final_block_pruned_to_token0_matches_the_dense_form(dtype, to
     assert (lg2 - lg2_d).abs().max().item() <= tol * max(lg2_d.abs().max().item(), 1.0)
 
 
+def test_ops_route_block_tail_fusions_keep_the_forward_at_d384():
+    """d = 384 per-op route: (a) everything separate, (b) a block's output projection + LN2 + FFN + next LN1 in one kernel,
+    (c) also the next block's q|k|v (and block 0's LN1 + q|k|v) from that kernel - the default.  Same rounding points, other
+    accumulation orders: the three agree to the stream's rounding, and each holds config 3's ceilings against the oracle."""
+    c = cm.CONFIGS[3]
+    spec = c["spec"]
+    p, m = _build(spec, c["w_seed"], "f16", "ops")
+    obs, k = cm.make_inputs(spec, 40, c["obs_seed"], c["mask"])
+    od, kd = obs.to(DEV), k.to(DEV)
+    assert m.fuse_block_tail and m.fuse_next_proj
+    lg_c, v_c = m.forward_stacked(od, kd)
+    m.fuse_next_proj = False
+    lg_b, v_b = m.forward_stacked(od, kd)
+    m.fuse_block_tail = False
+    lg_a, v_a = m.forward_stacked(od, kd)
+    ref_lg, _ = cm.forward(p, spec, obs, k)
+    scale = ref_lg.abs().max().item()
+    for lg in (lg_a, lg_b, lg_c):
+        assert (lg.cpu() - ref_lg).abs().max().item() <= 1.6e-2            # config 3's literal ceiling (see the 16-bit route test)
+    e_a = (lg_a.cpu() - ref_lg).abs().pow(2).mean().sqrt().item()
+    for lg in (lg_b, lg_c):
+        assert (lg - lg_a).abs().max().item() <= 1.2e-2 and scale > 5.0
+        e = (lg.cpu() - ref_lg).abs().pow(2).mean().sqrt().item()
+        assert e <= 1.15 * e_a, (e, e_a)                                   # no worse an error class than the separate launches
+    assert (v_c - v_a).abs().max().item() <= 1.2e-2 and (v_b - v_a).abs().max().item() <= 1.2e-2
+    # unpruned, with the fusions: the last block then also goes through the one-kernel tail (no LayerNorm behind it)
+    m.fuse_block_tail = m.fuse_next_proj = True
+    m.prune_final = False
+    lg_d, _ = m.forward_stacked(od, kd)
+    assert (lg_d - lg_c).abs().max().item() <= 1.2e-2
+
+
 def test_masked_slots_cannot_change_outputs_on_gpu():
     c = cm.CONFIGS[1]
     spec = c["spec"]

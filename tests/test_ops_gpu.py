@@ -384,6 +384,36 @@ def test_layernorm_and_packed_projection_in_one_kernel(dtype, rows, n_next, want
         assert torch.equal(b, qo[lo:hi])
 
 
+def test_block_tail_kernel_rejects_what_it_cannot_take():
+    d, Fh, rows = 384, 1536, 64
+    dt = torch.float16
+    x = _rand(rows + 1, d, dtype=dt, seed=1)
+    att = _rand(rows + 1, d, dtype=dt, seed=2)
+    wo = _rand(d, d, dtype=dt, seed=3, scale=0.05)
+    w0 = _rand(Fh, d, dtype=dt, seed=4, scale=0.05)
+    w2 = _rand(d, Fh, dtype=dt, seed=5, scale=0.03)
+    bo, b0, b2 = _rand(d, seed=6), _rand(Fh, seed=7), _rand(d, seed=8)
+    lw, lb = _rand(d, seed=9) + 1, _rand(d, seed=10)
+    img = ops.proj_ffn_pack(wo, bo, w0, b0, w2, b2)
+    with pytest.raises(RuntimeError):                      # an image packed for another shape
+        ops.proj_ffn_fused(att[:rows], x[:rows], img, Fh, lw, lb, n_next=1152, ln_w=lw, ln_b=lb)
+    with pytest.raises(RuntimeError):                      # a projection behind needs the LayerNorm it projects
+        ops.proj_ffn_fused(att[:rows], x[:rows], img, Fh, lw, lb, n_next=1152)
+    with pytest.raises(RuntimeError):                      # att and x of different shapes
+        ops.proj_ffn_fused(att[:rows - 1], x[:rows], img, Fh, lw, lb)
+    with pytest.raises(ops.Unsupported):                   # d = 256 has no such kernel
+        ops.proj_ffn_pack(_rand(256, 256, dtype=dt, seed=1), _rand(256, seed=2), _rand(1024, 256, dtype=dt, seed=3),
+                          _rand(1024, seed=4), _rand(256, 1024, dtype=dt, seed=5), _rand(256, seed=6))
+    # zero rows: nothing launched, empty outputs
+    xo, ho = ops.proj_ffn_fused(att[:0], x[:0], img, Fh, lw, lb, ln_w=lw, ln_b=lb)
+    assert xo.shape == (0, d) and ho.shape == (0, d)
+    # misaligned rows (a view 8 bytes into the allocation) are an error of the entry point, not a fault
+    flat = torch.zeros(rows * d + 8, dtype=dt, device=DEV)
+    xm = flat[4:4 + rows * d].view(rows, d)
+    with pytest.raises(RuntimeError):
+        ops.proj_ffn_fused(att[:rows], xm, img, Fh, lw, lb)
+
+
 def test_ffn_fused_unsupported_shapes_say_so():
     assert not ops.ffn_fused_supported(160, 640, torch.float16)
     assert not ops.ffn_fused_supported(128, 500, torch.float16)
