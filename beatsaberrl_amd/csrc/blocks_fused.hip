@@ -1256,13 +1256,6 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
         else up(0);
         for (int ch = 0; ch < nch; ++ch) {
             BFrag8 hid[2];
-            // ACT_IN_UP (the register-pipelined kernel, hidden not saved): the chunk's pre-activations are copied out of
-            // the accumulators and the activation of those 16 values per lane is issued one value per fragment step
-            // BETWEEN the MFMAs of the next up-projection stage (which refills the accumulators), instead of in a block
-            // of its own with the matrix pipe idle - with one wave per SIMD nothing else would fill that time
-            constexpr bool ACT_IN_UP = PIPE && !SAVE;
-            const bool act_now = !ACT_IN_UP || ch + 1 >= nch;
-            if (act_now) {
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
@@ -1270,7 +1263,6 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
                     hid[rt].w[ntl * 2] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][0]), apply_act16<ACT>(acc[ntl][rt][1]));
                     hid[rt].w[ntl * 2 + 1] = bpack2<DT>(apply_act16<ACT>(acc[ntl][rt][2]), apply_act16<ACT>(acc[ntl][rt][3]));
                 }
-            }
             if (SAVE) {
                 // the rounded hidden exactly as the down-projection consumes it: a lane holds 4 consecutive units of its
                 // row per tile of the chunk (these stores sit in the vmcnt queue like any other: they can only make the
@@ -1288,34 +1280,7 @@ __global__ __launch_bounds__(NW_ * 64, (ffn_wgs_per_cu<D, NW_>())) void ffn_rows
             // stage parities: W1(0) even, then {W1(ch + 1) odd, W2(ch) even} ..., W2(last) odd
             if constexpr (PIPE) {
                 // the stage in the ring and its first NBUF - 1 fragments were requested by the stage before
-                if (ch + 1 < nch) {                                                      // W1(ch + 1), then W2(ch): even
-                    if constexpr (ACT_IN_UP) {
-                        f32x4 pre[2][2];
-                        float hv[2][2][4];
-#pragma unroll
-                        for (int ntl = 0; ntl < 2; ++ntl)
-#pragma unroll
-                            for (int rt = 0; rt < 2; ++rt) pre[ntl][rt] = acc[ntl][rt];
-                        up_init(ch + 1);
-                        stage(2, [&](auto i_, const s16x8& wf) __attribute__((always_inline)) {
-                            up_mm(i_, wf);
-                            constexpr int i = decltype(i_)::value;
-                            if constexpr (i >= 2 && i < 18) {
-                                constexpr int v = i - 2, ntl = v / 8, rt = (v / 4) % 2, j = v % 4;
-                                hv[ntl][rt][j] = apply_act16<ACT>(pre[ntl][rt][j]);
-                            }
-                            if constexpr (i == 18) {
-#pragma unroll
-                                for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-                                    for (int ntl = 0; ntl < 2; ++ntl) {
-                                        hid[rt].w[ntl * 2] = bpack2<DT>(hv[ntl][rt][0], hv[ntl][rt][1]);
-                                        hid[rt].w[ntl * 2 + 1] = bpack2<DT>(hv[ntl][rt][2], hv[ntl][rt][3]);
-                                    }
-                            }
-                        });
-                    } else { up_init(ch + 1); stage(2, up_mm); }
-                }
+                if (ch + 1 < nch) { up_init(ch + 1); stage(2, up_mm); }                  // W1(ch + 1), then W2(ch): even
                 // W2(ch); an odd stage follows but the last, which ends the tile or (PROJ with a projection behind) is followed by an even one
                 stage(ch + 1 < nch ? 1 : (PROJ && a.nq > 0) ? 2 : 0, [&](auto i_, const s16x8& w2) __attribute__((always_inline)) {
                     constexpr int i = decltype(i_)::value;       // feature tile i
