@@ -1525,7 +1525,9 @@ __global__ __launch_bounds__(256) void next_pack_frags_kernel(ProjPackArgs a) {
     if (f == 0 && a.wo == nullptr) for (int k = lane; k < 2 * D; k += 64) a.vec_bo[k - D] = 0.f;
 }
 bool proj_ffn_shape_ok(int64_t d, int64_t F, int64_t n_next, int dtype) {
-    return d == 384 && ffn_packed_shape_ok(d, F, dtype) && n_next >= 0 && n_next % 64 == 0 && n_next <= 3 * d;
+    if (!(d == 384 && ffn_packed_shape_ok(d, F, dtype) && n_next >= 0 && n_next % 64 == 0 && n_next <= 3 * d)) return false;
+    // the vectors (b0, b2, three LayerNorm pairs' worth, bo, bn) must fit LDS beside the five-slot ring
+    return (size_t)(F + 6 * d + n_next) * 4 + 1024 + 5 * FfnRing<384, 4, 0>::STAGE_BYTES + 1024 <= (size_t)LDS_BUDGET;
 }
 int64_t proj_frag_bytes(int64_t d) { return (d / 32) * (d / 16) * 1024; }
 

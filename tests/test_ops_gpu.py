@@ -401,6 +401,8 @@ def test_block_tail_kernel_rejects_what_it_cannot_take():
         ops.proj_ffn_fused(att[:rows], x[:rows], img, Fh, lw, lb, n_next=1152)
     with pytest.raises(RuntimeError):                      # att and x of different shapes
         ops.proj_ffn_fused(att[:rows - 1], x[:rows], img, Fh, lw, lb)
+    # a hidden width whose vectors do not fit LDS beside the ring is "unsupported", not a launch failure
+    assert ops.proj_ffn_supported(d, 4096, dt, 1152) and not ops.proj_ffn_supported(d, 8192, dt, 1152)
     with pytest.raises(ops.Unsupported):                   # d = 256 has no such kernel
         ops.proj_ffn_pack(_rand(256, 256, dtype=dt, seed=1), _rand(256, seed=2), _rand(1024, 256, dtype=dt, seed=3),
                           _rand(1024, seed=4), _rand(256, 1024, dtype=dt, seed=5), _rand(256, seed=6))
